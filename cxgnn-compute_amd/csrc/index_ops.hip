@@ -1,0 +1,168 @@
+// Integer / index work on CSR graphs: transposition (the graph the backward
+// pass gathers over), row-id expansion, 1/degree edge values and relation
+// padding.  All results are bit-exact functions of their inputs.
+#include "cxg_common.hpp"
+
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+
+namespace cxg {
+namespace {
+
+constexpr int kBlock = 256;
+
+// rows[k] = row containing edge position pos(k): the r with ptr[r] <= p < ptr[r+1].
+__device__ __forceinline__ int64_t row_of_position(const int64_t* __restrict__ ptr, int64_t n_rows,
+                                                   int64_t p) {
+  // upper_bound(ptr[0..n_rows], p) - 1
+  int64_t lo = 0, hi = n_rows + 1;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (ptr[mid] <= p) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo - 1;
+}
+
+__global__ void transpose_fill_kernel(const int64_t* __restrict__ ptr, int64_t n_rows,
+                                      const int64_t* __restrict__ sorted_src,
+                                      const int64_t* __restrict__ perm, int64_t n_edges,
+                                      int64_t n_cols, int64_t* __restrict__ ptr_t,
+                                      int64_t* __restrict__ idx_t) {
+  const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (k < n_edges) idx_t[k] = row_of_position(ptr, n_rows, perm[k]);
+  if (k <= n_cols) {
+    // ptr_t[c] = number of edges whose source is < c
+    int64_t lo = 0, hi = n_edges;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (sorted_src[mid] < k) lo = mid + 1;
+      else hi = mid;
+    }
+    ptr_t[k] = lo;
+  }
+}
+
+__global__ void row_ids_kernel(const int64_t* __restrict__ ptr, int64_t n_rows, int64_t n_edges,
+                               int64_t* __restrict__ rows) {
+  const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (k < n_edges) rows[k] = row_of_position(ptr, n_rows, k + ptr[0]);
+}
+
+// One wave per row: val[e] = 1 / deg(row) for the row's edges.
+__global__ void edge_value_degree_kernel(const int64_t* __restrict__ ptr, int64_t n_rows,
+                                         float* __restrict__ out) {
+  const int lane = lane_id();
+  const int64_t r = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (r >= n_rows) return;
+  const int64_t b = ptr[r], e = ptr[r + 1];
+  if (e <= b) return;
+  const float v = 1.0f / (float)(e - b);
+  for (int64_t i = b + lane; i < e; i += CXG_WAVE) out[i] = v;
+}
+
+__global__ void pad_rel_kernel(int64_t* __restrict__ rel, int64_t* __restrict__ idx,
+                               const int64_t* __restrict__ count, int thres, int num_rel,
+                               int64_t base) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t slots = (int64_t)num_rel * (thres - 1);
+  if (t >= slots) return;
+  const int which = (int)(t / (thres - 1));
+  const int64_t mod = count[which] % thres;
+  const bool fill = (mod != 0) && ((t % (thres - 1)) < (thres - mod));
+  rel[base + t] = fill ? which : num_rel;
+  if (idx) idx[base + t] = -1;
+}
+
+int bits_for(int64_t n) {
+  int b = 1;
+  while (b < 63 && ((int64_t)1 << b) < n) ++b;
+  return b;
+}
+
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+}  // namespace
+}  // namespace cxg
+
+extern "C" {
+
+size_t cxg_csr_transpose_workspace_bytes(int64_t n_edges, int64_t n_cols) {
+  if (n_edges < 0 || n_cols < 0) return 0;
+  size_t temp = 0;
+  rocprim::counting_iterator<int64_t> iota(0);
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (const int64_t*)nullptr, (int64_t*)nullptr,
+                                           iota, (int64_t*)nullptr, (size_t)n_edges, 0,
+                                           cxg::bits_for(n_cols > 1 ? n_cols : 2), (hipStream_t)0);
+  if (e != hipSuccess) return 0;
+  return cxg::align256((size_t)n_edges * sizeof(int64_t)) + cxg::align256(temp) + 256;
+}
+
+int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows, int64_t n_cols,
+                          int64_t n_edges, int64_t* ptr_t, int64_t* idx_t, int64_t* perm,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+  CXG_REQUIRE(n_rows >= 0 && n_cols >= 0 && n_edges >= 0, CXG_ERR_ARG, "negative size");
+  CXG_REQUIRE(ptr && ptr_t, CXG_ERR_ARG, "null ptr");
+  CXG_REQUIRE(n_edges == 0 || (idx && idx_t && perm), CXG_ERR_ARG, "null idx/idx_t/perm");
+  const size_t need = cxg_csr_transpose_workspace_bytes(n_edges, n_cols);
+  CXG_REQUIRE(workspace && workspace_bytes >= need, CXG_ERR_WORKSPACE,
+              "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  CXG_REQUIRE(((uintptr_t)workspace & 255) == 0, CXG_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  int64_t* sorted_src = reinterpret_cast<int64_t*>(workspace);
+  const size_t off = cxg::align256((size_t)n_edges * sizeof(int64_t));
+  void* temp = reinterpret_cast<char*>(workspace) + off;
+  size_t temp_bytes = workspace_bytes - off;
+  if (n_edges > 0) {
+    rocprim::counting_iterator<int64_t> iota(0);
+    CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, idx, sorted_src, iota, perm,
+                                            (size_t)n_edges, 0, cxg::bits_for(n_cols > 1 ? n_cols : 2),
+                                            st));
+  }
+  const int64_t work = (n_edges > n_cols + 1) ? n_edges : n_cols + 1;
+  hipLaunchKernelGGL(cxg::transpose_fill_kernel, dim3((unsigned)cxg::ceil_div(work, cxg::kBlock)),
+                     dim3(cxg::kBlock), 0, st, ptr, n_rows, sorted_src, perm, n_edges, n_cols, ptr_t,
+                     idx_t);
+  CXG_LAUNCH_CHECK("transpose_fill_kernel");
+  return CXG_OK;
+}
+
+int cxg_csr_row_ids_i64(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int64_t* rows,
+                        void* stream) {
+  CXG_REQUIRE(n_rows >= 0 && n_edges >= 0, CXG_ERR_ARG, "negative size");
+  if (n_edges == 0) return CXG_OK;
+  CXG_REQUIRE(ptr && rows, CXG_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(cxg::row_ids_kernel, dim3((unsigned)cxg::ceil_div(n_edges, cxg::kBlock)),
+                     dim3(cxg::kBlock), 0, reinterpret_cast<hipStream_t>(stream), ptr, n_rows, n_edges,
+                     rows);
+  CXG_LAUNCH_CHECK("row_ids_kernel");
+  return CXG_OK;
+}
+
+int cxg_edge_value_degree_f32(const int64_t* ptr, int64_t n_rows, float* out, void* stream) {
+  CXG_REQUIRE(n_rows >= 0, CXG_ERR_ARG, "negative size");
+  if (n_rows == 0) return CXG_OK;
+  CXG_REQUIRE(ptr && out, CXG_ERR_ARG, "null pointer");
+  const int64_t threads = n_rows * CXG_WAVE;
+  hipLaunchKernelGGL(cxg::edge_value_degree_kernel,
+                     dim3((unsigned)cxg::ceil_div(threads, cxg::kBlock)), dim3(cxg::kBlock), 0,
+                     reinterpret_cast<hipStream_t>(stream), ptr, n_rows, out);
+  CXG_LAUNCH_CHECK("edge_value_degree_kernel");
+  return CXG_OK;
+}
+
+int cxg_pad_rel_i64(int64_t* rel, int64_t* idx, const int64_t* count, int thres, int num_rel,
+                    int64_t base, void* stream) {
+  CXG_REQUIRE(thres >= 1 && num_rel >= 0 && base >= 0, CXG_ERR_ARG, "bad thres/num_rel/base");
+  const int64_t slots = (int64_t)num_rel * (thres - 1);
+  if (slots == 0) return CXG_OK;
+  CXG_REQUIRE(rel && count, CXG_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(cxg::pad_rel_kernel, dim3((unsigned)cxg::ceil_div(slots, cxg::kBlock)),
+                     dim3(cxg::kBlock), 0, reinterpret_cast<hipStream_t>(stream), rel, idx, count, thres,
+                     num_rel, base);
+  CXG_LAUNCH_CHECK("pad_rel_kernel");
+  return CXG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,383 @@
+// CSR-by-destination SpMM for gfx950: sum / mean / edge-weighted (single and
+// multi-head), forward and -- on a transposed CSR -- backward.
+//
+// Work decomposition ("edge spans").  The edge array [ptr[0], ptr[n_rows]) is
+// cut into spans of T consecutive edges and every wavefront owns one span, so
+// the load per wave is the same for a degree-4 row and for a 17k-degree hub.
+// A wave locates the first row of its span with a 64-ary search over ptr, then
+// streams the span: 64 source ids are fetched with one coalesced load, each id
+// is broadcast to a scalar register and the whole wave gathers that source row
+// (64 lanes x V floats), U gathers in flight at a time.  Row boundaries are
+// wave-uniform, so a finished row is stored directly by the wave.  Rows that
+// cross a span boundary leave partial sums in a carry buffer; a second small
+// kernel adds the partials of each such row in span order.  No atomics: the
+// result is deterministic run to run.
+//
+// Semantics follow the reference kernels gen_fwd_sum / gen_fwd_mean /
+// gen_fwd_sum_edge_value[_multi_head] (src/cpp/src/aggr_kernel.cu:3-186) and
+// run_spmm_sharedmem* (src/cpp/src/spmm_kernel.cu:231-512).
+#include "cxg_common.hpp"
+
+namespace cxg {
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
+
+template <int V> struct Vec;
+template <> struct Vec<1> { using type = float; };
+template <> struct Vec<2> { using type = float2; };
+template <> struct Vec<4> { using type = float4; };
+
+template <int V> __device__ __forceinline__ typename Vec<V>::type vzero();
+template <> __device__ __forceinline__ float vzero<1>() { return 0.f; }
+template <> __device__ __forceinline__ float2 vzero<2>() { return make_float2(0.f, 0.f); }
+template <> __device__ __forceinline__ float4 vzero<4>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+
+__device__ __forceinline__ void vfma(float& a, float v, float w) { a += v * w; }
+__device__ __forceinline__ void vfma(float2& a, float2 v, float w) { a.x += v.x * w; a.y += v.y * w; }
+__device__ __forceinline__ void vfma(float4& a, float4 v, float w) {
+  a.x += v.x * w; a.y += v.y * w; a.z += v.z * w; a.w += v.w * w;
+}
+__device__ __forceinline__ void vadd(float& a, float v) { a += v; }
+__device__ __forceinline__ void vadd(float2& a, float2 v) { a.x += v.x; a.y += v.y; }
+__device__ __forceinline__ void vadd(float4& a, float4 v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; }
+__device__ __forceinline__ void vscale(float& a, float s) { a *= s; }
+__device__ __forceinline__ void vscale(float2& a, float s) { a.x *= s; a.y *= s; }
+__device__ __forceinline__ void vscale(float4& a, float s) { a.x *= s; a.y *= s; a.z *= s; a.w *= s; }
+
+template <typename IdxT>
+struct SpmmArgs {
+  const IdxT* ptr;
+  const IdxT* idx;
+  const float* x;
+  float* out;
+  const float* val;        // [*, heads] or null
+  const int64_t* perm;     // val row of edge position, or null
+  int64_t ldx, ldo;
+  int64_t n_rows;
+  int F;                   // floats per row (heads * channels)
+  int heads, channels;
+  int T;                   // edges per span (multiple of 64)
+  int mean, accumulate;
+  float* carry;            // [n_spans_cap][2][F]: head partial, tail partial
+  int64_t* tail_row;       // [n_spans_cap]: row whose tail partial the span holds, or -1
+};
+
+// WMODE: 0 = unweighted, 1 = one weight per edge (heads == 1), 2 = one weight
+// per edge and head (each lane's V columns lie in one head).
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, int U>
+__global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
+  using vec_t = typename Vec<V>::type;
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t n_rows = a.n_rows;
+  const int64_t e_begin = (int64_t)a.ptr[0];
+  const int64_t e_end = (int64_t)a.ptr[n_rows];
+  const int64_t total = e_end - e_begin;
+  const int T = a.T;
+  const int64_t n_spans = total > 0 ? (total + T - 1) / T : 1;
+  if (s >= n_spans) return;
+  const bool last = (s == n_spans - 1);
+  const int64_t e0 = e_begin + s * T;
+  const int n = (int)((e_end - e0) < (int64_t)T ? (e_end - e0) : (int64_t)T);
+
+  // column tile of this block (grid.y tiles rows wider than 64*V floats)
+  const int col = blockIdx.y * (CXG_WAVE * V) + lane * V;
+  const bool col_ok = GUARD ? (col < a.F) : true;
+  const int F = a.F;
+
+  const int64_t r_lo = wave_lower_bound(a.ptr, n_rows, e0);
+  bool is_head = (r_lo == n_rows) || ((int64_t)a.ptr[r_lo] > e0);
+  int64_t r = is_head ? r_lo - 1 : r_lo;
+
+  // Row ends of rows [rbase, rbase + 64) relative to e0, clamped to n + 1.
+  int64_t rbase = r;
+  auto load_row_ends = [&](int64_t rb) -> int {
+    int64_t q = rb + 1 + lane;
+    if (q > n_rows) q = n_rows;
+    const int64_t d = (int64_t)a.ptr[q] - e0;
+    return (int)(d < (int64_t)n + 1 ? d : (int64_t)n + 1);
+  };
+  int row_ends = load_row_ends(rbase);
+  int cur_start = is_head ? -1 : 0;
+  int cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
+
+  vec_t acc = vzero<V>();
+  float* const carry_head = a.carry + (size_t)(2 * s) * F;
+  float* const carry_tail = carry_head + F;
+
+  int head_of_lane = 0;
+  if (WMODE == 2) head_of_lane = col / a.channels;
+
+  auto next_row = [&]() {
+    ++r;
+    if (r - rbase == CXG_WAVE) {
+      rbase = r;
+      row_ends = load_row_ends(rbase);
+    }
+    cur_start = cur_end;
+    cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
+    is_head = false;
+  };
+  auto store_vec = [&](float* dst, vec_t v) {
+    if (col_ok) *reinterpret_cast<vec_t*>(dst + col) = v;
+  };
+  // Row r is complete inside this span: write it (or its head partial).
+  auto finish_row = [&]() {
+    if (is_head) {
+      store_vec(carry_head, acc);
+    } else {
+      float* dst = a.out + r * a.ldo;
+      if (a.mean) {
+        const int deg = cur_end - cur_start;
+        if (deg > 0) vscale(acc, 1.0f / (float)deg);
+      }
+      if (a.accumulate) {
+        if (col_ok) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
+      }
+      store_vec(dst, acc);
+    }
+    acc = vzero<V>();
+  };
+
+  for (int c0 = 0; c0 < n; c0 += CXG_WAVE) {
+    const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
+    int64_t my_src = 0;
+    int64_t my_vrow = 0;
+    float my_w = 0.f;
+    if (lane < cn) {
+      const int64_t pos = e0 + c0 + lane;
+      my_src = (int64_t)a.idx[pos];
+      if (PERM) my_vrow = a.perm[pos];
+      if (WMODE == 1 && !PERM) my_w = a.val[pos];
+    }
+    for (int b = 0; b < cn; b += U) {
+      vec_t v[U];
+      float w[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int jj = b + u;
+        if (jj < cn) {
+          const int64_t src = bcast_i64(my_src, jj);
+          const float* row = a.x + src * a.ldx;
+          v[u] = col_ok ? *reinterpret_cast<const vec_t*>(row + col) : vzero<V>();
+          if (WMODE == 1) {
+            if (PERM) w[u] = a.val[bcast_i64(my_vrow, jj)];
+            else w[u] = bcast_f32(my_w, jj);
+          } else if (WMODE == 2) {
+            const int64_t vrow = PERM ? bcast_i64(my_vrow, jj) : (e0 + c0 + jj);
+            w[u] = col_ok ? a.val[vrow * a.heads + head_of_lane] : 0.f;
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int jj = b + u;
+        if (jj < cn) {
+          const int j = c0 + jj;
+          while (j >= cur_end) {
+            finish_row();
+            next_row();
+          }
+          if (WMODE == 0) vadd(acc, v[u]);
+          else vfma(acc, v[u], w[u]);
+        }
+      }
+    }
+  }
+
+  // Rows that end at or before the span end, then the row (if any) that runs on.
+  int64_t tail = -1;
+  while (r < n_rows) {
+    if (cur_end > n) {
+      if (is_head) {
+        store_vec(carry_head, acc);
+      } else if (cur_start < n) {
+        store_vec(carry_tail, acc);
+        tail = r;
+      }
+      break;
+    }
+    if (!(is_head || cur_start < n || last)) break;
+    finish_row();
+    next_row();
+  }
+  if (lane == 0 && blockIdx.y == 0) a.tail_row[s] = tail;
+}
+
+// One wave per span: if the span holds the tail partial of row t, add the head
+// partials of the following spans that row t runs through, in span order.
+template <typename IdxT, int V, bool GUARD>
+__global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
+  using vec_t = typename Vec<V>::type;
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t e_begin = (int64_t)a.ptr[0];
+  const int64_t e_end = (int64_t)a.ptr[a.n_rows];
+  const int64_t total = e_end - e_begin;
+  const int T = a.T;
+  const int64_t n_spans = total > 0 ? (total + T - 1) / T : 1;
+  if (s >= n_spans) return;
+  const int64_t t = uniform_i64(a.tail_row[s]);
+  if (t < 0) return;
+  const int col = blockIdx.y * (CXG_WAVE * V) + lane * V;
+  const bool col_ok = GUARD ? (col < a.F) : true;
+  if (!col_ok) return;
+  const int F = a.F;
+  const int64_t row_begin = (int64_t)a.ptr[t];
+  const int64_t row_end = (int64_t)a.ptr[t + 1];
+  const int64_t s_last = (row_end - 1 - e_begin) / T;
+  vec_t acc = *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * s + 1) * F + col);
+  for (int64_t q = s + 1; q <= s_last; ++q)
+    vadd(acc, *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * q) * F + col));
+  if (a.mean) vscale(acc, 1.0f / (float)(row_end - row_begin));
+  float* dst = a.out + t * a.ldo;
+  if (a.accumulate) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
+  *reinterpret_cast<vec_t*>(dst + col) = acc;
+}
+
+// Span length: 512 edges for large graphs, shorter for small ones so that the
+// launch still has a few thousand waves.
+int choose_span(int64_t n_edges_cap) {
+  int64_t t = n_edges_cap / 16384;
+  t = (t + 63) / 64 * 64;
+  if (t < 64) t = 64;
+  if (t > 512) t = 512;
+  return (int)t;
+}
+
+struct Plan {
+  int T;
+  int64_t n_spans_cap;
+  size_t tail_bytes;   // aligned
+  size_t carry_bytes;
+};
+
+Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
+  Plan p;
+  p.T = choose_span(n_edges_cap);
+  p.n_spans_cap = n_edges_cap > 0 ? ceil_div(n_edges_cap, p.T) : 1;
+  p.tail_bytes = (size_t)((p.n_spans_cap * sizeof(int64_t) + 255) / 256 * 256);
+  p.carry_bytes = (size_t)p.n_spans_cap * 2 * (size_t)row_floats * sizeof(float);
+  return p;
+}
+
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM>
+int launch_spmm(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
+  constexpr int U = (V == 4) ? 8 : 16;
+  const int tile = CXG_WAVE * V;
+  dim3 grid((unsigned)ceil_div(n_spans_cap, kWavesPerBlock), (unsigned)ceil_div(a.F, tile), 1);
+  dim3 block(kBlock, 1, 1);
+  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, U>), grid, block, 0, stream, a);
+  CXG_LAUNCH_CHECK("spmm_span_kernel");
+  hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, V, GUARD>), grid, block, 0, stream, a);
+  CXG_LAUNCH_CHECK("spmm_fixup_kernel");
+  return CXG_OK;
+}
+
+template <typename IdxT, int WMODE, bool PERM>
+int dispatch_shape(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
+  // widest vector that divides the row (and the head, for per-head weights) and
+  // keeps every access aligned; among those the one needing the fewest column
+  // tiles, ties to the narrower vector (more lanes busy).
+  const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry |
+                               (uintptr_t)(a.ldx * 4) | (uintptr_t)(a.ldo * 4) | (uintptr_t)(a.F * 4);
+  int unit = (WMODE == 2) ? a.channels : a.F;
+  int best_v = 1;
+  int64_t best_tiles = ceil_div(a.F, CXG_WAVE);
+  for (int v = 2; v <= 4; v *= 2) {
+    if (unit % v != 0 || (align_bits & (uintptr_t)(4 * v - 1)) != 0) break;
+    const int64_t tiles = ceil_div(a.F, CXG_WAVE * v);
+    if (tiles < best_tiles) { best_tiles = tiles; best_v = v; }
+  }
+  const bool guard = (best_tiles * CXG_WAVE * best_v != a.F);
+#define CXG_CASE(VV)                                                                  \
+  if (best_v == VV) {                                                                  \
+    return guard ? launch_spmm<IdxT, VV, true, WMODE, PERM>(a, n_spans_cap, stream)   \
+                 : launch_spmm<IdxT, VV, false, WMODE, PERM>(a, n_spans_cap, stream); \
+  }
+  CXG_CASE(1) CXG_CASE(2) CXG_CASE(4)
+#undef CXG_CASE
+  return set_error(CXG_ERR_UNSUPPORTED, "no kernel for vector width %d", best_v);
+}
+
+template <typename IdxT>
+int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_t* perm,
+                const float* x, int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
+                int64_t n_edges_cap, int heads, int channels, unsigned flags, void* workspace,
+                size_t workspace_bytes, void* stream) {
+  CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
+  CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
+  CXG_REQUIRE((int64_t)heads * channels <= (1 << 20), CXG_ERR_UNSUPPORTED, "row too wide");
+  CXG_REQUIRE((flags & ~(CXG_SPMM_MEAN | CXG_SPMM_ACCUMULATE)) == 0, CXG_ERR_ARG, "unknown flag");
+  if (n_rows == 0) return CXG_OK;
+  CXG_REQUIRE(ptr && out, CXG_ERR_ARG, "null ptr/out");
+  CXG_REQUIRE(n_edges_cap == 0 || (idx && x), CXG_ERR_ARG, "null idx/x");
+  const int F = heads * channels;
+  CXG_REQUIRE(ldx >= F && ldo >= F, CXG_ERR_ARG, "row stride smaller than row");
+  CXG_REQUIRE(!perm || val, CXG_ERR_ARG, "val_perm without val");
+  const Plan plan = make_plan(n_edges_cap, F);
+  CXG_REQUIRE(workspace && workspace_bytes >= plan.tail_bytes + plan.carry_bytes, CXG_ERR_WORKSPACE,
+              "workspace of %zu bytes needed, %zu given", plan.tail_bytes + plan.carry_bytes,
+              workspace_bytes);
+  CXG_REQUIRE(((uintptr_t)workspace & 255) == 0, CXG_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+
+  SpmmArgs<IdxT> a;
+  a.ptr = ptr; a.idx = idx; a.x = x; a.out = out; a.val = val; a.perm = perm;
+  a.ldx = ldx; a.ldo = ldo; a.n_rows = n_rows; a.F = F; a.heads = heads; a.channels = channels;
+  a.T = plan.T;
+  a.mean = (flags & CXG_SPMM_MEAN) ? 1 : 0;
+  a.accumulate = (flags & CXG_SPMM_ACCUMULATE) ? 1 : 0;
+  a.tail_row = reinterpret_cast<int64_t*>(workspace);
+  a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (!val) return dispatch_shape<IdxT, 0, false>(a, plan.n_spans_cap, st);
+  if constexpr (sizeof(IdxT) == 8) {
+    if (heads == 1) {
+      return perm ? dispatch_shape<IdxT, 1, true>(a, plan.n_spans_cap, st)
+                  : dispatch_shape<IdxT, 1, false>(a, plan.n_spans_cap, st);
+    }
+    return perm ? dispatch_shape<IdxT, 2, true>(a, plan.n_spans_cap, st)
+                : dispatch_shape<IdxT, 2, false>(a, plan.n_spans_cap, st);
+  }
+  return set_error(CXG_ERR_UNSUPPORTED, "weighted SpMM needs int64 indices");
+}
+
+}  // namespace
+}  // namespace cxg
+
+extern "C" {
+
+size_t cxg_spmm_workspace_bytes(int64_t n_edges_cap, int64_t row_floats) {
+  if (n_edges_cap < 0 || row_floats < 1) return 0;
+  const cxg::Plan p = cxg::make_plan(n_edges_cap, row_floats);
+  return p.tail_bytes + p.carry_bytes;
+}
+
+int cxg_spmm_sum_f32(const int64_t* ptr, const int64_t* idx, const float* x, int64_t ldx,
+                     float* out, int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int feat,
+                     unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
+  return cxg::spmm_common<int64_t>(ptr, idx, nullptr, nullptr, x, ldx, out, ldo, n_rows,
+                                   n_edges_cap, 1, feat, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_sum_f32_i32(const int32_t* ptr, const int32_t* idx, const float* x, int64_t ldx,
+                         float* out, int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int feat,
+                         unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
+  return cxg::spmm_common<int32_t>(ptr, idx, nullptr, nullptr, x, ldx, out, ldo, n_rows,
+                                   n_edges_cap, 1, feat, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                          const int64_t* val_perm, const float* x, int64_t ldx, float* out,
+                          int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int heads, int channels,
+                          unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
+  return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
+                                   heads, channels, flags, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+"""Drop-in for the reference's pybind module ``cxgnncomp_backend``
+(src/cpp/python_bindings/binding.cpp:14-130), backed by libcxgnn_hip.so.
+
+Same function names, argument order and meaning.  Differences, all deliberate:
+  * errors raise ValueError / RuntimeError instead of exit(1)
+    (src/cpp/include/common.h:16-26);
+  * the nine launch integers of the ``*_configurable`` functions are accepted
+    and ignored -- the HIP kernels balance work by edge spans themselves;
+  * gradients w.r.t. node features are computed by gathering over a cached
+    transposed CSR instead of fp32 atomics, so they are deterministic;
+  * the autograd contexts keep the ptr/idx tensors alive instead of raw
+    pointers (src/cpp/src/aggr.cu:116-117).
+"""
+import enum
+
+import torch
+
+from . import _lib, _ops
+from ._ops import as_int, clear_graph_cache, set_graph_cache_capacity  # noqa: F401
+
+
+def _lib_version():
+    return _lib.load().cxg_version()
+
+
+# --------------------------------------------------------------------------- #
+# sum / mean aggregation  (binding.cpp:15-19, 37-41)
+# --------------------------------------------------------------------------- #
+def run_spmm_configurable(ptr, idx, vin, num_node, *launch_ints):
+    """out[r] = sum_e vin[idx[e]], r < num_node (src/cpp/src/spmm_host.cu:6-55)."""
+    if vin.dim() != 2:
+        raise ValueError("vin must be 2D")
+    return _ops.spmm(ptr, idx, vin, as_int(num_node))
+
+
+def run_spmm_configurable_int32(ptr, idx, vin, num_node, *launch_ints):
+    """int32 ptr/idx variant (src/cpp/src/spmm_host.cu:99-156)."""
+    if vin.dim() != 2:
+        raise ValueError("vin must be 2D")
+    return _ops.spmm(ptr, idx, vin, as_int(num_node))
+
+
+def run_spmm_configurable_bwd(ptr, idx, vin, grad_vout, num_node, *launch_ints):
+    """grad_vin[s] = sum_{e: idx[e]==s} grad_vout[row(e)], shaped like vin
+    (src/cpp/src/spmm_host.cu:57-97)."""
+    if grad_vout.dim() != 2:
+        raise ValueError("grad_vout must be 2D")
+    n = as_int(num_node)
+    g = _ops.transposed(ptr, idx, n, vin.shape[0])
+    return _ops.spmm(g.ptr_t, g.idx_t, grad_vout.contiguous(), vin.shape[0])
+
+
+class _SageFunction(torch.autograd.Function):
+    """SAGEFunction / SAGEEdgeValueFunction (src/cpp/src/aggr.cu:107-303)."""
+
+    @staticmethod
+    def forward(ctx, x, ptr, idx, edge_value, num_node, mean):
+        n = as_int(num_node)
+        if n == 0:
+            n = ptr.shape[0] - 1
+        ctx.n, ctx.mean, ctx.n_src = n, mean, x.shape[0]
+        ctx.x_shape = x.shape
+        x = x.contiguous()
+        if edge_value is None:
+            ctx.save_for_backward(ptr, idx)
+            return _ops.spmm(ptr, idx, x, n, mean=mean)
+        if mean:
+            # aggr.cu:158,163 aborts here with the same message
+            raise ValueError("DO NOT use mean with edge value")
+        edge_value = edge_value.contiguous()
+        x3 = x
+        if edge_value.dim() == 2 and x.dim() != 3:
+            raise ValueError("multi-head edge_value needs input [N, H, C]")
+        ctx.save_for_backward(ptr, idx, x, edge_value)
+        return _ops.spmm(ptr, idx, x3, n, val=edge_value)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        grad_out = grad_out.contiguous()
+        saved = ctx.saved_tensors
+        ptr, idx = saved[0], saved[1]
+        g = _ops.transposed(ptr, idx, ctx.n, ctx.n_src)
+        if len(saved) == 2:
+            if ctx.mean:
+                inv = _ops.inv_degree_transposed(g, ptr, ctx.n)
+                go = grad_out.reshape(ctx.n, -1)
+                gx = _ops.spmm(g.ptr_t, g.idx_t, go, ctx.n_src, val=inv)
+            else:
+                gx = _ops.spmm(g.ptr_t, g.idx_t, grad_out.reshape(ctx.n, -1), ctx.n_src)
+            return gx.reshape(ctx.x_shape), None, None, None, None, None
+        x, edge_value = saved[2], saved[3]
+        gx = _ops.spmm(g.ptr_t, g.idx_t, grad_out, ctx.n_src, val=edge_value, val_perm=g.perm)
+        gval = None
+        if ctx.needs_input_grad[3]:
+            gval = _ops.sddmm_csr(ptr, idx, x, grad_out, ctx.n, edge_value.shape)
+        return gx.reshape(ctx.x_shape), None, None, gval, None, None
+
+
+def sage_sum_forward(input, ptr, idx, num_node):
+    return _SageFunction.apply(input, ptr, idx, None, num_node, False)
+
+
+def sage_mean_forward(input, ptr, idx, num_node):
+    return _SageFunction.apply(input, ptr, idx, None, num_node, True)
+
+
+def sage_sum_forward_edge_value(input, ptr, idx, edge_value, num_node):
+    return _SageFunction.apply(input, ptr, idx, edge_value, num_node, False)
+
+
+def sage_mean_forward_edge_value(input, ptr, idx, edge_value, num_node):
+    return _SageFunction.apply(input, ptr, idx, edge_value, num_node, True)
+
+
+# --------------------------------------------------------------------------- #
+# multi-head weighted SpMM  (binding.cpp:57-74)
+# --------------------------------------------------------------------------- #
+class SPMM_MULTIHEAD_SCHEDULE(enum.IntEnum):
+    Naive = 0
+    PreReduce = 1
+    Optimal = 2
+
+
+Naive = SPMM_MULTIHEAD_SCHEDULE.Naive
+PreReduce = SPMM_MULTIHEAD_SCHEDULE.PreReduce
+Optimal = SPMM_MULTIHEAD_SCHEDULE.Optimal
+
+
+def edge_value_degree(ptr, num_dst, num_edge):
+    """val[e] = 1/deg(row(e)) (src/cpp/src/edge_softmax.cu:186-214)."""
+    return _ops.edge_value_degree(ptr, as_int(num_dst), as_int(num_edge))

@@ -1,0 +1,74 @@
+"""ctypes loader for libcxgnn_hip.so (the C ABI declared in include/cxgnn_hip.h).
+
+The library is built in-tree by ``build.py`` next to this package.  Nothing here
+falls back to another implementation: if the shared object is missing or a call
+fails, a RuntimeError is raised.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (loads the HIP runtime the library links against)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libcxgnn_hip.so"))
+
+_c = ctypes
+_P = _c.c_void_p
+_I64 = _c.c_int64
+_I32 = _c.c_int
+_U32 = _c.c_uint
+_SZ = _c.c_size_t
+_F32 = _c.c_float
+
+# name -> (restype, argtypes); mirrors include/cxgnn_hip.h one to one.
+SIGNATURES = {
+    "cxg_version": (_I32, []),
+    "cxg_last_error": (_c.c_char_p, []),
+    "cxg_spmm_workspace_bytes": (_SZ, [_I64, _I64]),
+    "cxg_spmm_sum_f32": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
+    "cxg_spmm_sum_f32_i32": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
+    "cxg_spmm_weighted_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32,
+                                     _U32, _P, _SZ, _P]),
+    "cxg_csr_transpose_workspace_bytes": (_SZ, [_I64, _I64]),
+    "cxg_csr_transpose_i64": (_I32, [_P, _P, _I64, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
+    "cxg_csr_row_ids_i64": (_I32, [_P, _I64, _I64, _P, _P]),
+    "cxg_edge_value_degree_f32": (_I32, [_P, _I64, _P, _P]),
+    "cxg_pad_rel_i64": (_I32, [_P, _P, _P, _I32, _I32, _I64, _P]),
+}
+
+_lib = None
+
+
+def load():
+    """Return the loaded library, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libcxgnn_hip.so not found at %s; build it with `python build.py` in %s"
+            % (LIB_PATH, os.path.dirname(os.path.dirname(LIB_PATH))))
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != 0:
+        msg = load().cxg_last_error().decode("utf-8", "replace")
+        if status == -1:
+            raise ValueError("cxgnn_hip: " + msg)
+        raise RuntimeError("cxgnn_hip (status %d): %s" % (status, msg))
+
+
+def ptr(t):
+    """Device address of a tensor (None -> NULL)."""
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(device):
+    return torch.cuda.current_stream(device).cuda_stream

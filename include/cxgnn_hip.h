@@ -1,0 +1,140 @@
+/*
+ * cxgnn_hip.h -- C ABI of libcxgnn_hip.so, the gfx950 (MI355X) graph-kernel
+ * library that stands in for the CUDA extension `cxgnncomp_backend` of
+ * xxcclong/CxGNN-Compute (pybind module: src/cpp/python_bindings/binding.cpp:14-130).
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless the name ends in `_host`;
+ *   - graphs are CSR by destination: ptr[n_rows+1], idx[...] = source ids,
+ *     both int64 (`using Index = int64_t`, src/cpp/include/common.h:15) unless a
+ *     function says int32;
+ *   - float tensors are fp32, row-major, contiguous (row stride given where a
+ *     caller may pass a view);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all
+ *     work is enqueued on it and nothing synchronises;
+ *   - every function returns 0 on success or a negative cxg_status; the message
+ *     is available from cxg_last_error() on the calling thread.  Nothing exits or
+ *     aborts the process (the reference's ASSERT macros call exit(1),
+ *     src/cpp/include/common.h:16-26);
+ *   - functions that need scratch memory take `workspace` + `workspace_bytes`;
+ *     the matching *_workspace_bytes() query says how much.  The library never
+ *     allocates device memory in those functions.
+ */
+#ifndef CXGNN_HIP_H
+#define CXGNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum cxg_status {
+  CXG_OK = 0,
+  CXG_ERR_ARG = -1,         /* null pointer, negative size, bad flag */
+  CXG_ERR_UNSUPPORTED = -2, /* shape outside what the kernels cover */
+  CXG_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+  CXG_ERR_HIP = -4          /* a HIP runtime call or kernel launch failed */
+} cxg_status;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int cxg_version(void);
+/* Message of the last failure on this thread ("" if none). */
+const char* cxg_last_error(void);
+
+/* ------------------------------------------------------------------------- */
+/* SpMM family: out[r, :] = reduce_{e in [ptr[r], ptr[r+1])} w[e] * x[idx[e], :] */
+/* ------------------------------------------------------------------------- */
+
+/* flags for cxg_spmm_* */
+#define CXG_SPMM_MEAN 1u       /* divide each row by its degree; empty rows stay 0 */
+#define CXG_SPMM_ACCUMULATE 2u /* out += result instead of out = result           */
+
+/* Bytes of workspace needed by cxg_spmm_* for a graph whose idx array has
+ * n_edges_cap entries and rows of `row_floats` floats (heads*channels). */
+size_t cxg_spmm_workspace_bytes(int64_t n_edges_cap, int64_t row_floats);
+
+/*
+ * Sum / mean aggregation.  Replaces run_spmm_configurable
+ * (src/cpp/src/spmm_host.cu:6-55; the nine launch integers of that function
+ * have no meaning here), sage_sum_forward / sage_mean_forward
+ * (src/cpp/src/aggr.cu:385-393, kernels src/cpp/src/aggr_kernel.cu:3-53).
+ * Rows [0, n_rows) of `out` are written; edges outside [ptr[0], ptr[n_rows])
+ * are ignored; n_edges_cap is the length of idx (>= ptr[n_rows]).
+ */
+int cxg_spmm_sum_f32(const int64_t* ptr, const int64_t* idx, const float* x,
+                     int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
+                     int64_t n_edges_cap, int feat, unsigned flags,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same with int32 ptr/idx.  Replaces run_spmm_configurable_int32
+ * (src/cpp/src/spmm_host.cu:99-156). */
+int cxg_spmm_sum_f32_i32(const int32_t* ptr, const int32_t* idx, const float* x,
+                         int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
+                         int64_t n_edges_cap, int feat, unsigned flags,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Edge-weighted aggregation, single- or multi-head:
+ *   out[r, h, c] = sum_e val[vrow(e), h] * x[idx[e], h, c],
+ *   vrow(e) = val_perm ? val_perm[e] : e.
+ * x is [n_src, heads, channels] (row stride ldx floats), val is
+ * [n_val_rows, heads].  Replaces sage_sum_forward_edge_value
+ * (src/cpp/src/aggr.cu:377-383, kernels aggr_kernel.cu:88-116,155-186) and
+ * spmm_multihead(..., Naive) (src/cpp/src/spmm_host.cu:158-196).  With
+ * val_perm = the edge permutation of a transposed CSR it also computes the
+ * input gradient A^T(val .* g) that the reference obtains with atomics
+ * (aggr_kernel.cu:287-319,403-441; spmm_multihead_bwd spmm_host.cu:198-214).
+ */
+int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx,
+                          const float* val, const int64_t* val_perm,
+                          const float* x, int64_t ldx, float* out, int64_t ldo,
+                          int64_t n_rows, int64_t n_edges_cap, int heads,
+                          int channels, unsigned flags, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Index work (bit-exact)                                                     */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * Transposed CSR of a CSR-by-destination graph with ptr[0] == 0 and
+ * n_edges == ptr[n_rows]:  ptr_t[n_cols+1], idx_t[n_edges] = destination row of
+ * each edge, perm[n_edges] = position of that edge in the original idx array.
+ * Edges of one source keep their original order (stable), so the transposed
+ * gather adds contributions in a fixed order.  This is the graph the backward
+ * pass runs cxg_spmm_* over; the reference reaches the same sums by atomic
+ * scatter (run_spmm_configurable_bwd, src/cpp/src/spmm_host.cu:57-97;
+ * gen_bwd_sum, src/cpp/src/aggr_kernel.cu:220-249).
+ */
+size_t cxg_csr_transpose_workspace_bytes(int64_t n_edges, int64_t n_cols);
+int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows,
+                          int64_t n_cols, int64_t n_edges, int64_t* ptr_t,
+                          int64_t* idx_t, int64_t* perm, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* rows[k] = row that owns edge position ptr[0] + k, k in [0, n_edges): the
+ * device form of `repeat_interleave(arange(n), deg)` used by
+ * SpMMValOP.backward (cxgnncomp/graph_kernel.py:31-34). */
+int cxg_csr_row_ids_i64(const int64_t* ptr, int64_t n_rows, int64_t n_edges,
+                        int64_t* rows, void* stream);
+
+/* out[e] = 1 / degree(row of e) for every edge of rows [0, n_rows).  Replaces
+ * edge_value_degree (src/cpp/src/edge_softmax.cu:186-214). */
+int cxg_edge_value_degree_f32(const int64_t* ptr, int64_t n_rows, float* out,
+                              void* stream);
+
+/*
+ * Relation padding.  For t in [0, num_rel*(thres-1)): r = t/(thres-1),
+ * m = count[r] % thres; rel[base+t] = (m != 0 && t%(thres-1) < thres-m) ? r
+ * : num_rel; if idx is not NULL, idx[base+t] = -1.  Replaces pad_rel and
+ * pad_rel_idx (src/cpp/src/stitch_kernel.cu:3-53).
+ */
+int cxg_pad_rel_i64(int64_t* rel, int64_t* idx, const int64_t* count, int thres,
+                    int num_rel, int64_t base, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CXGNN_HIP_H */
