@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Headline benchmark: forward + backward CSR-by-destination sum SpMM on the
+synthetic 2,449,029-node / 61,859,140-edge power-law graph, F=128 fp32, on one
+MI355X, through the C ABI of libcxgnn_hip.so.
+
+One step = one forward pass (out = A x over ptr/idx) plus one backward pass
+(grad_x = A^T g over the cached transposed CSR).  Graph generation, the
+transposition and all allocations of inputs happen before the timed region;
+inputs are resident in HBM when timing starts.
+
+Prints ONE JSON line.  ``value`` is the effective bandwidth: algorithmic bytes
+of the gather model (every edge fetches its 4F-byte source row and its 8-byte
+index; every output row is written once; ptr is read once) divided by time.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "cxgnn-compute_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the span kernel on the headline workload, from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy kernel;
+# the summaries are kept under profiles/.  None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE x 2.0000 + WRITE_SIZE x 1.0000 of one spmm_span_kernel launch
+    "c3_powerlaw_2.45M_nodes_61.9M_edges_F128": 25948237917,
+}
+
+WORKLOADS = {
+    # name: (nodes, undirected pairs, feature width)
+    "c3_powerlaw_2.45M_nodes_61.9M_edges_F128": (2449029, 30929570, 128),
+    "c2_powerlaw_169k_nodes_2.33M_edges_F128": (169343, 1166243, 128),
+}
+
+
+def spmm_bytes(n_rows, n_edges, feat, index_bytes=8):
+    return n_edges * (4 * feat + index_bytes) + 4 * n_rows * feat + index_bytes * (n_rows + 1)
+
+
+def cpu_baseline(ptr, idx, ptr_t, idx_t, n_nodes, feat, budget_s=12.0):
+    """The reference's own PyTorch SpMM (torch.sparse.mm on a CSR tensor,
+    cxgnncomp/codegen/torch_spmm.py:4-9, restated in oracle/pyref.py) on the
+    host cores, forward on (ptr, idx) and backward on the transposed CSR, over
+    a row prefix of the same graph sized to fit the time budget."""
+    import torch
+    from oracle import pyref
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(n_nodes, feat, generator=g)
+    ptr_c, idx_c = ptr.cpu(), idx.cpu()
+    ptrt_c, idxt_c = ptr_t.cpu(), idx_t.cpu()
+
+    def one(rows):
+        t0 = time.perf_counter()
+        pyref.spmm_torch(x, ptr_c, idx_c, rows)
+        pyref.spmm_torch(x, ptrt_c, idxt_c, rows)
+        return time.perf_counter() - t0
+
+    rows = max(1, n_nodes // 64)
+    t = one(rows)                      # also warms the thread pool
+    t = one(rows)
+    edges = int(ptr_c[rows]) + int(ptrt_c[rows])
+    per_edge = t / max(1, edges)
+    total_edges = int(ptr_c[n_nodes]) + int(ptrt_c[n_nodes])
+    frac = min(1.0, budget_s / 3.0 / max(per_edge * total_edges, 1e-9))
+    rows = max(1, int(n_nodes * frac))
+    times = [one(rows) for _ in range(3)]
+    t = sorted(times)[1]
+    nbytes = (spmm_bytes(rows, int(ptr_c[rows]), feat) + spmm_bytes(rows, int(ptrt_c[rows]), feat))
+    return {
+        "value": nbytes / t / 1e9,
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "torch.sparse.mm(CSR) fwd+bwd on the first %d of %d rows (%d edges) of the same graph, "
+                  "median of 3 runs, %.2f s each" % (rows, n_nodes, int(ptr_c[rows]) + int(ptrt_c[rows]), t),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3_powerlaw_2.45M_nodes_61.9M_edges_F128",
+                    choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three plain device copies of x (known size) before the timed "
+                         "region, to normalise rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
+    from cxgnncomp import synthetic
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    n_nodes, n_pairs, feat = WORKLOADS[args.workload]
+    ptr, idx = synthetic.powerlaw_symmetric_graph(n_nodes, n_pairs, seed=args.seed, device=dev)
+    n_edges = idx.shape[0]
+    torch.manual_seed(args.seed)
+    x = torch.randn(n_nodes, feat, device=dev)
+    grad_out = torch.randn(n_nodes, feat, device=dev)
+    graph_t = _ops.transposed(ptr, idx, n_nodes, n_nodes)   # one-time preparation, not timed
+    torch.cuda.synchronize()
+
+    if args.copy_probe:
+        probe = torch.empty_like(x)
+        for _ in range(3):
+            probe.copy_(x)
+        torch.cuda.synchronize()
+        del probe
+
+    zeros9 = (0,) * 9
+
+    def step(events=None):
+        if events is not None:
+            e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+            e0.record()
+        out = B.run_spmm_configurable(ptr, idx, x, n_nodes, *zeros9)
+        if events is not None:
+            e1.record()
+        gx = B.run_spmm_configurable_bwd(ptr, idx, x, grad_out, n_nodes, *zeros9)
+        if events is not None:
+            e2.record()
+            events.append((e0, e1, e2))
+        return out, gx
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(events)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    bytes_pass = spmm_bytes(n_nodes, n_edges, feat)
+    bytes_step = 2 * bytes_pass
+    flops_step = 2 * n_edges * feat
+    value = bytes_step / (ms_per_step * 1e-3) / 1e9
+
+    # Per-launch device time of the aggregation (span kernel + its fix-up) from
+    # HIP events recorded on the stream the kernels run on.
+    durs = []
+    for e0, e1, e2 in events:
+        durs.append(e0.elapsed_time(e1))
+        durs.append(e1.elapsed_time(e2))
+    launch_ms = sum(durs) / len(durs)
+    achieved = bytes_pass / (launch_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
+
+    result = {
+        "metric": "SpMM fwd+bwd GB/s (% of HBM peak) + GFLOP/s at 61.9M edges, F=128, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "nodes": n_nodes, "edges": n_edges, "feat": feat,
+                   "index_dtype": "int64", "op": "sum SpMM forward + transposed-graph backward"},
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "gflops": round(flops_step / (ms_per_step * 1e-3) / 1e9, 1),
+        "algorithmic_bytes_per_step": bytes_step,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "spmm_span_kernel (+ spmm_fixup_kernel), one cxg_spmm_sum_f32 call",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": traffic,
+            "launch_ms": round(launch_ms, 4),
+            "algorithmic_bytes_per_launch": bytes_pass,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(ptr, idx, graph_t.ptr_t, graph_t.idx_t, n_nodes, feat)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
