@@ -1,0 +1,283 @@
+// SDDMM for gfx950: per-edge dot products of a gathered source row with a
+// destination row,   out[e,h] = sum_c a[src(e),h,c] * b[dst(e),(h,)c].
+//
+// Two entry points share the inner product code:
+//   * CSR order (edges of a destination are consecutive): the destination row
+//     is loaded once per row and kept in registers while the wave streams the
+//     row's edges -- the reference's vertex-centric SDDMM
+//     (src/cpp/src/sddmm_kernel.cu:27-278) and the edge-value gradient fused in
+//     its weighted-SpMM backward (src/cpp/src/aggr_kernel.cu:321-361,443-491);
+//   * COO order (explicit src/dst arrays): sddmm_multihead
+//     (src/cpp/src/sddmm_kernel.cu:3-25).
+// Work is cut into spans of consecutive edges, one wavefront per span, like the
+// SpMM kernels; every output element is written exactly once (no atomics).
+#include "cxg_common.hpp"
+
+namespace cxg {
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
+constexpr int kSpan = 256;
+
+template <int V> struct Vec;
+template <> struct Vec<1> { using type = float; };
+template <> struct Vec<2> { using type = float2; };
+template <> struct Vec<4> { using type = float4; };
+
+__device__ __forceinline__ float vdot(float a, float b) { return a * b; }
+__device__ __forceinline__ float vdot(float2 a, float2 b) { return a.x * b.x + a.y * b.y; }
+__device__ __forceinline__ float vdot(float4 a, float4 b) {
+  return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+}
+template <int V> __device__ __forceinline__ typename Vec<V>::type vzero();
+template <> __device__ __forceinline__ float vzero<1>() { return 0.f; }
+template <> __device__ __forceinline__ float2 vzero<2>() { return make_float2(0.f, 0.f); }
+template <> __device__ __forceinline__ float4 vzero<4>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+
+// Sum over aligned groups of `group` lanes (power of two <= 64); every lane of a
+// group ends with the group's total.
+__device__ __forceinline__ float group_sum(float v, int group) {
+  for (int m = 1; m < group; m <<= 1) v += __shfl_xor(v, m, CXG_WAVE);
+  return v;
+}
+
+struct SddmmArgs {
+  const int64_t* ptr;   // CSR form
+  const int64_t* idx;
+  const int64_t* src;   // COO form
+  const int64_t* dst;
+  const float* a;       // [n_src, heads, channels]
+  const float* b;       // [n_dst, heads, channels] or [n_dst, channels]
+  float* out;           // [n_edges, heads]
+  int64_t n_rows, n_edges;
+  int heads, channels;
+  int b_heads;          // 1: b has a head dimension
+  int group;            // lanes per head = channels / V   (packed kernels)
+};
+
+// Packed layout: the heads*channels floats of a row are spread over the 64 lanes,
+// V consecutive floats per lane (heads*channels <= 64*V), `group` lanes per head.
+template <int V>
+__global__ __launch_bounds__(kBlock) void sddmm_csr_packed_kernel(SddmmArgs a) {
+  using vec_t = typename Vec<V>::type;
+  constexpr int U = (V == 4) ? 8 : 16;
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t n_rows = a.n_rows;
+  const int64_t e_begin = a.ptr[0];
+  const int64_t e_end = a.ptr[n_rows];
+  const int64_t e0 = e_begin + s * kSpan;
+  if (e0 >= e_end) return;
+  const int n = (int)((e_end - e0) < (int64_t)kSpan ? (e_end - e0) : (int64_t)kSpan);
+  const int F = a.heads * a.channels;
+  const int group = a.group;
+  const bool active = lane * V < F;
+  const int head = active ? (lane / group) : 0;
+  const int bcol = a.b_heads ? lane * V : (lane % group) * V;
+  const int64_t ldb = a.b_heads ? F : a.channels;
+  const bool writer = active && (lane % group == 0);
+
+  // row containing e0: last r with ptr[r] <= e0  (skip empty rows that start at e0)
+  int64_t r = wave_lower_bound(a.ptr, n_rows + 1, e0 + 1) - 1;
+  int64_t rbase = r;
+  auto load_row_ends = [&](int64_t rb) -> int {
+    int64_t q = rb + 1 + lane;
+    if (q > n_rows) q = n_rows;
+    const int64_t d = (int64_t)a.ptr[q] - e0;
+    return (int)(d < (int64_t)n + 1 ? d : (int64_t)n + 1);
+  };
+  int row_ends = load_row_ends(rbase);
+  int cur_end = bcast_i32(row_ends, 0);
+  vec_t brow = active ? *reinterpret_cast<const vec_t*>(a.b + r * ldb + bcol) : vzero<V>();
+
+  for (int c0 = 0; c0 < n; c0 += CXG_WAVE) {
+    const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
+    int64_t my_src = 0;
+    if (lane < cn) my_src = a.idx[e0 + c0 + lane];
+    for (int b0 = 0; b0 < cn; b0 += U) {
+      vec_t v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (b0 + u < cn) {
+          const int64_t src = bcast_i64(my_src, b0 + u);
+          v[u] = active ? *reinterpret_cast<const vec_t*>(a.a + src * F + lane * V) : vzero<V>();
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (b0 + u < cn) {
+          const int j = c0 + b0 + u;
+          while (j >= cur_end) {
+            ++r;
+            if (r - rbase == CXG_WAVE) { rbase = r; row_ends = load_row_ends(rbase); }
+            cur_end = bcast_i32(row_ends, (int)(r - rbase));
+            if (j < cur_end)
+              brow = active ? *reinterpret_cast<const vec_t*>(a.b + r * ldb + bcol) : vzero<V>();
+          }
+          const float p = group_sum(vdot(v[u], brow), group);
+          if (writer) a.out[(e0 + j) * a.heads + head] = p;
+        }
+      }
+    }
+  }
+}
+
+template <int V>
+__global__ __launch_bounds__(kBlock) void sddmm_coo_packed_kernel(SddmmArgs a) {
+  using vec_t = typename Vec<V>::type;
+  constexpr int U = (V == 4) ? 4 : 8;
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t e0 = s * kSpan;
+  if (e0 >= a.n_edges) return;
+  const int n = (int)((a.n_edges - e0) < (int64_t)kSpan ? (a.n_edges - e0) : (int64_t)kSpan);
+  const int F = a.heads * a.channels;
+  const int group = a.group;
+  const bool active = lane * V < F;
+  const int head = active ? (lane / group) : 0;
+  const int bcol = a.b_heads ? lane * V : (lane % group) * V;
+  const int64_t ldb = a.b_heads ? F : a.channels;
+  const bool writer = active && (lane % group == 0);
+  for (int c0 = 0; c0 < n; c0 += CXG_WAVE) {
+    const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
+    int64_t my_src = 0, my_dst = 0;
+    if (lane < cn) { my_src = a.src[e0 + c0 + lane]; my_dst = a.dst[e0 + c0 + lane]; }
+    for (int b0 = 0; b0 < cn; b0 += U) {
+      vec_t va[U], vb[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (b0 + u < cn) {
+          const int64_t src = bcast_i64(my_src, b0 + u);
+          const int64_t dst = bcast_i64(my_dst, b0 + u);
+          va[u] = active ? *reinterpret_cast<const vec_t*>(a.a + src * F + lane * V) : vzero<V>();
+          vb[u] = active ? *reinterpret_cast<const vec_t*>(a.b + dst * ldb + bcol) : vzero<V>();
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (b0 + u < cn) {
+          const float p = group_sum(vdot(va[u], vb[u]), group);
+          if (writer) a.out[(e0 + c0 + b0 + u) * a.heads + head] = p;
+        }
+      }
+    }
+  }
+}
+
+// General layout (any heads / channels): one wave-wide reduction per (edge, head).
+// COO == false walks CSR rows (dst = row), COO == true reads src/dst arrays.
+template <bool COO>
+__global__ __launch_bounds__(kBlock) void sddmm_general_kernel(SddmmArgs a) {
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t e_begin = COO ? 0 : a.ptr[0];
+  const int64_t e_end = COO ? a.n_edges : a.ptr[a.n_rows];
+  const int64_t e0 = e_begin + s * kSpan;
+  if (e0 >= e_end) return;
+  const int n = (int)((e_end - e0) < (int64_t)kSpan ? (e_end - e0) : (int64_t)kSpan);
+  const int C = a.channels, H = a.heads;
+  int64_t r = 0;
+  if (!COO) r = wave_lower_bound(a.ptr, a.n_rows + 1, e0 + 1) - 1;
+  for (int j = 0; j < n; ++j) {
+    const int64_t e = e0 + j;
+    int64_t src, dst;
+    if (COO) {
+      src = a.src[e];
+      dst = a.dst[e];
+    } else {
+      while (e >= a.ptr[r + 1]) ++r;
+      src = a.idx[e];
+      dst = r;
+    }
+    for (int h = 0; h < H; ++h) {
+      const float* pa = a.a + (src * H + h) * C;
+      const float* pb = a.b_heads ? a.b + (dst * H + h) * C : a.b + dst * C;
+      float p = 0.f;
+      for (int c = lane; c < C; c += CXG_WAVE) p += pa[c] * pb[c];
+      p = group_sum(p, CXG_WAVE);
+      if (lane == 0) a.out[e * H + h] = p;
+    }
+  }
+}
+
+bool is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+
+// Vector width for the packed kernels, or 0 if the shape needs the general one.
+int packed_vec(const SddmmArgs& a) {
+  const int F = a.heads * a.channels;
+  const uintptr_t bits = (uintptr_t)a.a | (uintptr_t)a.b;
+  for (int v = 1; v <= 4; v *= 2) {
+    if (a.channels % v != 0) break;
+    if ((bits & (uintptr_t)(4 * v - 1)) != 0) break;
+    const int g = a.channels / v;
+    if (F <= CXG_WAVE * v && is_pow2(g) && g <= CXG_WAVE) return v;
+  }
+  return 0;
+}
+
+int check_common(const float* a, const float* b, float* out, int heads, int channels) {
+  CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
+  CXG_REQUIRE(a && b && out, CXG_ERR_ARG, "null feature/output pointer");
+  return CXG_OK;
+}
+
+}  // namespace
+}  // namespace cxg
+
+extern "C" {
+
+int cxg_sddmm_csr_f32(const int64_t* ptr, const int64_t* idx, const float* src_feat,
+                      const float* dst_feat, float* out, int64_t n_rows, int64_t n_edges_cap,
+                      int heads, int channels, int dst_has_heads, void* stream) {
+  CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
+  if (n_rows == 0 || n_edges_cap == 0) return CXG_OK;
+  CXG_REQUIRE(ptr && idx, CXG_ERR_ARG, "null ptr/idx");
+  int rc = cxg::check_common(src_feat, dst_feat, out, heads, channels);
+  if (rc) return rc;
+  cxg::SddmmArgs a{};
+  a.ptr = ptr; a.idx = idx; a.a = src_feat; a.b = dst_feat; a.out = out;
+  a.n_rows = n_rows; a.n_edges = n_edges_cap; a.heads = heads; a.channels = channels;
+  a.b_heads = dst_has_heads ? 1 : 0;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)cxg::ceil_div(cxg::ceil_div(n_edges_cap, cxg::kSpan), cxg::kWavesPerBlock));
+  dim3 block(cxg::kBlock);
+  const int v = cxg::packed_vec(a);
+  if (v) a.group = channels / v;
+  if (v == 4) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<4>, grid, block, 0, st, a);
+  else if (v == 2) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<2>, grid, block, 0, st, a);
+  else if (v == 1) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<1>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(cxg::sddmm_general_kernel<false>, grid, block, 0, st, a);
+  CXG_LAUNCH_CHECK("sddmm_csr kernel");
+  return CXG_OK;
+}
+
+int cxg_sddmm_coo_f32(const int64_t* src, const int64_t* dst, const float* src_feat,
+                      const float* dst_feat, float* out, int64_t n_edges, int heads, int channels,
+                      int dst_has_heads, void* stream) {
+  CXG_REQUIRE(n_edges >= 0, CXG_ERR_ARG, "negative size");
+  if (n_edges == 0) return CXG_OK;
+  CXG_REQUIRE(src && dst, CXG_ERR_ARG, "null src/dst");
+  int rc = cxg::check_common(src_feat, dst_feat, out, heads, channels);
+  if (rc) return rc;
+  cxg::SddmmArgs a{};
+  a.src = src; a.dst = dst; a.a = src_feat; a.b = dst_feat; a.out = out;
+  a.n_edges = n_edges; a.heads = heads; a.channels = channels;
+  a.b_heads = dst_has_heads ? 1 : 0;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)cxg::ceil_div(cxg::ceil_div(n_edges, cxg::kSpan), cxg::kWavesPerBlock));
+  dim3 block(cxg::kBlock);
+  const int v = cxg::packed_vec(a);
+  if (v) a.group = channels / v;
+  if (v == 4) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<4>, grid, block, 0, st, a);
+  else if (v == 2) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<2>, grid, block, 0, st, a);
+  else if (v == 1) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<1>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(cxg::sddmm_general_kernel<true>, grid, block, 0, st, a);
+  CXG_LAUNCH_CHECK("sddmm_coo kernel");
+  return CXG_OK;
+}
+
+}  // extern "C"

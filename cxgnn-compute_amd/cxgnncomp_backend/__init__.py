@@ -129,3 +129,108 @@ Optimal = SPMM_MULTIHEAD_SCHEDULE.Optimal
 def edge_value_degree(ptr, num_dst, num_edge):
     """val[e] = 1/deg(row(e)) (src/cpp/src/edge_softmax.cu:186-214)."""
     return _ops.edge_value_degree(ptr, as_int(num_dst), as_int(num_edge))
+
+
+def spmm_multihead(ptr, idx, val, vin, num_node, schedule=Optimal, block_size=256):
+    """src/cpp/src/spmm_host.cu:158-196.  Naive: out[r,h,c]; PreReduce/Optimal:
+    out[r,c] summed over heads."""
+    if vin.dim() != 3:
+        raise ValueError("vin must be 3D, [num_node, num_head, feat_len]")
+    if val.dim() != 2:
+        raise ValueError("val must be 2D, [num_edge, num_head]")
+    if val.shape[1] != vin.shape[1]:
+        raise ValueError("num_head mismatch %d %d" % (vin.shape[1], val.shape[1]))
+    out = _ops.spmm(ptr, idx, vin, as_int(num_node), val=val)
+    if SPMM_MULTIHEAD_SCHEDULE(int(schedule)) == SPMM_MULTIHEAD_SCHEDULE.Naive:
+        return out
+    return _ops.head_sum(out)
+
+
+def run_spmm_multihead_configurable(ptr, idx, val, vin, num_node, *launch_ints):
+    """src/cpp/src/spmm_host.cu:216-256: head-pre-reduced output [num_node, feat]."""
+    return spmm_multihead(ptr, idx, val, vin, num_node, PreReduce)
+
+
+def spmm_multihead_bwd(ptr, idx, val, grad_output, grad_x, num_node, schedule=Optimal, block_size=256):
+    """grad_x[idx[e],h,:] += val[e,h] * grad_output[r,h,:] into the caller's grad_x
+    (src/cpp/src/spmm_host.cu:198-214)."""
+    n = as_int(num_node)
+    g = _ops.transposed(ptr, idx, n, grad_x.shape[0])
+    _ops.spmm(g.ptr_t, g.idx_t, grad_output.contiguous(), grad_x.shape[0], val=val, val_perm=g.perm,
+              out=grad_x, accumulate=True)
+
+
+# --------------------------------------------------------------------------- #
+# SDDMM  (binding.cpp:76-79)
+# --------------------------------------------------------------------------- #
+def run_sddmm(src, dst, src_feat, dst_feat, output, num_edge):
+    """output[e,h] = <src_feat[src[e],h,:], dst_feat[dst[e],(h,):]>
+    (src/cpp/src/sddmm_host.cu:4-14).  A 2-D dst_feat is shared by all heads as
+    in the reference kernel; a 3-D dst_feat is taken per head."""
+    _ops.sddmm_coo(src, dst, src_feat, dst_feat, output, as_int(num_edge))
+
+
+def run_sddmm_vertex_centric(ptr, idx, src_feat, dst_feat, num_node, *launch_ints):
+    """Same values in CSR edge order, new [E,H] tensor (src/cpp/src/sddmm_host.cu:16-59)."""
+    return _ops.sddmm_csr(ptr, idx, src_feat, dst_feat, as_int(num_node))
+
+
+# --------------------------------------------------------------------------- #
+# edge attention  (binding.cpp:22-25, 33)
+# --------------------------------------------------------------------------- #
+class _EdgeSoftmaxFunction(torch.autograd.Function):
+    """EdgeSoftMaxFunction (src/cpp/src/edge_softmax.cu:97-177)."""
+
+    @staticmethod
+    def forward(ctx, ptr, idx, att_dst, att_src, num_edge, relu_l):
+        att_dst = att_dst.contiguous()
+        att_src = att_src.contiguous()
+        out, mask = _ops.edge_softmax_fwd(ptr, idx, att_dst, att_src, as_int(num_edge), relu_l)
+        ctx.save_for_backward(ptr, idx, out, mask)
+        ctx.n_dst, ctx.n_src, ctx.slope = att_dst.shape[0], att_src.shape[0], float(relu_l)
+        ctx.mark_non_differentiable(mask)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        ptr, idx, out, mask = ctx.saved_tensors
+        g_dst, t_edge = _ops.edge_softmax_bwd(ptr, out, mask, grad_out.contiguous(), ctx.n_dst, ctx.slope)
+        g = _ops.transposed(ptr, idx, ctx.n_dst, ctx.n_src)
+        g_src = _ops.narrow_gather_sum(g.ptr_t, g.perm, t_edge, ctx.n_src)
+        return None, None, g_dst, g_src, None, None
+
+
+def edge_attention(ptr, idx, att_dst, att_src, num_edge, relu_l):
+    """softmax_row(leaky_relu(att_dst[r] + att_src[idx[e]])) -> [num_edge, heads]
+    (src/cpp/src/edge_softmax.cu:179-184; note dst before src)."""
+    return _EdgeSoftmaxFunction.apply(ptr, idx, att_dst, att_src, num_edge, relu_l)
+
+
+def spmv(ptr, idx, input, num_dst):
+    """out[r] = sum_e input[idx[e]] (src/cpp/src/edge_softmax.cu:234-244)."""
+    return _ops.narrow_gather_sum(ptr, idx, input, as_int(num_dst))
+
+
+# --------------------------------------------------------------------------- #
+# gather (edge -> node scatter-add)  (binding.cpp:19)
+# --------------------------------------------------------------------------- #
+class _GatherFunction(torch.autograd.Function):
+    """GatherFunction (src/cpp/src/aggr.cu:395-448)."""
+
+    @staticmethod
+    def forward(ctx, input, dest, num_node):
+        n = as_int(num_node)
+        if n <= 0:
+            raise ValueError("num_node must be > 0")
+        ctx.save_for_backward(dest)
+        return _ops.scatter_add_rows(input.contiguous(), dest, n)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (dest,) = ctx.saved_tensors
+        return _ops.gather_rows(grad_out.contiguous(), dest), None, None
+
+
+def gather(input, dest, num_node):
+    """out[dest[e]] += input[e], out [num_node, F] (src/cpp/src/aggr.cu:445-448)."""
+    return _GatherFunction.apply(input, dest, num_node)

@@ -29,6 +29,14 @@ SIGNATURES = {
     "cxg_spmm_sum_f32_i32": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
     "cxg_spmm_weighted_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32,
                                      _U32, _P, _SZ, _P]),
+    "cxg_sddmm_csr_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P]),
+    "cxg_sddmm_coo_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "cxg_edge_softmax_fwd_f32": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I32, _F32, _P]),
+    "cxg_edge_softmax_bwd_f32": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I32, _F32, _P]),
+    "cxg_narrow_gather_sum_f32": (_I32, [_P, _P, _P, _P, _I64, _I32, _P]),
+    "cxg_scatter_add_rows_f32": (_I32, [_P, _P, _P, _I64, _I32, _P]),
+    "cxg_gather_rows_f32": (_I32, [_P, _P, _P, _I64, _I32, _P]),
+    "cxg_head_sum_f32": (_I32, [_P, _P, _I64, _I32, _I32, _P]),
     "cxg_csr_transpose_workspace_bytes": (_SZ, [_I64, _I64]),
     "cxg_csr_transpose_i64": (_I32, [_P, _P, _I64, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
     "cxg_csr_row_ids_i64": (_I32, [_P, _I64, _I64, _P, _P]),

@@ -213,3 +213,173 @@ def csr_row_ids(ptr, n_rows, n_edges):
                                      _lib.current_stream(ptr.device))
     _lib.check(st)
     return rows
+
+
+# --------------------------------------------------------------------------- #
+# SDDMM / edge softmax / narrow row sums
+# --------------------------------------------------------------------------- #
+def _feat3(t, name):
+    _req(t, name, torch.float32, (2, 3))
+    return t if t.dim() == 3 else t.unsqueeze(1)
+
+
+def sddmm_csr(ptr, idx, src_feat, dst_feat, n_rows, out_shape=None, out=None):
+    """out[e,h] = <src_feat[idx[e],h,:], dst_feat[row(e),(h,):]> in CSR edge order.
+
+    src_feat [Ns,H,C] or [Ns,C]; dst_feat [Nd,H,C], or [Nd,C] (shared by all
+    heads when H > 1).  Result is [E,H] ([E] when out_shape says so)."""
+    lib = _lib.load()
+    _check_graph(ptr, idx, n_rows)
+    a = _feat3(src_feat, "src_feat")
+    heads, channels = a.shape[1], a.shape[2]
+    _req(dst_feat, "dst_feat", torch.float32, (2, 3))
+    if dst_feat.dim() == 3:
+        b_heads = 1
+        if dst_feat.shape[1] != heads or dst_feat.shape[2] != channels:
+            raise ValueError("dst_feat shape %s does not match src_feat %s"
+                             % (tuple(dst_feat.shape), tuple(src_feat.shape)))
+    else:
+        b_heads = 1 if heads == 1 else 0
+        if dst_feat.shape[1] != channels:
+            raise ValueError("dst_feat has %d channels, src_feat %d" % (dst_feat.shape[1], channels))
+    if dst_feat.shape[0] < n_rows:
+        raise ValueError("dst_feat has fewer rows than num_node")
+    n_cap = idx.shape[0]
+    if out is None:
+        out = torch.zeros((n_cap, heads), dtype=torch.float32, device=a.device)
+    else:
+        _req(out, "out", torch.float32)
+        if out.numel() < n_cap * heads:
+            raise ValueError("output too small")
+    with torch.cuda.device(a.device):
+        st = lib.cxg_sddmm_csr_f32(ptr.data_ptr(), _lib.ptr(idx), a.data_ptr(), dst_feat.data_ptr(),
+                                   out.data_ptr(), n_rows, n_cap, heads, channels, b_heads,
+                                   _lib.current_stream(a.device))
+    _lib.check(st)
+    if out_shape is not None:
+        return out.reshape(out_shape)
+    return out
+
+
+def sddmm_coo(src, dst, src_feat, dst_feat, out, n_edges):
+    lib = _lib.load()
+    _req(src, "src", torch.int64, 1)
+    _req(dst, "dst", torch.int64, 1)
+    if src.shape[0] < n_edges or dst.shape[0] < n_edges:
+        raise ValueError("src/dst shorter than num_edge")
+    a = _feat3(src_feat, "src_feat")
+    heads, channels = a.shape[1], a.shape[2]
+    _req(dst_feat, "dst_feat", torch.float32, (2, 3))
+    if dst_feat.dim() == 3:
+        b_heads = 1
+        if dst_feat.shape[1] != heads or dst_feat.shape[2] != channels:
+            raise ValueError("dst_feat shape does not match src_feat")
+    else:
+        b_heads = 1 if heads == 1 else 0
+        if dst_feat.shape[1] != channels:
+            raise ValueError("dst_feat has %d channels, src_feat %d" % (dst_feat.shape[1], channels))
+    _req(out, "output", torch.float32)
+    if out.numel() < n_edges * heads:
+        raise ValueError("output too small")
+    with torch.cuda.device(a.device):
+        st = lib.cxg_sddmm_coo_f32(src.data_ptr(), dst.data_ptr(), a.data_ptr(), dst_feat.data_ptr(),
+                                   out.data_ptr(), n_edges, heads, channels, b_heads,
+                                   _lib.current_stream(a.device))
+    _lib.check(st)
+    return out
+
+
+def edge_softmax_fwd(ptr, idx, att_dst, att_src, n_edges, slope):
+    lib = _lib.load()
+    _req(att_dst, "att_dst", torch.float32, 2)
+    _req(att_src, "att_src", torch.float32, 2)
+    n_dst, heads = att_dst.shape
+    if att_src.shape[1] != heads:
+        raise ValueError("att_src/att_dst head mismatch")
+    _check_graph(ptr, idx, n_dst)
+    if idx.shape[0] < n_edges:
+        raise ValueError("idx shorter than num_edge")
+    out = torch.empty((n_edges, heads), dtype=torch.float32, device=att_dst.device)
+    mask = torch.empty((n_edges, heads), dtype=torch.bool, device=att_dst.device)
+    with torch.cuda.device(att_dst.device):
+        st = lib.cxg_edge_softmax_fwd_f32(ptr.data_ptr(), _lib.ptr(idx), att_dst.data_ptr(),
+                                          att_src.data_ptr(), _lib.ptr(out), _lib.ptr(mask), n_dst,
+                                          heads, float(slope), _lib.current_stream(att_dst.device))
+    _lib.check(st)
+    return out, mask
+
+
+def edge_softmax_bwd(ptr, out, mask, grad, n_dst, slope):
+    """Returns (g_dst [n_dst,H], t_edge [E,H])."""
+    lib = _lib.load()
+    _req(out, "out", torch.float32, 2)
+    _req(grad, "grad", torch.float32, 2)
+    _req(mask, "mask", torch.bool, 2)
+    heads = out.shape[1]
+    g_dst = torch.empty((n_dst, heads), dtype=torch.float32, device=out.device)
+    t_edge = torch.zeros_like(out)
+    with torch.cuda.device(out.device):
+        st = lib.cxg_edge_softmax_bwd_f32(ptr.data_ptr(), _lib.ptr(out), _lib.ptr(mask), _lib.ptr(grad),
+                                          _lib.ptr(g_dst), _lib.ptr(t_edge), n_dst, heads, float(slope),
+                                          _lib.current_stream(out.device))
+    _lib.check(st)
+    return g_dst, t_edge
+
+
+def narrow_gather_sum(ptr, sel, inp, n_rows):
+    """out[r,:] = sum_{k in row r} inp[sel[k],:] (sel None: inp[k,:]); inp [M] or [M,W]."""
+    lib = _lib.load()
+    _req(ptr, "ptr", torch.int64, 1)
+    if n_rows + 1 > ptr.shape[0]:
+        raise ValueError("num rows does not fit ptr")
+    if sel is not None:
+        _req(sel, "sel", torch.int64, 1)
+    _req(inp, "input", torch.float32, (1, 2))
+    width = 1 if inp.dim() == 1 else inp.shape[1]
+    shape = (n_rows,) if inp.dim() == 1 else (n_rows, width)
+    out = torch.empty(shape, dtype=torch.float32, device=inp.device)
+    with torch.cuda.device(inp.device):
+        st = lib.cxg_narrow_gather_sum_f32(ptr.data_ptr(), _lib.ptr(sel), _lib.ptr(inp), _lib.ptr(out),
+                                           n_rows, width, _lib.current_stream(inp.device))
+    _lib.check(st)
+    return out
+
+
+def head_sum(x):
+    """[N, H, C] -> [N, C], summed over heads."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 3)
+    out = torch.empty((x.shape[0], x.shape[2]), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_head_sum_f32(_lib.ptr(x), _lib.ptr(out), x.shape[0], x.shape[1], x.shape[2],
+                                  _lib.current_stream(x.device))
+    _lib.check(st)
+    return out
+
+
+def scatter_add_rows(inp, dest, n_nodes):
+    """out[dest[e]] += inp[e] into a fresh zero [n_nodes, F] tensor."""
+    lib = _lib.load()
+    _req(inp, "input", torch.float32, 2)
+    _req(dest, "dest", torch.int64, 1)
+    if inp.shape[0] < dest.shape[0]:
+        raise ValueError("input has fewer rows than dest")
+    out = torch.zeros((n_nodes, inp.shape[1]), dtype=torch.float32, device=inp.device)
+    with torch.cuda.device(inp.device):
+        st = lib.cxg_scatter_add_rows_f32(_lib.ptr(inp), _lib.ptr(dest), _lib.ptr(out), dest.shape[0],
+                                          inp.shape[1], _lib.current_stream(inp.device))
+    _lib.check(st)
+    return out
+
+
+def gather_rows(inp, sel):
+    """out[e] = inp[sel[e]]."""
+    lib = _lib.load()
+    _req(inp, "input", torch.float32, 2)
+    _req(sel, "sel", torch.int64, 1)
+    out = torch.empty((sel.shape[0], inp.shape[1]), dtype=torch.float32, device=inp.device)
+    with torch.cuda.device(inp.device):
+        st = lib.cxg_gather_rows_f32(_lib.ptr(inp), _lib.ptr(sel), _lib.ptr(out), sel.shape[0],
+                                     inp.shape[1], _lib.current_stream(inp.device))
+    _lib.check(st)
+    return out

@@ -95,6 +95,80 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx,
                           size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- */
+/* SDDMM and edge softmax                                                      */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * out[e, h] = sum_c src_feat[idx[e], h, c] * dst_feat[row(e), (h,) c] for every
+ * edge position e in [ptr[0], ptr[n_rows]); out is indexed by edge position and
+ * has `heads` floats per edge.  dst_has_heads = 0 means dst_feat is
+ * [n_dst, channels] (the layout of the reference kernels), 1 means
+ * [n_dst, heads, channels].  Replaces run_sddmm_vertex_centric
+ * (src/cpp/src/sddmm_host.cu:16-59) and the edge-value gradient of
+ * gen_bwd_sum_edge_value[_multi_head]_edge_grad
+ * (src/cpp/src/aggr_kernel.cu:321-361,443-491).
+ */
+int cxg_sddmm_csr_f32(const int64_t* ptr, const int64_t* idx, const float* src_feat,
+                      const float* dst_feat, float* out, int64_t n_rows,
+                      int64_t n_edges_cap, int heads, int channels,
+                      int dst_has_heads, void* stream);
+
+/* Same product over explicit src[e] / dst[e] arrays.  Replaces run_sddmm
+ * (src/cpp/src/sddmm_host.cu:4-14, kernel src/cpp/src/sddmm_kernel.cu:3-25). */
+int cxg_sddmm_coo_f32(const int64_t* src, const int64_t* dst, const float* src_feat,
+                      const float* dst_feat, float* out, int64_t n_edges, int heads,
+                      int channels, int dst_has_heads, void* stream);
+
+/*
+ * GAT edge attention: out[e,h] = softmax over the edges of row r of
+ * leaky_relu(att_dst[r,h] + att_src[idx[e],h], slope); mask[e,h] = (pre-softmax
+ * activation > 0).  att_dst is [n_dst, heads], att_src [n_src, heads], out and
+ * mask [n_edges, heads]; rows without edges write nothing.  Replaces
+ * edge_softmax_fwd (src/cpp/src/edge_softmax.cu:3-42, host :97-132).
+ */
+int cxg_edge_softmax_fwd_f32(const int64_t* ptr, const int64_t* idx,
+                             const float* att_dst, const float* att_src, float* out,
+                             uint8_t* mask, int64_t n_dst, int heads, float slope,
+                             void* stream);
+
+/*
+ * Backward of the above (edge_softmax_bwd, src/cpp/src/edge_softmax.cu:44-95):
+ * s = sum_row out*grad; t = out*(grad - s) * (mask ? 1 : slope);
+ * g_dst[r,h] = sum_row t when the row has activations of both signs, else 0;
+ * t_edge[e,h] = t.  The source gradient g_src[s,h] = sum over the edges leaving
+ * s of t is obtained with cxg_narrow_gather_sum_f32 over the transposed CSR
+ * (sel = its edge permutation) where the reference uses atomicAdd (:85).
+ */
+int cxg_edge_softmax_bwd_f32(const int64_t* ptr, const float* out, const uint8_t* mask,
+                             const float* grad, float* g_dst, float* t_edge,
+                             int64_t n_dst, int heads, float slope, void* stream);
+
+/* out[r, 0..width) = sum_{k in [ptr[r], ptr[r+1])} in[sel ? sel[k] : k, 0..width)
+ * for narrow rows (a few floats).  With width 1 and sel = idx this is spmv
+ * (src/cpp/src/edge_softmax.cu:216-244). */
+int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const float* in,
+                              float* out, int64_t n_rows, int width, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Row helpers                                                                 */
+/* ------------------------------------------------------------------------- */
+
+/* out[dest[e], :] += in[e, :] for e < n_edges (fp32 hardware atomics; the caller
+ * zeroes out).  Replaces gather_fwd (src/cpp/src/aggr.cu:42-51, host :395-421). */
+int cxg_scatter_add_rows_f32(const float* in, const int64_t* dest, float* out,
+                             int64_t n_edges, int feat, void* stream);
+
+/* out[e, :] = in[sel[e], :] for e < n_rows_out.  Replaces gather_bwd
+ * (src/cpp/src/aggr.cu:53-62, host :423-443). */
+int cxg_gather_rows_f32(const float* in, const int64_t* sel, float* out,
+                        int64_t n_rows_out, int feat, void* stream);
+
+/* out[n, c] = sum_h in[n, h, c]: the head reduction of the PreReduce / Optimal
+ * schedules of spmm_multihead (src/cpp/src/spmm_multihead_kernel.cu:3-36). */
+int cxg_head_sum_f32(const float* in, float* out, int64_t n_rows, int heads,
+                     int channels, void* stream);
+
+/* ------------------------------------------------------------------------- */
 /* Index work (bit-exact)                                                     */
 /* ------------------------------------------------------------------------- */
 
