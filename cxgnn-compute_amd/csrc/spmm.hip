@@ -62,11 +62,27 @@ struct SpmmArgs {
   int mean, accumulate;
   float* carry;            // [n_spans_cap][2][F]: head partial, tail partial
   int64_t* tail_row;       // [n_spans_cap]: row whose tail partial the span holds, or -1
+  // extended gather (EXT kernels only); every pointer may be null
+  const uint8_t* mask;     // skip edges whose mask byte is 0
+  const int64_t* mask_perm;// mask index of edge position (null: the position itself)
+  const int32_t* rel;      // source row += rel[e] * rel_stride
+  int64_t rel_stride;
+  const int64_t* src_map;  // source row = src_map[source row]
+  const int64_t* targets;  // row r is added (atomically) into out[targets[r]]
 };
+
+__device__ __forceinline__ void atomic_add_vec(float* p, float v) { unsafeAtomicAdd(p, v); }
+__device__ __forceinline__ void atomic_add_vec(float* p, float2 v) {
+  unsafeAtomicAdd(p, v.x); unsafeAtomicAdd(p + 1, v.y);
+}
+__device__ __forceinline__ void atomic_add_vec(float* p, float4 v) {
+  unsafeAtomicAdd(p, v.x); unsafeAtomicAdd(p + 1, v.y);
+  unsafeAtomicAdd(p + 2, v.z); unsafeAtomicAdd(p + 3, v.w);
+}
 
 // WMODE: 0 = unweighted, 1 = one weight per edge (heads == 1), 2 = one weight
 // per edge and head (each lane's V columns lie in one head).
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, int U>
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int U>
 __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   using vec_t = typename Vec<V>::type;
   const int lane = lane_id();
@@ -128,6 +144,8 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   auto finish_row = [&]() {
     if (is_head) {
       store_vec(carry_head, acc);
+    } else if (EXT && a.targets) {
+      if (col_ok && cur_end > cur_start) atomic_add_vec(a.out + a.targets[r] * a.ldo + col, acc);
     } else {
       float* dst = a.out + r * a.ldo;
       if (a.mean) {
@@ -150,6 +168,11 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     if (lane < cn) {
       const int64_t pos = e0 + c0 + lane;
       my_src = (int64_t)a.idx[pos];
+      if (EXT) {
+        if (a.rel) my_src += (int64_t)a.rel[pos] * a.rel_stride;
+        if (a.src_map) my_src = a.src_map[my_src];
+        if (a.mask && !a.mask[a.mask_perm ? a.mask_perm[pos] : pos]) my_src = -1;
+      }
       if (PERM) my_vrow = a.perm[pos];
       if (WMODE == 1 && !PERM) my_w = a.val[pos];
     }
@@ -162,7 +185,8 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
         if (jj < cn) {
           const int64_t src = bcast_i64(my_src, jj);
           const float* row = a.x + src * a.ldx;
-          v[u] = col_ok ? *reinterpret_cast<const vec_t*>(row + col) : vzero<V>();
+          if (EXT && src < 0) v[u] = vzero<V>();
+          else v[u] = col_ok ? *reinterpret_cast<const vec_t*>(row + col) : vzero<V>();
           if (WMODE == 1) {
             if (PERM) w[u] = a.val[bcast_i64(my_vrow, jj)];
             else w[u] = bcast_f32(my_w, jj);
@@ -233,6 +257,10 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   vec_t acc = *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * s + 1) * F + col);
   for (int64_t q = s + 1; q <= s_last; ++q)
     vadd(acc, *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * q) * F + col));
+  if (a.targets) {
+    atomic_add_vec(a.out + a.targets[t] * a.ldo + col, acc);
+    return;
+  }
   if (a.mean) vscale(acc, 1.0f / (float)(row_end - row_begin));
   float* dst = a.out + t * a.ldo;
   if (a.accumulate) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
@@ -265,20 +293,20 @@ Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
   return p;
 }
 
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM>
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT>
 int launch_spmm(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
   constexpr int U = (V == 4) ? 8 : 16;
   const int tile = CXG_WAVE * V;
   dim3 grid((unsigned)ceil_div(n_spans_cap, kWavesPerBlock), (unsigned)ceil_div(a.F, tile), 1);
   dim3 block(kBlock, 1, 1);
-  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, U>), grid, block, 0, stream, a);
+  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U>), grid, block, 0, stream, a);
   CXG_LAUNCH_CHECK("spmm_span_kernel");
   hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, V, GUARD>), grid, block, 0, stream, a);
   CXG_LAUNCH_CHECK("spmm_fixup_kernel");
   return CXG_OK;
 }
 
-template <typename IdxT, int WMODE, bool PERM>
+template <typename IdxT, int WMODE, bool PERM, bool EXT = false>
 int dispatch_shape(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
   // widest vector that divides the row (and the head, for per-head weights) and
   // keeps every access aligned; among those the one needing the fewest column
@@ -296,19 +324,28 @@ int dispatch_shape(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t str
   const bool guard = (best_tiles * CXG_WAVE * best_v != a.F);
 #define CXG_CASE(VV)                                                                  \
   if (best_v == VV) {                                                                  \
-    return guard ? launch_spmm<IdxT, VV, true, WMODE, PERM>(a, n_spans_cap, stream)   \
-                 : launch_spmm<IdxT, VV, false, WMODE, PERM>(a, n_spans_cap, stream); \
+    return guard ? launch_spmm<IdxT, VV, true, WMODE, PERM, EXT>(a, n_spans_cap, stream)   \
+                 : launch_spmm<IdxT, VV, false, WMODE, PERM, EXT>(a, n_spans_cap, stream); \
   }
   CXG_CASE(1) CXG_CASE(2) CXG_CASE(4)
 #undef CXG_CASE
   return set_error(CXG_ERR_UNSUPPORTED, "no kernel for vector width %d", best_v);
 }
 
+struct SpmmExt {
+  const uint8_t* mask = nullptr;
+  const int64_t* mask_perm = nullptr;
+  const int32_t* rel = nullptr;
+  int64_t rel_stride = 0;
+  const int64_t* src_map = nullptr;
+  const int64_t* targets = nullptr;
+};
+
 template <typename IdxT>
 int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_t* perm,
                 const float* x, int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
                 int64_t n_edges_cap, int heads, int channels, unsigned flags, void* workspace,
-                size_t workspace_bytes, void* stream) {
+                size_t workspace_bytes, void* stream, const SpmmExt* ext = nullptr) {
   CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
   CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
   CXG_REQUIRE((int64_t)heads * channels <= (1 << 20), CXG_ERR_UNSUPPORTED, "row too wide");
@@ -333,7 +370,17 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   a.accumulate = (flags & CXG_SPMM_ACCUMULATE) ? 1 : 0;
   a.tail_row = reinterpret_cast<int64_t*>(workspace);
   a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
+  a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0;
+  a.src_map = nullptr; a.targets = nullptr;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (ext) {
+    CXG_REQUIRE(!val, CXG_ERR_UNSUPPORTED, "extended gather takes no edge weights");
+    CXG_REQUIRE(!(ext->targets && a.mean), CXG_ERR_ARG, "targets cannot be combined with mean");
+    a.mask = ext->mask; a.mask_perm = ext->mask_perm; a.rel = ext->rel; a.rel_stride = ext->rel_stride;
+    a.src_map = ext->src_map; a.targets = ext->targets;
+    if constexpr (sizeof(IdxT) == 8) return dispatch_shape<IdxT, 0, false, true>(a, plan.n_spans_cap, st);
+    return set_error(CXG_ERR_UNSUPPORTED, "extended gather needs int64 indices");
+  }
   if (!val) return dispatch_shape<IdxT, 0, false>(a, plan.n_spans_cap, st);
   if constexpr (sizeof(IdxT) == 8) {
     if (heads == 1) {
@@ -378,6 +425,20 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx, const float* v
   if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
   return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
                                    heads, channels, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_ext_f32(const int64_t* ptr, const int64_t* idx, const float* x, int64_t ldx, float* out,
+                     int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int feat, unsigned flags,
+                     const uint8_t* mask, const int64_t* mask_perm, const int32_t* rel,
+                     int64_t rel_stride, const int64_t* src_map, const int64_t* targets,
+                     void* workspace, size_t workspace_bytes, void* stream) {
+  cxg::SpmmExt ext;
+  ext.mask = mask; ext.mask_perm = mask_perm; ext.rel = rel; ext.rel_stride = rel_stride;
+  ext.src_map = src_map; ext.targets = targets;
+  if (mask_perm && !mask) return cxg::set_error(CXG_ERR_ARG, "mask_perm without mask");
+  if (rel && rel_stride <= 0) return cxg::set_error(CXG_ERR_ARG, "rel needs a positive rel_stride");
+  return cxg::spmm_common<int64_t>(ptr, idx, nullptr, nullptr, x, ldx, out, ldo, n_rows, n_edges_cap,
+                                   1, feat, flags, workspace, workspace_bytes, stream, &ext);
 }
 
 }  // extern "C"

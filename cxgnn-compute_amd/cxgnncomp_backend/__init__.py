@@ -234,3 +234,6 @@ class _GatherFunction(torch.autograd.Function):
 def gather(input, dest, num_node):
     """out[dest[e]] += input[e], out [num_node, F] (src/cpp/src/aggr.cu:445-448)."""
     return _GatherFunction.apply(input, dest, num_node)
+
+from ._rel import (aggr_rel, selective_aggr, selective_aggr_bwd, target_aggr,  # noqa: E402,F401
+                   target_aggr_backward)

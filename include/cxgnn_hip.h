@@ -94,6 +94,42 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx,
                           int channels, unsigned flags, void* workspace,
                           size_t workspace_bytes, void* stream);
 
+/*
+ * Sum aggregation with optional extras, each enabled by a non-NULL pointer:
+ *   mask      [E] bytes: edges whose byte is 0 are skipped; the byte of edge
+ *             position e is mask[mask_perm ? mask_perm[e] : e];
+ *   rel       [E] int32: the gathered row is x[rel[e]*rel_stride + idx[e]];
+ *   src_map   the gathered row is x[src_map[...]];
+ *   targets   [n_rows]: row r is added with fp32 atomics into out[targets[r]]
+ *             (out must be initialised by the caller) instead of stored.
+ * Replaces selective_aggr / selective_aggr_bwd (src/cpp/src/aggr.cu:483-514,
+ * kernels aggr_kernel.cu:493-555; use CXG_SPMM_ACCUMULATE, and for the backward
+ * the transposed CSR with mask_perm = its edge permutation), target_aggr /
+ * target_aggr_backward (aggr.cu:450-481, aggr_kernel.cu:557-607; backward =
+ * transposed CSR with src_map = targets and CXG_SPMM_ACCUMULATE) and aggr_rel
+ * forward (src/cpp/src/rel_spmm.cu:8-70).
+ */
+int cxg_spmm_ext_f32(const int64_t* ptr, const int64_t* idx, const float* x,
+                     int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
+                     int64_t n_edges_cap, int feat, unsigned flags,
+                     const uint8_t* mask, const int64_t* mask_perm,
+                     const int32_t* rel, int64_t rel_stride,
+                     const int64_t* src_map, const int64_t* targets,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Transposed aggregation by atomic scatter into the caller's buffer:
+ *   gx[idx[e] (+ rel[e]*rel_stride), :] += (val ? val[e] : 1) * g[row(e), :]
+ * for unmasked edges of rows [0, n_rows).  Replaces aggr_rel_bwd
+ * (src/cpp/src/rel_spmm.cu:72-136) and is the no-preprocessing form of
+ * gen_bwd_sum (src/cpp/src/aggr_kernel.cu:220-249).
+ */
+int cxg_spmm_scatter_atomic_f32(const int64_t* ptr, const int64_t* idx,
+                                const int32_t* rel, int64_t rel_stride,
+                                const float* val, const uint8_t* mask,
+                                const float* g, float* gx, int64_t n_rows,
+                                int64_t n_edges_cap, int feat, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* SDDMM and edge softmax                                                      */
 /* ------------------------------------------------------------------------- */
