@@ -237,3 +237,6 @@ def gather(input, dest, num_node):
 
 from ._rel import (aggr_rel, selective_aggr, selective_aggr_bwd, target_aggr,  # noqa: E402,F401
                    target_aggr_backward)
+from ._typed import (aggr_rel_direct, aggr_rgcn_direct_func, pad_rel, pad_rel_idx,  # noqa: E402,F401
+                     seastar_backward, seastar_forward, typed_linear, typed_linear_s2d,
+                     typed_linear_s2e)

@@ -1,0 +1,241 @@
+"""Typed GEMM, relation segmentation and the relational ops built on them
+(binding.cpp:45-54): pad_rel*, typed_linear*, aggr_rel_direct,
+aggr_rgcn_direct_func, seastar_*."""
+import torch
+
+from . import _lib, _ops
+from ._ops import _req, _workspace, as_int
+
+GEMM_ACCUMULATE = 1
+GEMM_ATOMIC = 2
+
+
+def rel_segment(types, num_rel):
+    """Stable grouping of rows by relation: returns (perm [n] int64, seg_ptr [num_rel+1] int64)."""
+    lib = _lib.load()
+    if types.dtype not in (torch.int32, torch.int64):
+        raise ValueError("types must be int32 or int64, got %s" % types.dtype)
+    _req(types, "types", types.dtype, 1)
+    n = types.shape[0]
+    dev = types.device
+    perm = torch.empty(n, dtype=torch.int64, device=dev)
+    seg = torch.empty(num_rel + 1, dtype=torch.int64, device=dev)
+    nb = 4 if types.dtype == torch.int32 else 8
+    ws = _workspace(lib.cxg_rel_segment_workspace_bytes(n, num_rel, nb), dev)
+    fn = lib.cxg_rel_segment_i32 if nb == 4 else lib.cxg_rel_segment_i64
+    with torch.cuda.device(dev):
+        st = fn(_lib.ptr(types), n, num_rel, _lib.ptr(perm), seg.data_ptr(), ws.data_ptr(), ws.numel(),
+                _lib.current_stream(dev))
+    _lib.check(st)
+    return perm, seg
+
+
+def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n_out=None,
+               accumulate=False, atomic=False, bf16=False):
+    """out[dst(i)] (=|+=) a[src(i)] @ w[r] for rows i of segment r (see cxg_typed_gemm_f32).
+
+    a [*, K] fp32, w [R, K, N] fp32.  With bf16=True the operands are rounded to
+    bf16 (W transposed to [R, N, K]) and multiplied on the bf16 matrix cores."""
+    lib = _lib.load()
+    _req(a, "a", torch.float32 if not (bf16 and a.dtype == torch.bfloat16) else torch.bfloat16, 2)
+    if w.dim() != 3:
+        raise ValueError("weights must be [num_rel, K, N]")
+    R, K, N = w.shape
+    if a.shape[1] != K:
+        raise ValueError("incompatible dimensions: a has %d columns, weights K=%d" % (a.shape[1], K))
+    _req(seg_ptr, "seg_ptr", torch.int64, 1)
+    if seg_ptr.shape[0] < R + 1:
+        raise ValueError("seg_ptr needs num_rel+1 entries")
+    for t, name in ((src_idx, "src_idx"), (dst_idx, "dst_idx")):
+        if t is not None:
+            _req(t, name, torch.int64, 1)
+            if t.shape[0] < m_rows:
+                raise ValueError("%s shorter than the number of rows" % name)
+    if src_idx is None and a.shape[0] < m_rows:
+        raise ValueError("a has fewer rows than M")
+    if out is None:
+        if n_out is None:
+            n_out = m_rows
+        out = torch.empty((n_out, N), dtype=torch.float32, device=a.device)
+    else:
+        _req(out, "output", torch.float32, 2)
+        if out.shape[1] != N:
+            raise ValueError("output has %d columns, weights N=%d" % (out.shape[1], N))
+    if dst_idx is None and out.shape[0] < m_rows:
+        raise ValueError("output has fewer rows than M")
+    flags = (GEMM_ACCUMULATE if accumulate else 0) | (GEMM_ATOMIC if atomic else 0)
+    stream = _lib.current_stream(a.device)
+    with torch.cuda.device(a.device):
+        if bf16:
+            a16 = a if a.dtype == torch.bfloat16 else a.to(torch.bfloat16)
+            wt16 = w.detach().transpose(1, 2).contiguous().to(torch.bfloat16)
+            st = lib.cxg_typed_gemm_bf16(a16.data_ptr(), K, wt16.data_ptr(), out.data_ptr(), N,
+                                         _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
+                                         m_rows, K, N, R, flags, stream)
+        else:
+            _req(w, "weights", torch.float32, 3)
+            st = lib.cxg_typed_gemm_f32(a.data_ptr(), K, w.data_ptr(), out.data_ptr(), N,
+                                        _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
+                                        m_rows, K, N, R, flags, stream)
+    _lib.check(st)
+    return out
+
+
+# --------------------------------------------------------------------------- #
+# pad_rel / pad_rel_idx  (binding.cpp:51-52)
+# --------------------------------------------------------------------------- #
+def _pad_rel(rel, idx, count, thres, num_rel, base):
+    lib = _lib.load()
+    thres, num_rel, base = int(thres), int(num_rel), as_int(base)
+    _req(rel, "rel", torch.int64, 1)
+    _req(count, "count", torch.int64, 1)
+    if count.shape[0] < num_rel:
+        raise ValueError("count has %d entries, num_rel=%d (use bincount(minlength=num_rel))"
+                         % (count.shape[0], num_rel))
+    need = base + num_rel * (thres - 1)
+    if rel.shape[0] < need:
+        raise ValueError("rel has %d entries, %d needed" % (rel.shape[0], need))
+    if idx is not None:
+        _req(idx, "idx", torch.int64, 1)
+        if idx.shape[0] < need:
+            raise ValueError("idx has %d entries, %d needed" % (idx.shape[0], need))
+    with torch.cuda.device(rel.device):
+        st = lib.cxg_pad_rel_i64(rel.data_ptr(), _lib.ptr(idx), count.data_ptr(), thres, num_rel, base,
+                                 _lib.current_stream(rel.device))
+    _lib.check(st)
+
+
+def pad_rel(rel, count, thres, num_rel, base):
+    """In place on rel (src/cpp/src/stitch_kernel.cu:23-38,48-53)."""
+    _pad_rel(rel, None, count, thres, num_rel, base)
+
+
+def pad_rel_idx(rel, idx, count, thres, num_rel, base):
+    """In place on rel and idx (src/cpp/src/stitch_kernel.cu:3-21,40-46)."""
+    _pad_rel(rel, idx, count, thres, num_rel, base)
+
+
+# --------------------------------------------------------------------------- #
+# per-row typed linear  (binding.cpp:48-50)
+# --------------------------------------------------------------------------- #
+def _typed_rows(vin, weights, output, types, src_id, dst_id, atomic):
+    if types.dtype != torch.int32:
+        raise ValueError("types must be int32")
+    num = types.shape[0] if src_id is None else src_id.shape[0]
+    if num == 0:
+        return
+    perm, seg = rel_segment(types[:num].contiguous(), weights.shape[0])
+    src = perm if src_id is None else src_id[perm]
+    dst = perm if dst_id is None else dst_id[perm]
+    typed_gemm(vin, weights, seg, num, src_idx=src, dst_idx=dst, out=output, accumulate=True,
+               atomic=atomic)
+
+
+def typed_linear(vin, weights, output, types, in_feat_tile=32):
+    """output[i] += vin[i] @ weights[types[i]] (src/cpp/src/rel_spmm.cu:231-269)."""
+    _typed_rows(vin, weights, output, types, None, None, False)
+
+
+def typed_linear_s2e(vin, weights, output, src_id, types, in_feat_tile=32):
+    """output[i] += vin[src_id[i]] @ weights[types[i]] (src/cpp/src/rel_spmm.cu:271-312)."""
+    _typed_rows(vin, weights, output, types, src_id, None, False)
+
+
+def typed_linear_s2d(vin, weights, output, src_id, dst_id, types, in_feat_tile=32):
+    """output[dst_id[i]] += vin[src_id[i]] @ weights[types[i]], atomically
+    (src/cpp/src/rel_spmm.cu:314-358)."""
+    _typed_rows(vin, weights, output, types, src_id, dst_id, True)
+
+
+# --------------------------------------------------------------------------- #
+# fused relational aggregate + transform  (binding.cpp:46-47, 53-54)
+# --------------------------------------------------------------------------- #
+def _edge_segments(ptr, idx, rel, n, num_rel):
+    n_edges = int(ptr[n].item())
+    perm, seg = rel_segment(rel[:n_edges].contiguous(), num_rel)
+    rows = _ops.csr_row_ids(ptr, n, n_edges)
+    return n_edges, idx[:n_edges][perm], rows[perm], seg
+
+
+def _weight_grad(x, g, src, dst, seg, shape):
+    """grad_W[r] = sum over the rows of segment r of x[src]^T g[dst]; the row
+    gather is ours, the K x cnt x N product per relation is a plain library GEMM."""
+    gw = torch.zeros(shape, dtype=torch.float32, device=x.device)
+    bounds = seg.tolist()
+    for r in range(shape[0]):
+        b, e = bounds[r], bounds[r + 1]
+        if e > b:
+            xs = _ops.gather_rows(x, src[b:e].contiguous())
+            gs = _ops.gather_rows(g, dst[b:e].contiguous())
+            gw[r] = torch.mm(xs.t(), gs)
+    return gw
+
+
+class _RgcnFusedFunction(torch.autograd.Function):
+    """out[r] = sum_e x[idx[e]] @ W[rel[e]] (aggr_rgcn_direct_kernel,
+    src/cpp/src/rel_spmm.cu:138-181).  The reference's backward returns zeros
+    (rel_spmm.cu:400-432); the true gradients are computed here."""
+
+    @staticmethod
+    def forward(ctx, x, ptr, idx, weights, rel, num_node):
+        n = as_int(num_node)
+        if n == 0:
+            n = ptr.shape[0] - 1
+        if x.shape[1] != weights.shape[1]:
+            raise ValueError("feat_len weight size %d %d" % (x.shape[1], weights.shape[1]))
+        x = x.contiguous()
+        weights = weights.contiguous()
+        n_edges, src, dst, seg = _edge_segments(ptr, idx, rel, n, weights.shape[0])
+        out = torch.zeros((n, weights.shape[2]), dtype=torch.float32, device=x.device)
+        typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=dst, out=out, atomic=True)
+        ctx.save_for_backward(x, weights, src, dst, seg)
+        ctx.n_edges = n_edges
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weights, src, dst, seg = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        gx = gw = None
+        if ctx.needs_input_grad[0]:
+            gx = torch.zeros_like(x)
+            typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), seg, ctx.n_edges, src_idx=dst,
+                       dst_idx=src, out=gx, atomic=True)
+        if ctx.needs_input_grad[3]:
+            gw = _weight_grad(x, grad_out, src, dst, seg, weights.shape)
+        return gx, None, None, gw, None, None
+
+
+def aggr_rgcn_direct_func(input, ptr, idx, weights, rel, num_node):
+    """src/cpp/src/rel_spmm.cu:442-467 (rel int32)."""
+    if weights.dim() != 3:
+        raise ValueError("weights must be [num_rel, in, out]")
+    return _RgcnFusedFunction.apply(input, ptr, idx, weights, rel, num_node)
+
+
+def aggr_rel_direct(input, ptr, idx, weights, etype, num_node, num_rel):
+    """src/cpp/src/rel_spmm.cu:434-440."""
+    if int(num_rel) != weights.shape[0]:
+        raise ValueError("num_rel=%d but weights has %d relations" % (int(num_rel), weights.shape[0]))
+    return _RgcnFusedFunction.apply(input, ptr, idx, weights, etype, num_node)
+
+
+def seastar_forward(input, ptr, idx, weights, etype):
+    """Seastar RGCN baseline forward (src/cpp/src/rel_spmm.cu:469-521): the same
+    sum_e x[idx[e]] @ W[etype[e]] over all rows of ptr."""
+    with torch.no_grad():
+        return _RgcnFusedFunction.apply(input, ptr, idx, weights, etype, ptr.shape[0] - 1)
+
+
+def seastar_backward(input, ptr, idx, weights, etype, grad):
+    """Returns [grad_input, grad_weights] (src/cpp/src/rel_spmm.cu:523-579)."""
+    n = ptr.shape[0] - 1
+    x = input.contiguous()
+    weights = weights.contiguous()
+    grad = grad.contiguous()
+    n_edges, src, dst, seg = _edge_segments(ptr, idx, etype, n, weights.shape[0])
+    gx = torch.zeros_like(x)
+    typed_gemm(grad, weights.transpose(1, 2).contiguous(), seg, n_edges, src_idx=dst, dst_idx=src, out=gx,
+               atomic=True)
+    gw = _weight_grad(x, grad, src, dst, seg, weights.shape)
+    return [gx, gw]

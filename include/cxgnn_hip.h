@@ -186,6 +186,55 @@ int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const floa
                               float* out, int64_t n_rows, int width, void* stream);
 
 /* ------------------------------------------------------------------------- */
+/* Typed (relation-segmented) GEMM -- the MFMA path                            */
+/* ------------------------------------------------------------------------- */
+
+#define CXG_GEMM_ACCUMULATE 1u /* C += A W instead of C = A W                      */
+#define CXG_GEMM_ATOMIC 2u     /* add with fp32 atomics (several rows share a dst) */
+
+/*
+ * C[dst(i), :] = A[src(i), :] @ W[r] for the rows i in [seg_ptr[r], seg_ptr[r+1]),
+ * r in [0, R); src(i) = src_idx ? src_idx[i] : i, dst(i) = dst_idx ? dst_idx[i] : i;
+ * a negative src or dst skips the row.  A is [*, K] (row stride lda), W is
+ * [R, K, N], C is [*, N] (row stride ldc), all fp32; seg_ptr is a device array of
+ * R+1 row offsets (see cxg_rel_segment_*).  Computed with
+ * v_mfma_f32_32x32x2_f32.  Replaces typed_matmul
+ * (cxgnncomp/codegen/triton_typed_matmul.py:752-860: src_idx only = its
+ * "single index" kernel with dst = src, seq_output = dst NULL, both = double
+ * index) and, with row maps and CXG_GEMM_ACCUMULATE / CXG_GEMM_ATOMIC, the
+ * per-row kernels typed_linear / typed_linear_s2e / typed_linear_s2d
+ * (src/cpp/src/rel_spmm.cu:231-358).
+ */
+int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c,
+                       int64_t ldc, const int64_t* src_idx, const int64_t* dst_idx,
+                       const int64_t* seg_ptr, int64_t M, int K, int N, int R,
+                       unsigned flags, void* stream);
+
+/* Same contraction with bf16 operands on v_mfma_f32_32x32x16_bf16: A is bf16
+ * [*, K], w_t is the transposed weight stack W^T as bf16 [R, N, K]; C stays fp32.
+ * K and lda must be multiples of 8. */
+int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, float* c,
+                        int64_t ldc, const int64_t* src_idx, const int64_t* dst_idx,
+                        const int64_t* seg_ptr, int64_t M, int K, int N, int R,
+                        unsigned flags, void* stream);
+
+/*
+ * Relation segmentation: perm[k] = original row of the k-th row in relation
+ * order (stable), seg_ptr[r] = number of rows with relation id < r for r in
+ * [0, num_rel].  Ids equal to num_rel (the padding sentinel of pad_rel) sort
+ * last and are not covered by any segment.  Replaces the bincount + sort of
+ * TypedLinearE2EOP.preprocess / TypedLinearS2DSort
+ * (cxgnncomp/typed_linear.py:74-87,262-283).  index_bytes is 4 or 8.
+ */
+size_t cxg_rel_segment_workspace_bytes(int64_t n, int num_rel, int index_bytes);
+int cxg_rel_segment_i64(const int64_t* types, int64_t n, int num_rel, int64_t* perm,
+                        int64_t* seg_ptr, void* workspace, size_t workspace_bytes,
+                        void* stream);
+int cxg_rel_segment_i32(const int32_t* types, int64_t n, int num_rel, int64_t* perm,
+                        int64_t* seg_ptr, void* workspace, size_t workspace_bytes,
+                        void* stream);
+
+/* ------------------------------------------------------------------------- */
 /* Row helpers                                                                 */
 /* ------------------------------------------------------------------------- */
 

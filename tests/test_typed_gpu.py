@@ -1,0 +1,181 @@
+"""Typed GEMM (MFMA), relation segmentation, pad_rel and the fused RGCN op
+through cxgnncomp_backend vs the oracle.
+
+fp32 MFMA path: 1e-4 relative / 1e-5 absolute at O(1) output scale.
+bf16 MFMA path (stated tolerance): operands are rounded to bf16 (8 significant
+bits), products accumulate in fp32; against the oracle run on the same
+bf16-rounded operands the bound is the fp32 one, against the unrounded fp32
+oracle it is 2e-2 relative to the row scale."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import announce, assert_close
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("n,R", [(0, 3), (1, 1), (1000, 7), (50000, 16), (777, 40)])
+def test_rel_segment_bit_exact(dtype, n, R):
+    from cxgnncomp_backend import _typed
+    g = torch.Generator().manual_seed(n + R)
+    types = torch.randint(0, R + 1, (n,), generator=g).to(dtype)   # value R = padding sentinel
+    announce("rel_segment n=%d R=%d %s" % (n, R, dtype))
+    perm, seg = _typed.rel_segment(types.cuda(), R)
+    t = types.numpy().astype(np.int64)
+    want_perm = np.argsort(t, kind="stable")
+    want_seg = np.searchsorted(t[want_perm], np.arange(R + 1), side="left")
+    assert np.array_equal(_np(perm), want_perm)
+    assert np.array_equal(_np(seg), want_seg)
+
+
+SHAPES = [(128, 128, 16, 5000), (64, 64, 3, 1000), (32, 40, 4, 700), (96, 47, 5, 900),
+          (128, 256, 2, 300), (256, 128, 7, 2000), (64, 200, 1, 130), (128, 16, 6, 999)]
+
+
+def _typed_problem(K, N, R, M, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g) / K ** 0.5
+    w = torch.randn(R, K, N, generator=g)
+    p = torch.arange(1, R + 1, dtype=torch.float64) ** -1.2
+    types = torch.multinomial(p, M, replacement=True, generator=g).to(torch.int32)
+    if R > 2:
+        types[types == 1] = 0                     # one empty relation
+    return x, w, types
+
+
+@pytest.mark.parametrize("K,N,R,M", SHAPES)
+def test_typed_linear_f32(K, N, R, M):
+    import cxgnncomp_backend as B
+    x, w, types = _typed_problem(K, N, R, M, K + N + R)
+    base = torch.randn(M, N) / 8
+    out = base.clone().cuda()
+    announce("typed_linear K=%d N=%d R=%d M=%d" % (K, N, R, M))
+    B.typed_linear(x.cuda(), w.cuda(), out, types.cuda(), 32)
+    torch.cuda.synchronize()
+    ref = oracle.typed_linear(x.numpy(), w.numpy(), types.numpy(), out=base.numpy())
+    assert_close(_np(out), ref, RTOL, 2 * ATOL, "typed_linear")
+
+
+@pytest.mark.parametrize("K,N,R,M", SHAPES[:4])
+def test_typed_linear_s2e_s2d(K, N, R, M):
+    import cxgnncomp_backend as B
+    x, w, types = _typed_problem(K, N, R, M, 3 * K + N)
+    n_src, n_dst = 300, 150
+    g = torch.Generator().manual_seed(1)
+    xs = torch.randn(n_src, K, generator=g) / K ** 0.5
+    src = torch.randint(0, n_src, (M,), generator=g)
+    dst = torch.randint(0, n_dst, (M,), generator=g)
+    out = torch.zeros(M, N).cuda()
+    announce("typed_linear_s2e K=%d N=%d R=%d M=%d" % (K, N, R, M))
+    B.typed_linear_s2e(xs.cuda(), w.cuda(), out, src.cuda(), types.cuda(), 32)
+    ref = oracle.typed_linear(xs.numpy(), w.numpy(), types.numpy(), src=src.numpy(), n_out=M)
+    assert_close(_np(out), ref, RTOL, ATOL, "s2e")
+    out2 = torch.zeros(n_dst, N).cuda()
+    announce("typed_linear_s2d K=%d N=%d R=%d M=%d" % (K, N, R, M))
+    B.typed_linear_s2d(xs.cuda(), w.cuda(), out2, src.cuda(), dst.cuda(), types.cuda(), 32)
+    ref2 = oracle.typed_linear(xs.numpy(), w.numpy(), types.numpy(), src=src.numpy(), dst=dst.numpy(),
+                               n_out=n_dst)
+    scale = max(1.0, float(np.abs(ref2).max()))
+    assert_close(_np(out2) / scale, ref2 / scale, RTOL, ATOL, "s2d")
+
+
+@pytest.mark.parametrize("K,N,R,M", [(128, 128, 16, 5000), (64, 64, 3, 1000), (96, 40, 4, 700),
+                                     (256, 128, 7, 2000)])
+def test_typed_gemm_bf16(K, N, R, M):
+    from cxgnncomp_backend import _typed
+    x, w, types = _typed_problem(K, N, R, M, 5 * K + N)
+    perm, seg = _typed.rel_segment(types.cuda(), R)
+    announce("typed_gemm bf16 K=%d N=%d R=%d M=%d" % (K, N, R, M))
+    out = _typed.typed_gemm(x.cuda(), w.cuda(), seg, M, src_idx=perm, dst_idx=perm, bf16=True)
+    torch.cuda.synchronize()
+    xr = x.to(torch.bfloat16).float().numpy()
+    wr = w.to(torch.bfloat16).float().numpy()
+    ref_rounded = oracle.typed_linear(xr, wr, types.numpy())
+    assert_close(_np(out), ref_rounded, RTOL, 2 * ATOL, "bf16 vs oracle on bf16-rounded operands")
+    ref = oracle.typed_linear(x.numpy(), w.numpy(), types.numpy())
+    scale = np.abs(ref).max()
+    assert np.abs(_np(out) - ref).max() <= 2e-2 * scale, "bf16 vs fp32 oracle"
+
+
+@pytest.mark.parametrize("thres", [256, 32, 2])
+def test_pad_rel_bit_exact(thres):
+    import cxgnncomp_backend as B
+    R, n = 9, 5000
+    g = torch.Generator().manual_seed(thres)
+    types = torch.randint(0, R - 1, (n,), generator=g)          # highest id absent
+    count = torch.bincount(types, minlength=R)
+    new_types = torch.full((n + R * (thres - 1),), -7, dtype=torch.int64)
+    new_types[:n] = types
+    new_idx = torch.full_like(new_types, -9)
+    new_idx[:n] = torch.arange(n)
+    a = new_types.clone().cuda()
+    announce("pad_rel thres=%d" % thres)
+    B.pad_rel(a, count.cuda(), thres, R, n)
+    want = oracle.pad_rel(new_types.numpy(), count.numpy(), thres, R, n)
+    assert np.array_equal(_np(a), want)
+    a2, i2 = new_types.clone().cuda(), new_idx.clone().cuda()
+    announce("pad_rel_idx thres=%d" % thres)
+    B.pad_rel_idx(a2, i2, count.cuda(), thres, R, n)
+    want_r, want_i = oracle.pad_rel(new_types.numpy(), count.numpy(), thres, R, n, idx=new_idx.numpy())
+    assert np.array_equal(_np(a2), want_r) and np.array_equal(_np(i2), want_i)
+    # each relation's padded count is a multiple of thres (what the padding is for)
+    padded = np.bincount(_np(a), minlength=R + 1)[:R]
+    assert (padded % thres == 0).all()
+
+
+def test_rgcn_fused_toy_all_ones():
+    """example/prof_rgcn.py:22-51: x = ones[128,128], W = ones, one row with 31
+    neighbours -> every output element is 31 * 128 = 3968."""
+    import cxgnncomp_backend as B
+    ptr = torch.tensor([0, 31])
+    idx = torch.arange(1, 32)
+    rel = (torch.arange(31) % 7).int()
+    x = torch.ones(128, 128)
+    w = torch.ones(7, 128, 128)
+    announce("rgcn fused toy")
+    out = B.aggr_rgcn_direct_func(x.cuda(), ptr.cuda(), idx.cuda(), w.cuda(), rel.cuda(), 1)
+    assert out.shape == (1, 128)
+    assert torch.all(out.cpu() == 3968.0)
+
+
+@pytest.mark.parametrize("K,N,R", [(128, 128, 16), (64, 32, 3)])
+def test_rgcn_fused_forward_backward(K, N, R):
+    import cxgnncomp_backend as B
+    from cxgnncomp import synthetic as S
+    ptr, idx, etype, _ = S.hetero_graph(3000, 40000, num_rel=R, seed=4)
+    n = ptr.shape[0] - 1
+    torch.manual_seed(14)
+    x = torch.randn(n, K) / (K ** 0.5 * 4)
+    w = torch.randn(R, K, N) * 0.5
+    g = torch.randn(n, N) / 4
+    xg = x.cuda().requires_grad_(True)
+    wg = w.cuda().requires_grad_(True)
+    rel = etype.int()
+    announce("aggr_rel_direct K=%d N=%d R=%d" % (K, N, R))
+    out = B.aggr_rel_direct(xg, ptr.cuda(), idx.cuda(), wg, rel.cuda(), n, R)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.rgcn_fused(x.numpy(), ptr.numpy(), idx.numpy(), w.numpy(), rel.numpy(), n)
+    assert_close(_np(out), ref, RTOL, 2 * ATOL, "rgcn fused fwd")
+    # gradients from autograd through the pure-torch restatement in float64
+    from oracle import pyref
+    x64 = x.double().requires_grad_(True)
+    w64 = w.double().requires_grad_(True)
+    o64 = pyref.typed_linear_s2d_sort(x64, w64, ptr, idx, etype, n)
+    o64.backward(g.double())
+    assert_close(_np(xg.grad), x64.grad.numpy(), RTOL, 2 * ATOL, "grad x")
+    sc = float(w64.grad.abs().max())
+    assert_close(_np(wg.grad) / sc, w64.grad.numpy() / sc, RTOL, 2 * ATOL, "grad w")
+    announce("seastar fwd/bwd K=%d" % K)
+    so = B.seastar_forward(x.cuda(), ptr.cuda(), idx.cuda(), w.cuda(), etype.cuda())
+    assert_close(_np(so), ref, RTOL, 2 * ATOL, "seastar fwd")
+    sgx, sgw = B.seastar_backward(x.cuda(), ptr.cuda(), idx.cuda(), w.cuda(), etype.cuda(), g.cuda())
+    assert_close(_np(sgx), x64.grad.numpy(), RTOL, 2 * ATOL, "seastar grad x")
