@@ -1,0 +1,394 @@
+"""Aggregation autograd ops and graph convolution layers of the reference
+(cxgnncomp/graph_conv.py) on the HIP backend.  Layers take the graph as
+``(ptr, idx)`` = CSR by destination plus the number of destination rows.
+
+PyTorch Geometric and torch_scatter are not needed: ``Linear``/``glorot`` are
+replaced by torch.nn.Linear with Glorot-uniform weights, and the op-wise edge
+softmax is written with core torch ops.
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+from torch.nn import Parameter
+
+import cxgnncomp_backend
+from cxgnncomp_backend import (aggr_rel, aggr_rgcn_direct_func, edge_attention, gather,
+                               sage_mean_forward, sage_sum_forward, sage_sum_forward_edge_value,
+                               selective_aggr, selective_aggr_bwd)
+
+from .graph_kernel import SpMMValOP
+from .timer import TimerOP
+from .typed_linear import (TypedLinearE2EOP, TypedLinearS2DAggrMMOP, TypedLinearS2DMMAggrOP,
+                           TypedLinearS2DPushOP, TypedLinearS2DSort)
+from .util import global_tuner, log
+
+for _name in ("edge_attention", "sage_sum_forward_edge_value", "gather", "sage_sum_forward",
+              "aggr_rel", "sage_mean_forward"):
+    torch.fx.wrap(_name)
+
+
+def glorot(tensor):
+    """Glorot/Xavier uniform over the last two dimensions (what PyG's ``glorot`` does)."""
+    if tensor is not None:
+        bound = math.sqrt(6.0 / (tensor.size(-2) + tensor.size(-1)))
+        tensor.data.uniform_(-bound, bound)
+
+
+def _num(v):
+    return int(v.item()) if isinstance(v, torch.Tensor) else int(v)
+
+
+class AggrOP(torch.autograd.Function):
+    """Sum aggregation through the tuner entry point (upstream :34-77).  Upstream's
+    backward re-runs the forward kernel on grad_out, which equals A^T g only for a
+    symmetric square graph; the backward here is the true transposed aggregation
+    (identical on symmetric graphs)."""
+
+    @staticmethod
+    def forward(ctx, x, ptr, idx, num_center):
+        n = _num(num_center)
+        ctx.save_for_backward(ptr, idx)
+        ctx.n, ctx.n_src = n, x.shape[0]
+        return global_tuner.tune_graph(n, idx.shape[0], x.shape[-1],
+                                       cxgnncomp_backend.run_spmm_configurable,
+                                       [ptr, idx, x.contiguous(), n])
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        ptr, idx = ctx.saved_tensors
+        like = grad_out.new_empty((ctx.n_src, 0))
+        grad_x = global_tuner.tune_graph(ctx.n, idx.shape[0], grad_out.shape[-1],
+                                         cxgnncomp_backend.run_spmm_configurable_bwd,
+                                         [ptr, idx, like, grad_out.contiguous(), ctx.n])
+        return grad_x, None, None, None
+
+
+class AggrDirectedOP(AggrOP):
+    """Upstream :80-114: forward as AggrOP, backward by run_spmm_configurable_bwd --
+    which is what AggrOP does here as well."""
+
+
+class SeastarRGCNOP(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, x, weights, ptr, idx, rel, num_center):
+        rel = rel.to(torch.int64)
+        ctx.save_for_backward(x, weights, ptr, idx, rel)
+        return cxgnncomp_backend.seastar_forward(x, ptr, idx, weights, rel)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weights, ptr, idx, rel = ctx.saved_tensors
+        grad_x, grad_weight = cxgnncomp_backend.seastar_backward(x, ptr, idx, weights, rel, grad_out)
+        return grad_x, grad_weight, None, None, None, None
+
+
+class RGCNOP(torch.autograd.Function):
+    """Transform all nodes per relation, then masked aggregation (upstream :205-243)."""
+
+    @staticmethod
+    def forward(ctx, x, weights, ptr, idx, rel, num_center):
+        n = _num(num_center)
+        ctx.save_for_backward(x, weights, ptr, idx, rel)
+        output = torch.zeros([n, weights.shape[-1]], device=x.device)
+        for i in range(weights.shape[0]):
+            w = TimerOP.apply(weights[i], f"mm{i}", True)
+            t = TimerOP.apply(torch.mm(x, w), f"mm{i}", False)
+            t = TimerOP.apply(t, f"selective{i}", True)
+            selective_aggr(t, ptr, idx, (rel == i), output, n)
+            output = TimerOP.apply(output, f"selective{i}", False)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weights, ptr, idx, rel = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        grad_x = torch.zeros_like(x)
+        grad_weights = []
+        n = grad_out.shape[0]
+        for i in range(weights.shape[0]):
+            g_sel = torch.zeros([x.shape[0], grad_out.shape[-1]], device=x.device)
+            g_sel = TimerOP.apply(g_sel, f"selective_bwd{i}", True)
+            selective_aggr_bwd(grad_out, ptr, idx, (rel == i), g_sel, n)
+            g_sel = TimerOP.apply(g_sel, f"selective_bwd{i}", False)
+            g_sel = TimerOP.apply(g_sel, f"mm_bwd{i}", True)
+            grad_x += torch.mm(g_sel, weights[i].t())
+            g_sel = TimerOP.apply(g_sel, f"mm_bwd{i}", False)
+            grad_weights.append(torch.mm(x.t(), g_sel))
+        return grad_x, torch.stack(grad_weights), None, None, None, None
+
+
+def RGCNOP_sorted(x, weights, src, dst, num_feat_per_rel, num_center):
+    """Edges pre-sorted by relation: per segment gather -> linear -> index_add_ (:246-257)."""
+    output = torch.zeros([num_center, weights.shape[-1]], device=x.device)
+    start = 0
+    for i in range(weights.shape[0]):
+        c = int(num_feat_per_rel[i])
+        output.index_add_(0, dst[start:start + c], F.linear(x[src[start:start + c]], weights[i].T))
+        start += c
+    return output
+
+
+RGCNOP2 = TypedLinearS2DAggrMMOP          # aggregate-then-transform variant (upstream :260-292)
+
+
+class RGCNOP3(torch.autograd.Function):
+    """Fused aggregate+transform (upstream :295-306, whose backward returns random
+    tensors); the gradients here are the true ones."""
+
+    @staticmethod
+    def forward(ctx, x, weights, ptr, idx, rel, num_center):
+        with torch.enable_grad():
+            xd = x.detach().requires_grad_(True)
+            wd = weights.detach().requires_grad_(True)
+            out = aggr_rgcn_direct_func(xd, ptr, idx, wd, rel.int(), _num(num_center))
+        ctx.inner = (xd, wd, out)
+        return out.detach()
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        xd, wd, out = ctx.inner
+        gx, gw = torch.autograd.grad(out, (xd, wd), grad_out)
+        return gx, gw, None, None, None, None
+
+
+def run_rgcn4(x, ptr, idx, edge_types, linear, num_center, num_edge, preproccessed):
+    """Gather source rows per edge, typed transform edge->edge, sum the consecutive
+    edge rows of every destination (upstream :309-326)."""
+    x_idxed = x[idx[:num_edge]]
+    out = TypedLinearE2EOP.apply(x_idxed, linear, edge_types, preproccessed)
+    new_idx = torch.arange(0, num_edge, device=x_idxed.device)
+    return AggrDirectedOP.apply(out, ptr, new_idx, num_center)
+
+
+class MySageConv(torch.nn.Module):
+
+    def __init__(self, in_channels, hidden_channels, root_weight=True, bias=True):
+        super().__init__()
+        self.in_channels = in_channels
+        self.hidden_channels = hidden_channels
+        self.root_weight = root_weight
+        self.lin_l = torch.nn.Linear(in_channels, hidden_channels, bias=bias)
+        if root_weight:
+            self.lin_r = torch.nn.Linear(in_channels, hidden_channels, bias=False)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.lin_l.reset_parameters()
+        if self.root_weight:
+            self.lin_r.reset_parameters()
+
+    def forward(self, x, ptr, idx, num_node):
+        if self.in_channels > self.hidden_channels:
+            out = sage_mean_forward(self.lin_l(x), ptr, idx, num_node)
+        else:
+            out = self.lin_l(sage_mean_forward(x, ptr, idx, num_node))
+        if self.root_weight:
+            out = out + self.lin_r(x[:num_node] if num_node != 0 else x)
+        return out
+
+
+class MyGINConv(torch.nn.Module):
+
+    def __init__(self, in_channels, hidden_channels):
+        super().__init__()
+        self.in_channels = in_channels
+        self.hidden_channels = hidden_channels
+        self.nn = torch.nn.Linear(in_channels, hidden_channels, bias=False)
+        self.init_eps = 0.2
+        self.eps = torch.nn.Parameter(torch.Tensor([self.init_eps]))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.nn.reset_parameters()
+        self.eps.data.fill_(self.init_eps)
+
+    def forward(self, x, ptr, idx, num_node):
+        out = sage_mean_forward(x, ptr, idx, num_node)
+        return self.nn(out + (1 + self.eps) * x[:num_node])
+
+
+class MyRGCNConv(torch.nn.Module):
+
+    def __init__(self, in_channels, hidden_channels, num_rel):
+        super().__init__()
+        assert num_rel > 0
+        self.in_channels = in_channels
+        self.hidden_channels = hidden_channels
+        self.num_rel = num_rel
+        self.linear = torch.nn.Parameter(torch.randn(num_rel, in_channels, hidden_channels))
+        self.register_parameter("rel_weight", self.linear)
+        self.single_linear = torch.nn.Linear(in_channels, hidden_channels)
+        self.reset_parameters()
+        self.preprocessed = []
+
+    def reset_parameters(self):
+        glorot(self.linear)
+        self.single_linear.reset_parameters()
+
+    def forward(self, x, ptr, idx, edge_types, num_node):
+        if idx.shape[0] > 1e8:
+            return RGCNOP.apply(x, self.linear, ptr, idx, edge_types, num_node)
+        if len(self.preprocessed) == 0:
+            self.preprocessed = TypedLinearE2EOP.preprocess(self.linear, edge_types)
+        out = run_rgcn4(x, ptr, idx, edge_types, self.linear, num_node, num_edge=edge_types.shape[0],
+                        preproccessed=self.preprocessed)
+        deg = ptr[1:] - ptr[:-1]
+        return out / deg.unsqueeze(-1)[:out.shape[0]]
+
+
+class MyGATConv(torch.nn.Module):
+
+    def __init__(self, in_channels, out_channels, heads=1, concat=False, negative_slope=0.2,
+                 dropout=0.0, bias=True, layer=-1):
+        super().__init__()
+        assert heads > 0
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.heads = heads
+        self.concat = concat
+        self.negative_slope = negative_slope
+        self.dropout = dropout
+        self.layer = layer
+        self.lin_src = Parameter(torch.Tensor(heads * out_channels, in_channels))
+        self.att_src = Parameter(torch.Tensor(1, heads, out_channels))
+        self.att_dst = Parameter(torch.Tensor(1, heads, out_channels))
+        if bias:
+            self.bias = Parameter(torch.Tensor(heads * out_channels if concat else out_channels))
+        else:
+            self.bias = None
+        self.edge_softmax_schedule = "fused"
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        glorot(self.lin_src)
+        glorot(self.att_src)
+        glorot(self.att_dst)
+        if self.bias is not None:
+            self.bias.data.fill_(0)
+
+    def edge_softmax_fused(self, ptr, idx, att_src, att_dst, num_edge, relu_l):
+        return edge_attention(ptr=ptr, idx=idx, att_src=att_src, att_dst=att_dst, num_edge=num_edge,
+                              relu_l=relu_l)
+
+    def edge_softmax_opwise(self, ptr, idx, att_src, att_dst, num_edge, relu_l):
+        """Op-by-op softmax over each destination's edges (upstream :437-448, there with
+        torch_scatter's segment_csr / gather_csr)."""
+        n = ptr.shape[0] - 1
+        seg = torch.repeat_interleave(torch.arange(n, device=ptr.device), ptr[1:] - ptr[:-1])[:num_edge]
+        alpha = F.leaky_relu(att_src.index_select(0, idx[:num_edge]) + att_dst[seg], relu_l)
+        segh = seg.unsqueeze(1).expand(-1, alpha.shape[1])
+        with torch.no_grad():
+            amax = torch.full((n, alpha.shape[1]), -float("inf"), dtype=alpha.dtype, device=alpha.device)
+            amax = amax.scatter_reduce(0, segh, alpha, "amax", include_self=True)[seg]
+        alpha = torch.exp(alpha - amax)
+        total = torch.zeros((n, alpha.shape[1]), dtype=alpha.dtype, device=alpha.device)
+        total = total.index_add(0, seg, alpha) + 1e-16
+        return alpha / total[seg]
+
+    def edge_softmax(self, ptr, idx, att_src, att_dst, num_edge, relu_l):
+        if self.edge_softmax_schedule == "fused":
+            return self.edge_softmax_fused(ptr, idx, att_src, att_dst, num_edge, relu_l)
+        return self.edge_softmax_opwise(ptr, idx, att_src, att_dst, num_edge, relu_l)
+
+    def forward_many(self, x, ptr, idx, num_dst, num_src, num_edge):
+        H, C = self.heads, self.out_channels
+        assert x.dim() == 2
+        x = TimerOP.apply(x, "linear1", True)
+        x_src = x_dst = F.linear(x[:num_src], self.lin_src).view(-1, H, C)
+        x_src = TimerOP.apply(x_src, "linear1", False)
+        x_src = TimerOP.apply(x_src, "sum1", True)
+        alpha_src = (x_src * self.att_src).sum(dim=-1).view(-1, H)
+        alpha_dst = (x_dst[:num_dst] * self.att_dst).sum(dim=-1).view(-1, H)
+        alpha_dst = TimerOP.apply(alpha_dst, "sum1", False)
+        alpha_dst = TimerOP.apply(alpha_dst, "softmax1", True)
+        edge_value = self.edge_softmax(ptr=ptr, idx=idx, att_src=alpha_src, att_dst=alpha_dst,
+                                       num_edge=num_edge, relu_l=self.negative_slope)
+        edge_value = TimerOP.apply(edge_value, "softmax1", False)
+        edge_value = TimerOP.apply(edge_value, "aggregation", True)
+        if self.heads == 1:
+            out = sage_sum_forward_edge_value(x_src, ptr, idx, edge_value.squeeze(), num_dst)
+        else:
+            out = SpMMValOP.apply(x_src, ptr, idx, edge_value, num_dst)
+        out = TimerOP.apply(out, "aggregation", False)
+        if self.concat:
+            out = out.view(-1, H * C)
+        elif out.shape[1] == self.heads:
+            out = out.mean(dim=1)
+        return out + self.bias if self.bias is not None else out
+
+    def forward_1(self, x, ptr, idx, num_dst, num_src, num_edge):
+        w = self.lin_src.T.view(-1, self.heads, self.out_channels)
+        x = TimerOP.apply(x, "einsum1", True)
+        alpha_src = torch.einsum("mn,nho,ho->mh", x, w, self.att_src.squeeze(0)).view(-1, self.heads)
+        alpha_dst = torch.einsum("mn,nho,ho->mh", x[:num_dst], w, self.att_dst.squeeze(0)).view(-1, self.heads)
+        alpha_dst = TimerOP.apply(alpha_dst, "einsum1", False)
+        alpha_dst = TimerOP.apply(alpha_dst, "softmax1", True)
+        edge_value = self.edge_softmax(ptr=ptr, idx=idx, att_src=alpha_src, att_dst=alpha_dst,
+                                       num_edge=num_edge, relu_l=self.negative_slope)
+        edge_value = TimerOP.apply(edge_value, "softmax1", False)
+        if self.out_channels < self.in_channels:
+            x = TimerOP.apply(x, "mm1", True)
+            t = torch.mm(x, self.lin_src.T).view(-1, self.heads, self.out_channels)
+            t = TimerOP.apply(t, "mm1", False)
+            t = TimerOP.apply(t, "aggregation", True)
+            x = sage_sum_forward_edge_value(t, ptr, idx, edge_value, num_dst).squeeze()
+            x = TimerOP.apply(x, "aggregation", False)
+        else:
+            x = TimerOP.apply(x, "aggregation", True)
+            x = sage_sum_forward_edge_value(x, ptr, idx, edge_value.squeeze(), num_dst)
+            x = TimerOP.apply(x, "aggregation", False)
+            x = TimerOP.apply(x, "mm1", True)
+            x = torch.mm(x, self.lin_src.T)
+            x = TimerOP.apply(x, "mm1", False)
+        return x + self.bias if self.bias is not None else x
+
+    def forward(self, x, ptr, idx, num_dst, num_src, num_edge):
+        ptr = ptr[:num_dst + 1]
+        idx = idx[:num_edge]
+        if self.heads == 1:
+            return self.forward_1(x, ptr, idx, num_dst, num_src, num_edge)
+        return self.forward_many(x, ptr, idx, num_dst, num_src, num_edge)
+
+
+class MyGCNConv(torch.nn.Module):
+
+    def __init__(self, in_channels, out_channels, normalize=False, bias=True):
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.normalize = normalize
+        self.lin = torch.nn.Linear(in_channels, out_channels, bias=False)
+        self.bias = torch.nn.Parameter(torch.Tensor(out_channels)) if bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        glorot(self.lin.weight)
+        if self.bias is not None:
+            self.bias.data.fill_(0)
+
+    def gcn_norm(self, ptr, idx):
+        """1 / in-degree per edge, 0 where the degree is 0 (upstream :587-596)."""
+        deg = ptr[1:] - ptr[:-1]
+        edge_value = deg.repeat_interleave(deg).float().pow(-1)
+        edge_value.masked_fill_(edge_value == float("inf"), 0.0)
+        return edge_value
+
+    def forward(self, x, ptr, idx, num_node):
+        x = TimerOP.apply(x, "linear", True)
+        mm_before = self.in_channels > self.out_channels
+        out = self.lin(x) if mm_before else x
+        out = TimerOP.apply(out, "linear", False)
+        if self.normalize:
+            out = TimerOP.apply(out, "aggregation", True)
+            TimerOP.apply(out, "gcn norm", True)
+            edge_value = self.gcn_norm(ptr, idx)
+            TimerOP.apply(edge_value, "gcn norm", False)
+            out = sage_sum_forward_edge_value(out, ptr, idx, edge_value, num_node)
+            out = TimerOP.apply(out, "aggregation", False)
+        else:
+            out = AggrOP.apply(out, ptr, idx, num_node)
+        if not mm_before:
+            out = self.lin(out)
+        return out + self.bias if self.bias is not None else out

@@ -240,3 +240,8 @@ from ._rel import (aggr_rel, selective_aggr, selective_aggr_bwd, target_aggr,  #
 from ._typed import (aggr_rel_direct, aggr_rgcn_direct_func, pad_rel, pad_rel_idx,  # noqa: E402,F401
                      seastar_backward, seastar_forward, typed_linear, typed_linear_s2d,
                      typed_linear_s2e)
+from ._schedule import (COMPUTEOP, REDUCEOP, GSpMM_u, GSpMM_u_e, gen_edge_type_mag240m,  # noqa: E402,F401
+                        rel_schedule, topo_sort)
+
+SUM, MAX, MIN, MEAN = REDUCEOP.SUM, REDUCEOP.MAX, REDUCEOP.MIN, REDUCEOP.MEAN
+ADD, MUL, DIV, SUB = COMPUTEOP.ADD, COMPUTEOP.MUL, COMPUTEOP.DIV, COMPUTEOP.SUB

@@ -1,0 +1,112 @@
+"""Host-side scheduling helpers of the reference backend (binding.cpp:27,31-33,
+106-119): rel_schedule, gen_edge_type_mag240m, topo_sort, and the dgSPARSE-style
+GSpMM entry points, written as vectorised tensor index arithmetic."""
+import enum
+
+import torch
+
+from . import _ops
+
+
+def _rows_of_edges(ptr, n):
+    return torch.repeat_interleave(torch.arange(n, device=ptr.device), ptr[1:n + 1] - ptr[:n])
+
+
+def rel_schedule(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel):
+    """Per-relation sub-CSRs (src/cpp/src/schedule.cu:5-63).  For every relation r the
+    rows that have at least one edge of type r: ptr_r, idx_r (edge order kept) and
+    target_r (original row ids); then a [num_rel, L] table, L = len(num_node_in_layer)-1,
+    whose entry [r, l] is the number of kept rows among the first num_node_in_layer[l]
+    rows.  Returns the 3*num_rel + 1 tensors in that order, on the inputs' device
+    (upstream works on CPU tensors)."""
+    n = csr_ptr.shape[0] - 1
+    num_rel = int(num_rel)
+    rows = _rows_of_edges(csr_ptr, n)
+    e = rows.shape[0]
+    idx = csr_idx[:e]
+    rel = rel[:e]
+    layers = [int(v) for v in num_node_in_layer.tolist()]
+    num_layer = len(layers) - 1
+    table = torch.zeros((num_rel, max(num_layer, 0)), dtype=torch.int64, device=csr_ptr.device)
+    out = []
+    for r in range(num_rel):
+        m = rel == r
+        cnt = torch.bincount(rows[m], minlength=n)
+        keep = cnt > 0
+        target = torch.nonzero(keep).flatten()
+        sub_ptr = torch.cat([cnt.new_zeros(1), torch.cumsum(cnt[keep], 0)])
+        out += [sub_ptr, idx[m], target]
+        kept_before = torch.cumsum(keep.to(torch.int64), 0)
+        # upstream walks rows in order and records layer l when it reaches row
+        # num_node_in_layer[l]-1; a boundary that lies behind the walk is never met
+        pos = -1
+        for l in range(num_layer):
+            i = layers[l] - 1
+            if i <= pos or i >= n:
+                break
+            table[r, l] = kept_before[i]
+            pos = i
+    out.append(table)
+    return out
+
+
+_PAPER = 121751666
+_PAPER_AUTHOR = 244134778
+
+
+def gen_edge_type_mag240m(ptr, idx, sub_to_full):
+    """Edge types of a MAG240M sub-graph from global id ranges
+    (src/cpp/src/aggr.cu:516-566): paper<-paper 0, paper<-author 1, author<-paper 2,
+    author<-institute 3, institute<-author 4."""
+    n = ptr.shape[0] - 1
+    rows = _rows_of_edges(ptr, n)
+    e = rows.shape[0]
+    center = sub_to_full[rows]
+    nbr = sub_to_full[idx[:e]]
+
+    def kind(v):
+        return (v >= _PAPER).to(torch.int64) + (v >= _PAPER_AUTHOR).to(torch.int64)
+    ck, nk = kind(center), kind(nbr)
+    table = torch.tensor([[0, 1, -1], [2, -1, 3], [-1, 4, -1]], device=ptr.device)
+    et = table[ck, nk]
+    if bool((et < 0).any()):
+        raise ValueError("edge between node kinds that MAG240M does not connect")
+    out = torch.zeros_like(idx)
+    out[:e] = et
+    return out
+
+
+def topo_sort(csr_ptr, csr_idx, degree):
+    raise NotImplementedError("topo_sort (src/cpp/src/schedule.cu:72-128) is not used by any "
+                              "aggregation path and is not provided")
+
+
+class REDUCEOP(enum.IntEnum):
+    SUM = 0
+    MAX = 1
+    MIN = 2
+    MEAN = 3
+
+
+class COMPUTEOP(enum.IntEnum):
+    ADD = 0
+    MUL = 1
+    DIV = 2
+    SUB = 3
+
+
+def GSpMM_u(A_rowptr, A_colind, B, op):
+    """int32-CSR SpMM without edge values (binding.cpp:97-104); SUM and MEAN."""
+    op = REDUCEOP(int(op))
+    if op not in (REDUCEOP.SUM, REDUCEOP.MEAN):
+        raise NotImplementedError("GSpMM_u supports SUM and MEAN")
+    if A_rowptr.dtype != torch.int32 or A_colind.dtype != torch.int32:
+        raise ValueError("GSpMM_u takes int32 rowptr/colind")
+    return _ops.spmm(A_rowptr, A_colind, B, A_rowptr.shape[0] - 1, mean=(op == REDUCEOP.MEAN))
+
+
+def GSpMM_u_e(A_rowptr, A_colind, A_csrVal, B, re_op, comp_op):
+    """int32-CSR SpMM with edge values (binding.cpp:86-95); SUM of MUL."""
+    if REDUCEOP(int(re_op)) != REDUCEOP.SUM or COMPUTEOP(int(comp_op)) != COMPUTEOP.MUL:
+        raise NotImplementedError("GSpMM_u_e supports REDUCEOP.SUM with COMPUTEOP.MUL")
+    return _ops.spmm(A_rowptr.long(), A_colind.long(), B, A_rowptr.shape[0] - 1, val=A_csrVal)

@@ -1,0 +1,342 @@
+"""The cxgnncomp Python surface (autograd ops, typed_linear family, conv layers,
+alternative-implementation names) on the GPU against CPU restatements."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import announce, assert_close
+from oracle import pyref
+from test_spmm_gpu import ATOL, RTOL, _graph, _scale
+
+pytestmark = pytest.mark.gpu
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+def _hetero(n=2000, e=30000, R=5, seed=6):
+    from cxgnncomp import synthetic as S
+    ptr, idx, etype, _ = S.hetero_graph(n, e, num_rel=R, seed=seed)
+    return ptr, idx, etype
+
+
+def _rgcn_reference(x, w, ptr, idx, rel, n, g):
+    """Forward and gradients of sum_e x[idx[e]] @ W[rel[e]] by autograd through the
+    reference's pure-torch relation-sorted form, in float64 on the CPU."""
+    x64 = x.double().requires_grad_(True)
+    w64 = w.double().requires_grad_(True)
+    out = pyref.typed_linear_s2d_sort(x64, w64, ptr, idx, rel, n)
+    out.backward(g.double())
+    return out.detach().numpy(), x64.grad.numpy(), w64.grad.numpy()
+
+
+@pytest.mark.parametrize("opname", ["AggrOP", "AggrDirectedOP"])
+def test_aggr_ops_true_transposed_backward(opname):
+    import cxgnncomp
+    from cxgnncomp import graph_conv
+    from cxgnncomp import synthetic as S
+    op = getattr(graph_conv, opname)
+    # bipartite, non-symmetric: 900 destinations, 1500 sources
+    ptr, idx, nn, ne = S.sampled_batch(num_seeds=900, fanouts=(6,), id_space=1400, seed=3)
+    n_dst, n_src = nn[0], nn[1]
+    torch.manual_seed(15)
+    x = (torch.randn(n_src, 64) / 3).cuda().requires_grad_(True)
+    g = torch.randn(n_dst, 64) / 3
+    announce("%s fwd+bwd" % opname)
+    out = op.apply(x, ptr.cuda(), idx.cuda(), torch.tensor(n_dst))
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    assert_close(_np(out), oracle.spmm(ptr.numpy(), idx.numpy(), _np(x), n_dst), RTOL, ATOL, "fwd")
+    assert_close(_np(x.grad), oracle.spmm_bwd(ptr.numpy(), idx.numpy(), g.numpy(), n_dst, n_src), RTOL, ATOL, "bwd")
+    assert "run_spmm_configurable_lazy" in cxgnncomp.global_tuner.cache
+
+
+def test_spmm_val_op():
+    from cxgnncomp.graph_kernel import SpMMValOP
+    ptr, idx = _graph("powerlaw")
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    H, C = 4, 64
+    torch.manual_seed(16)
+    sc = _scale(ptr)
+    x = (torch.randn(n, H, C) * sc).cuda().requires_grad_(True)
+    val = torch.rand(E, H).cuda().requires_grad_(True)
+    g = torch.randn(n, H, C) * sc
+    announce("SpMMValOP H=4 C=64")
+    out = SpMMValOP.apply(x, ptr.cuda(), idx.cuda(), val, n)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    p, i = ptr.numpy(), idx.numpy()
+    assert_close(_np(out), oracle.spmm(p, i, _np(x), n, val=_np(val)), RTOL, ATOL, "fwd")
+    assert_close(_np(x.grad), oracle.spmm_bwd(p, i, g.numpy(), n, n, val=_np(val)), RTOL, ATOL, "grad x")
+    assert_close(_np(val.grad), oracle.edge_grad(p, i, _np(x), g.numpy(), n), RTOL, ATOL, "grad val (per head)")
+
+
+def test_typed_matmul_index_modes():
+    import cxgnncomp
+    torch.manual_seed(17)
+    M, K, N, R = 700, 64, 48, 4
+    a = torch.randn(M, K) / 8
+    b = torch.randn(R, K, N)
+    rel = torch.sort(torch.randint(0, R, (M,)))[0]
+    src = torch.randint(0, M, (M,))
+    dst = torch.randperm(M)
+    ac, bc, rc = a.cuda(), b.cuda(), rel.cuda()
+    announce("typed_matmul no index")
+    c = cxgnncomp.typed_matmul(ac, bc, rc)
+    ref = pyref.typed_matmul(a.double(), b.double(), rel).numpy()
+    assert_close(_np(c), ref, RTOL, ATOL, "no index")
+    announce("typed_matmul seq_output")
+    c = cxgnncomp.typed_matmul(ac, bc, rc, M, src.cuda(), seq_output=True)
+    ref = pyref.typed_matmul(a.double(), b.double(), rel, src).numpy()
+    assert_close(_np(c), ref, RTOL, ATOL, "seq output")
+    announce("typed_matmul double index")
+    c = cxgnncomp.typed_matmul(ac, bc, rc, M, src.cuda(), dst.cuda())
+    assert_close(_np(c), pyref.typed_matmul(a.double(), b.double(), rel, src, dst).numpy(), RTOL, ATOL, "double")
+    announce("typed_matmul single index (permutation with padding)")
+    perm = torch.randperm(M)
+    padded = torch.cat([perm, torch.full((9,), -1)])
+    relp = torch.cat([rel, torch.full((9,), R)])
+    c = cxgnncomp.typed_matmul(ac, bc, relp.cuda(), M, padded.cuda())
+    want = torch.zeros(M, N, dtype=torch.float64)
+    want[perm] = torch.bmm(a[perm].double().unsqueeze(1), b[rel].double()).squeeze(1)
+    assert_close(_np(c), want.numpy(), RTOL, ATOL, "single index")
+    announce("typed_matmul unsorted rel")
+    rel_u = torch.randint(0, R, (M,))
+    c = cxgnncomp.typed_matmul(ac, bc, rel_u.cuda())
+    assert_close(_np(c), pyref.typed_matmul(a.double(), b.double(), rel_u).numpy(), RTOL, ATOL, "unsorted")
+
+
+def test_typed_linear_e2e_and_s2e_ops():
+    import cxgnncomp
+    torch.manual_seed(18)
+    E, K, N, R, n_src = 3000, 64, 32, 5, 400
+    types = torch.randint(0, R - 1, (E,))                 # highest relation absent
+    w = torch.randn(R, K, N) / 4
+    x = torch.randn(E, K) / 8
+    g = torch.randn(E, N)
+    pre = cxgnncomp.TypedLinearE2EOP.preprocess(w.cuda(), types.cuda(), 32)
+    sorted_types, num_item, indices, count = pre
+    assert num_item == E and count.device.type == "cpu" and count.tolist() == torch.bincount(types, minlength=R).tolist()
+    st, _, ind, _ = pyref.e2e_preprocess(R, types.numpy(), 32)
+    assert np.array_equal(_np(sorted_types), st) and np.array_equal(_np(indices), ind)
+    xg = x.cuda().requires_grad_(True)
+    wg = w.cuda().requires_grad_(True)
+    announce("TypedLinearE2EOP fwd+bwd")
+    out = cxgnncomp.TypedLinearE2EOP.apply(xg, wg, types.cuda(), pre)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    ref = torch.bmm(x64.unsqueeze(1), w64[types]).squeeze(1)
+    ref.backward(g.double())
+    assert out.shape == (E, N)
+    assert_close(_np(out), ref.detach().numpy(), RTOL, ATOL, "e2e fwd")
+    assert_close(_np(xg.grad), x64.grad.numpy(), RTOL, 2 * ATOL, "e2e grad x")
+    sc = float(w64.grad.abs().max())
+    assert_close(_np(wg.grad) / sc, w64.grad.numpy() / sc, RTOL, ATOL, "e2e grad w")
+    # without a preprocessed list the op prepares itself
+    out2 = cxgnncomp.TypedLinearE2EOP.apply(x.cuda(), w.cuda(), types.cuda())
+    assert torch.equal(out2, out.detach())
+    # source -> edge
+    xs = torch.randn(n_src, K) / 8
+    src = torch.randint(0, n_src, (E,))
+    xsg = xs.cuda().requires_grad_(True)
+    wg2 = w.cuda().requires_grad_(True)
+    announce("TypedLinearS2EOP fwd+bwd")
+    out = cxgnncomp.TypedLinearS2EOP.apply(xsg, wg2, types.cuda(), src.cuda(), [], 32)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    xs64, w64 = xs.double().requires_grad_(True), w.double().requires_grad_(True)
+    ref = torch.bmm(xs64[src].unsqueeze(1), w64[types]).squeeze(1)
+    ref.backward(g.double())
+    assert_close(_np(out), ref.detach().numpy(), RTOL, ATOL, "s2e fwd")
+    sx = float(xs64.grad.abs().max())
+    assert_close(_np(xsg.grad) / sx, xs64.grad.numpy() / sx, RTOL, ATOL, "s2e grad x")
+    assert_close(_np(wg2.grad) / sc, w64.grad.numpy() / sc, RTOL, 2 * ATOL, "s2e grad w")
+
+
+@pytest.mark.parametrize("opname", ["RGCNOP", "RGCNOP2", "RGCNOP3", "SeastarRGCNOP",
+                                    "TypedLinearS2DMMAggrOP", "TypedLinearS2DAggrMMOP"])
+def test_rgcn_op_variants(opname):
+    import cxgnncomp
+    from cxgnncomp import graph_conv
+    cxgnncomp.set_timers()
+    ptr, idx, etype = _hetero()
+    n = ptr.shape[0] - 1
+    K, N, R = 64, 32, 5
+    torch.manual_seed(19)
+    x = torch.randn(n, K) / 16
+    w = torch.randn(R, K, N) / 2
+    g = torch.randn(n, N) / 4
+    want, want_gx, want_gw = _rgcn_reference(x, w, ptr, idx, etype, n, g)
+    op = getattr(graph_conv, opname, None) or getattr(cxgnncomp, opname)
+    xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    announce("%s fwd+bwd" % opname)
+    out = op.apply(xg, wg, ptr.cuda(), idx.cuda(), etype.cuda(), n)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    assert_close(_np(out), want, RTOL, 2 * ATOL, opname + " fwd")
+    assert_close(_np(xg.grad), want_gx, RTOL, 2 * ATOL, opname + " grad x")
+    sc = float(np.abs(want_gw).max())
+    assert_close(_np(wg.grad) / sc, want_gw / sc, RTOL, 2 * ATOL, opname + " grad w")
+
+
+def test_rgcn_named_variants_and_prune_path():
+    import cxgnncomp
+    import cxgnncomp_backend as B
+    ptr, idx, etype = _hetero()
+    n = ptr.shape[0] - 1
+    K, N, R = 64, 32, 5
+    torch.manual_seed(20)
+    x = torch.randn(n, K) / 16
+    w = torch.randn(R, K, N) / 2
+    want = oracle.rgcn_fused(x.numpy(), ptr.numpy(), idx.numpy(), w.numpy(), etype.numpy(), n)
+    pc, ic, ec, xc, wc = ptr.cuda(), idx.cuda(), etype.cuda(), x.cuda(), w.cuda()
+    for name in ("rgcn_triton", "rgcn_triton_opt", "rgcn_scatter"):
+        announce(name)
+        assert_close(_np(getattr(cxgnncomp, name)(xc, pc, ic, ec, wc, n)), want, RTOL, 2 * ATOL, name)
+    for name in ("rgcn_full_mm", "rgcn_full_mm2"):
+        announce(name)
+        assert_close(_np(getattr(cxgnncomp, name)(xc, pc, ic, ec, wc, n, R)), want, RTOL, 2 * ATOL, name)
+    announce("rel_schedule on GPU tensors + rgcn_prune_mm")
+    meta = B.rel_schedule(pc, ic, ec.int(), torch.tensor([n, n]), R)
+    want_meta = oracle.rel_schedule(ptr.numpy(), idx.numpy(), etype.numpy(), [n, n], R)
+    for gmeta, wmeta in zip(meta, want_meta):
+        assert np.array_equal(_np(gmeta), wmeta)
+    assert_close(_np(cxgnncomp.rgcn_prune_mm(xc, wc, meta, n, R)), want, RTOL, 2 * ATOL, "prune mm")
+    announce("rgcn_just_aggr / rgcn_just_aggr_prune")
+    agg = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n)
+    wk = torch.zeros(R, K, K)
+    assert_close(_np(cxgnncomp.rgcn_just_aggr(xc, pc, ic, ec, wk.cuda(), n, R)), agg, RTOL, ATOL, "just aggr")
+    assert_close(_np(cxgnncomp.rgcn_just_aggr_prune(xc, meta, n, R)), agg, RTOL, ATOL, "just aggr prune")
+    announce("TypedLinearS2DPushOP")
+    dst = torch.repeat_interleave(torch.arange(n), ptr[1:] - ptr[:-1])
+    got = cxgnncomp.TypedLinearS2DPushOP(xc, wc, ec, ic, dst.cuda(), R, n, idx.shape[0])
+    assert_close(_np(got), want, RTOL, 2 * ATOL, "push op")
+
+
+def test_alternative_spmm_sddmm_names_and_prof():
+    import cxgnncomp
+    ptr, idx = _graph("uniform")
+    n = ptr.shape[0] - 1
+    torch.manual_seed(21)
+    x = torch.randn(n, 64) / 4
+    val = torch.rand(idx.shape[0])
+    pc, ic, xc = ptr.cuda(), idx.cuda(), x.cuda()
+    announce("spmm_triton / spmm_torch / spmm_mm_triton")
+    a = cxgnncomp.spmm_triton(xc, pc, ic, n)
+    b = cxgnncomp.spmm_torch(xc, pc, ic, n)
+    assert_close(_np(a), _np(b), 1e-4, 1e-5, "hip vs torch.sparse.mm on the GPU")
+    a = cxgnncomp.spmm_triton(xc, pc, ic, n, val.cuda())
+    assert_close(_np(a), oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n, val=val.numpy()), RTOL, ATOL, "val")
+    w = torch.randn(16, 64) / 8
+    got = cxgnncomp.spmm_mm_triton(xc, pc, ic, w.cuda(), n)
+    want = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n).astype(np.float64) @ w.numpy().T
+    assert_close(_np(got), want, 1e-4, 1e-4, "spmm+mm")
+    announce("sddmm_dense")
+    dst = torch.repeat_interleave(torch.arange(n), ptr[1:] - ptr[:-1])
+    srcf = torch.randn(n, 64, 4) / 8                       # [num_src, feat, head]
+    got = cxgnncomp.sddmm_dense(xc, srcf.cuda(), dst.cuda(), ic, idx.shape[0])
+    want = np.einsum("ek,ekh->eh", x.numpy()[dst.numpy()].astype(np.float64), srcf.numpy()[idx.numpy()])
+    assert_close(_np(got), want, RTOL, ATOL, "sddmm_dense")
+    res = cxgnncomp.prof("spmm", "hip", lambda: cxgnncomp.spmm_triton(xc, pc, ic, n), display=False)
+    assert len(res) == 3 and res[1] <= res[0] <= res[2] and cxgnncomp.global_res[-1] == res
+
+
+def test_conv_layers_forward_backward():
+    """Layers against the same layer evaluated on the CPU with dense torch ops."""
+    import cxgnncomp
+    cxgnncomp.set_timers()
+    ptr, idx = _graph("powerlaw")
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    p, i = ptr.numpy(), idx.numpy()
+    dst = torch.repeat_interleave(torch.arange(n), ptr[1:] - ptr[:-1])
+    deg = (ptr[1:] - ptr[:-1]).double()
+    torch.manual_seed(22)
+    x = torch.randn(n, 32) / 20
+    pc, ic = ptr.cuda(), idx.cuda()
+
+    def agg(t, weight=None):
+        msg = t[idx] if weight is None else t[idx] * weight.reshape(E, *([1] * (t.dim() - 1)))
+        return torch.zeros((n,) + tuple(t.shape[1:]), dtype=t.dtype).index_add_(0, dst, msg)
+
+    def check(layer, ref_fn, args, name):
+        xg = x.cuda().requires_grad_(True)
+        layer = layer.cuda()
+        announce(name)
+        out = layer(xg, *args)
+        out.sum().backward()
+        torch.cuda.synchronize()
+        x64 = x.double().requires_grad_(True)
+        params = {k: v.detach().double().cpu() for k, v in layer.named_parameters()}
+        ref = ref_fn(x64, params)
+        ref.sum().backward()
+        assert_close(_np(out), ref.detach().numpy(), 2e-4, 2e-5, name + " fwd")
+        sc = max(1.0, float(x64.grad.abs().max()))
+        assert_close(_np(xg.grad) / sc, x64.grad.numpy() / sc, 2e-4, 2e-5, name + " grad x")
+
+    inv = torch.where(deg > 0, 1.0 / deg.clamp(min=1), torch.zeros_like(deg))
+    check(cxgnncomp.MyGCNConv(32, 48), lambda t, P: agg(t) @ P["lin.weight"].T + P["bias"], (pc, ic, n), "GCN sum")
+    check(cxgnncomp.MyGCNConv(32, 16, normalize=True),
+          lambda t, P: agg(t @ P["lin.weight"].T, inv[dst]) + P["bias"], (pc, ic, n), "GCN 1/deg, linear first")
+    check(cxgnncomp.MySageConv(32, 48),
+          lambda t, P: (agg(t) * inv[:, None]) @ P["lin_l.weight"].T + P["lin_l.bias"] + t @ P["lin_r.weight"].T,
+          (pc, ic, n), "SAGE mean")
+    check(cxgnncomp.MyGINConv(32, 24),
+          lambda t, P: (agg(t) * inv[:, None] + (1 + P["eps"]) * t) @ P["nn.weight"].T, (pc, ic, n), "GIN")
+
+    def gat_ref(H, C, concat):
+        def f(t, P):
+            xs = (t @ P["lin_src"].T).view(-1, H, C)
+            a_s = (xs * P["att_src"]).sum(-1)
+            a_d = (xs * P["att_dst"]).sum(-1)
+            ev = pyref.edge_softmax_opwise(ptr, idx, a_s, a_d, E, 0.2)
+            out = agg(xs, None) * 0
+            out = torch.zeros(n, H, C, dtype=t.dtype).index_add_(0, dst, xs[idx] * ev.unsqueeze(-1))
+            out = out.view(-1, H * C) if concat else out.mean(dim=1)
+            return out + P["bias"]
+        return f
+    check(cxgnncomp.MyGATConv(32, 16, heads=4, concat=True), gat_ref(4, 16, True), (pc, ic, n, n, E), "GAT 4 heads")
+    check(cxgnncomp.MyGATConv(32, 16, heads=2, concat=False), gat_ref(2, 16, False), (pc, ic, n, n, E), "GAT mean heads")
+    check(cxgnncomp.MyGATConv(32, 16, heads=1), gat_ref(1, 16, False), (pc, ic, n, n, E), "GAT 1 head, out<in")
+    check(cxgnncomp.MyGATConv(32, 64, heads=1), gat_ref(1, 64, False), (pc, ic, n, n, E), "GAT 1 head, out>in")
+
+
+def test_rgcn_conv_layer():
+    import cxgnncomp
+    cxgnncomp.set_timers()
+    ptr, idx, etype = _hetero(n=1500, e=20000, R=4, seed=8)
+    n = ptr.shape[0] - 1
+    torch.manual_seed(23)
+    x = torch.randn(n, 32) / 8
+    layer = cxgnncomp.MyRGCNConv(32, 32, 4).cuda()
+    xg = x.cuda().requires_grad_(True)
+    announce("MyRGCNConv")
+    out = layer(xg, ptr.cuda(), idx.cuda(), etype.cuda(), n)
+    out.sum().backward()
+    torch.cuda.synchronize()
+    w = layer.linear.detach().cpu()
+    g = torch.ones(n, 32)
+    deg = (ptr[1:] - ptr[:-1]).double().unsqueeze(-1)
+    x64 = x.double().requires_grad_(True)
+    ref = pyref.typed_linear_s2d_sort(x64, w.double(), ptr, idx, etype, n) / deg
+    ref.backward(g.double())
+    assert_close(_np(out), ref.detach().numpy(), RTOL, 2 * ATOL, "rgcn conv fwd")
+    assert_close(_np(xg.grad), x64.grad.numpy(), RTOL, 2 * ATOL, "rgcn conv grad x")
+    assert len(layer.preprocessed) == 4
+
+
+def test_schedule_helpers_on_gpu_tensors():
+    import cxgnncomp
+    ptr, idx = _graph("powerlaw")
+    want_ptr, want_target = oracle.neighbor_grouping(ptr.numpy(), 32)
+    announce("neighbor_grouping on GPU tensors")
+    gp, gt = cxgnncomp.neighbor_grouping(ptr.cuda(), 32)
+    assert gp.is_cuda and np.array_equal(_np(gp), want_ptr) and np.array_equal(_np(gt), want_target)
+    flag = torch.rand(ptr.shape[0] - 1) < 0.2
+    a = cxgnncomp.remove_from_graph(ptr.cuda(), idx.cuda(), flag.cuda())
+    b = cxgnncomp.remove_from_graph(ptr, idx, flag)
+    assert torch.equal(a[0].cpu(), b[0]) and torch.equal(a[1].cpu(), b[1])
