@@ -1,0 +1,134 @@
+"""The headline configuration at full size (2,449,029 nodes / 61,859,140 edges,
+F=128) and the GAT configuration on the same graph, checked through properties
+that do not need a full CPU recomputation, plus an oracle comparison on sampled
+rows.  Features are scaled by 1/sqrt(max degree) so that hub rows stay O(1) and the
+1e-4 / 1e-5 aggregation tolerance applies."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import announce, assert_close
+
+pytestmark = pytest.mark.gpu
+
+N_NODES, N_PAIRS = 2449029, 30929570
+
+
+@pytest.fixture(scope="module")
+def big():
+    from cxgnncomp import synthetic as S
+    announce("generate headline graph on the GPU")
+    ptr, idx = S.powerlaw_symmetric_graph(N_NODES, N_PAIRS, seed=0, device="cuda")
+    torch.cuda.synchronize()
+    return ptr, idx
+
+
+def _rows_sample(ptr, rng, k=300):
+    deg = (ptr[1:] - ptr[:-1]).cpu().numpy()
+    hubs = np.argsort(deg)[-8:]
+    rest = rng.integers(0, deg.shape[0], k)
+    empty = np.nonzero(deg == 0)[0][:8]
+    return np.unique(np.concatenate([hubs, rest, empty]))
+
+
+def _sub_csr(ptr, idx, rows):
+    """CSR of the selected rows only (CPU numpy), sources unchanged."""
+    p = ptr.cpu().numpy()
+    starts, ends = p[rows], p[rows + 1]
+    sub_ptr = np.concatenate([[0], np.cumsum(ends - starts)])
+    pos = np.concatenate([np.arange(s, e) for s, e in zip(starts, ends)]) if len(rows) else np.zeros(0, np.int64)
+    return sub_ptr, idx[torch.from_numpy(pos).cuda()].cpu().numpy(), pos
+
+
+def test_graph_shape(big):
+    ptr, idx = big
+    assert idx.shape[0] == 61859140 and int(ptr[-1]) == 61859140
+    deg = ptr[1:] - ptr[:-1]
+    assert 14000 < int(deg.max()) < 22000
+    assert torch.equal(torch.bincount(idx, minlength=N_NODES), deg)      # symmetric multiset
+
+
+def test_headline_spmm_properties(big):
+    import cxgnncomp_backend as B
+    ptr, idx = big
+    deg = ptr[1:] - ptr[:-1]
+    sc = 1.0 / float(deg.max()) ** 0.5
+    torch.manual_seed(0)
+    x = torch.randn(N_NODES, 128, device="cuda") * sc
+    z = (0,) * 9
+    announce("fwd F=128 full size")
+    out = B.run_spmm_configurable(ptr, idx, x, N_NODES, *z)
+    announce("bwd (transposed CSR) full size")
+    gx = B.run_spmm_configurable_bwd(ptr, idx, x, x, N_NODES, *z)
+    torch.cuda.synchronize()
+    # 1. A is symmetric as a multiset, so A^T x == A x up to the order of additions
+    assert_close(gx.cpu().numpy(), out.cpu().numpy(), 1e-4, 1e-5, "A^T x == A x on the symmetric graph")
+    # 2. all-ones features give the degree exactly (integers < 2^24 are exact in fp32)
+    ones = torch.ones(N_NODES, 128, device="cuda")
+    d = B.run_spmm_configurable(ptr, idx, ones, N_NODES, *z)
+    assert torch.equal(d[:, 0].long(), deg) and torch.equal(d[:, 127].long(), deg)
+    # 3. run-to-run determinism (no atomics on this path)
+    out2 = B.run_spmm_configurable(ptr, idx, x, N_NODES, *z)
+    assert torch.equal(out, out2)
+    # 4. mean == sum / degree, empty rows stay zero
+    m = B.sage_mean_forward(x, ptr, idx, N_NODES)
+    want = torch.where(deg[:, None] > 0, out / deg.clamp(min=1)[:, None].float(), torch.zeros_like(out))
+    assert_close(m.cpu().numpy(), want.cpu().numpy(), 1e-5, 1e-7, "mean")
+    # 5. oracle on sampled rows (hubs, random rows, empty rows)
+    rng = np.random.default_rng(0)
+    rows = _rows_sample(ptr, rng)
+    sub_ptr, sub_idx, _ = _sub_csr(ptr, idx, rows)
+    ref = oracle.spmm(sub_ptr, sub_idx, x.cpu().numpy(), len(rows))
+    assert_close(out[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, 1e-4, 1e-5, "sampled rows vs oracle")
+    # 6. total mass: sum over rows of A x == sum over nodes of deg * x (checksum of checksums)
+    lhs = out.double().sum(dim=0)
+    rhs = (x.double() * deg[:, None].double()).sum(dim=0)
+    # (2.4M fp32 outputs, each rounded once: the sum carries ~sqrt(N) * 6e-8 * |row| of noise;
+    #  a single dropped or doubled edge moves a column by ~1e-2)
+    assert_close(lhs.cpu().numpy(), rhs.cpu().numpy(), 1e-6, 2e-3, "column checksums")
+
+
+def test_gat_configuration_full_size(big):
+    """4 heads x 64 channels on the 61.9M-edge graph: fused softmax, multi-head
+    weighted SpMM and its edge-value gradient."""
+    import cxgnncomp_backend as B
+    from cxgnncomp.graph_kernel import SpMMValOP
+    ptr, idx = big
+    E = idx.shape[0]
+    deg = ptr[1:] - ptr[:-1]
+    H, C = 4, 64
+    torch.manual_seed(1)
+    att_src = torch.randn(N_NODES, H, device="cuda", requires_grad=True)
+    att_dst = torch.randn(N_NODES, H, device="cuda", requires_grad=True)
+    announce("edge_attention full size")
+    ev = B.edge_attention(ptr=ptr, idx=idx, att_dst=att_dst, att_src=att_src, num_edge=E, relu_l=0.2)
+    torch.cuda.synchronize()
+    # rows of the softmax sum to one
+    sums = B.spmv(ptr, torch.arange(E, device="cuda"), ev.detach()[:, 0].contiguous(), N_NODES)
+    nz = deg > 0
+    assert float((sums[nz] - 1).abs().max()) < 1e-5
+    rng = np.random.default_rng(1)
+    rows = _rows_sample(ptr, rng, 200)
+    sub_ptr, sub_idx, pos = _sub_csr(ptr, idx, rows)
+    ref, mask = oracle.edge_softmax_fwd(sub_ptr, sub_idx, att_dst.detach()[torch.from_numpy(rows).cuda()].cpu().numpy(),
+                                        att_src.detach().cpu().numpy(), len(sub_idx), 0.2)
+    got = ev.detach()[torch.from_numpy(pos).cuda()].cpu().numpy()
+    assert_close(got, ref, 2e-4, 1e-7, "softmax on sampled rows vs oracle")
+    x = (torch.randn(N_NODES, H, C, device="cuda") / 8).requires_grad_(True)
+    announce("SpMMValOP fwd+bwd full size")
+    out = SpMMValOP.apply(x, ptr, idx, ev, N_NODES)
+    g = torch.randn(N_NODES, H, C, device="cuda") / 8
+    out.backward(g)
+    torch.cuda.synchronize()
+    ref_out = oracle.spmm(sub_ptr, sub_idx, x.detach().cpu().numpy(), len(rows), val=got)
+    assert_close(out.detach()[torch.from_numpy(rows).cuda()].cpu().numpy(), ref_out, 1e-4, 1e-5, "weighted spmm rows")
+    # adjoint identity over the whole graph: <A_w x, g> == <x, A_w^T g>
+    lhs = float((out.detach().double() * g.double()).sum())
+    rhs = float((x.detach().double() * x.grad.double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * max(1.0, abs(lhs))
+    assert att_src.grad is not None and att_dst.grad is not None
+    assert torch.isfinite(att_src.grad).all() and torch.isfinite(att_dst.grad).all()
+    # every edge term of the softmax gradient reaches exactly one source and one destination,
+    # and a row whose activations share a sign contributes zero in total to both
+    assert abs(float(att_src.grad.double().sum()) - float(att_dst.grad.double().sum())) < 1e-2
