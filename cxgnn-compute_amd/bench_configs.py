@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Per-operator throughput on the five benchmark configurations (one JSON line per
+measurement).  ``bench.py`` at the repository root reports the headline metric;
+this script is the wider table: every op of the graph-kernel path at the shape it
+has in each configuration, as milliseconds, effective GB/s (algorithmic bytes of
+the gather model / time), GFLOP/s and fraction of the 8 TB/s HBM peak (or of the
+matrix-core peak for the typed GEMM).
+
+Usage: python bench_configs.py [--configs c1,c2,c3,c4,c5] [--iters 10]
+"""
+import argparse
+import json
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+
+import torch  # noqa: E402
+
+HBM = 8000.0          # GB/s
+MFMA_F32 = 157300.0   # GFLOP/s
+MFMA_BF16 = 2500000.0
+
+
+def timeit(fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def report(cfg, op, ms, nbytes=None, flops=None, peak_flops=None, note=""):
+    rec = {"config": cfg, "op": op, "ms": round(ms, 4)}
+    if nbytes:
+        gbs = nbytes / ms / 1e6
+        rec["eff_GBps"] = round(gbs, 1)
+        rec["frac_hbm"] = round(gbs / HBM, 4)
+    if flops:
+        gf = flops / ms / 1e6
+        rec["GFLOPps"] = round(gf, 1)
+        if peak_flops:
+            rec["frac_mfma"] = round(gf / peak_flops, 4)
+    if note:
+        rec["note"] = note
+    print(json.dumps(rec), flush=True)
+
+
+def spmm_bytes(rows, edges, row_floats, val_floats=0):
+    return edges * (4 * row_floats + 8 + 4 * val_floats) + 4 * rows * row_floats + 8 * (rows + 1)
+
+
+def bench_aggregation(cfg, ptr, idx, n_dst, n_src, feat, iters, weighted=True):
+    import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
+    E = int(ptr[n_dst])
+    x = torch.randn(n_src, feat, device="cuda")
+    g = torch.randn(n_dst, feat, device="cuda")
+    gt = _ops.transposed(ptr, idx, n_dst, n_src)
+    z = (0,) * 9
+    report(cfg, "spmm_sum_fwd F=%d" % feat, timeit(lambda: B.run_spmm_configurable(ptr, idx, x, n_dst, *z), iters),
+           spmm_bytes(n_dst, E, feat), E * feat)
+    report(cfg, "spmm_sum_bwd F=%d" % feat,
+           timeit(lambda: B.run_spmm_configurable_bwd(ptr, idx, x, g, n_dst, *z), iters),
+           spmm_bytes(n_src, E, feat), E * feat)
+    report(cfg, "spmm_mean_fwd F=%d" % feat, timeit(lambda: _ops.spmm(ptr, idx, x, n_dst, mean=True), iters),
+           spmm_bytes(n_dst, E, feat), E * feat)
+    if weighted:
+        val = B.edge_value_degree(ptr, n_dst, idx.shape[0])
+        report(cfg, "spmm_weighted_fwd(1/deg) F=%d" % feat,
+               timeit(lambda: _ops.spmm(ptr, idx, x, n_dst, val=val), iters),
+               spmm_bytes(n_dst, E, feat, 1), 2 * E * feat)
+        report(cfg, "spmm_weighted_bwd F=%d" % feat,
+               timeit(lambda: _ops.spmm(gt.ptr_t, gt.idx_t, g, n_src, val=val, val_perm=gt.perm), iters),
+               spmm_bytes(n_src, E, feat, 1) + 8 * E, 2 * E * feat)
+
+
+def c1(iters):
+    from cxgnncomp import synthetic as S
+    ptr, idx = S.uniform_graph(10000, 100000, device="cuda")
+    bench_aggregation("c1", ptr, idx, 10000, 10000, 64, iters)
+
+
+def c2(iters):
+    from cxgnncomp import synthetic as S
+    ptr, idx = S.powerlaw_directed_symmetrised(169343, 1166243, device="cuda")
+    for f in (128, 256):
+        bench_aggregation("c2", ptr, idx, 169343, 169343, f, iters)
+
+
+def c3(iters):
+    import cxgnncomp_backend as B
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    N = 2449029
+    ptr, idx = S.powerlaw_symmetric_graph(N, 30929570, device="cuda")
+    E = idx.shape[0]
+    bench_aggregation("c3", ptr, idx, N, N, 128, iters, weighted=False)
+    H, C = 4, 64
+    att_s = torch.randn(N, H, device="cuda")
+    att_d = torch.randn(N, H, device="cuda")
+    ev, mask = _ops.edge_softmax_fwd(ptr, idx, att_d, att_s, E, 0.2)
+    sm_bytes = E * (8 + 4 * H) + 4 * E * H + E * H + 4 * N * H + 8 * (N + 1)
+    report("c3", "edge_softmax_fwd H=4", timeit(lambda: _ops.edge_softmax_fwd(ptr, idx, att_d, att_s, E, 0.2), iters),
+           sm_bytes, 6 * E * H)
+    gev = torch.randn(E, H, device="cuda")
+    gt = _ops.transposed(ptr, idx, N, N)
+
+    def sm_bwd():
+        g_dst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, gev, N, 0.2)
+        return _ops.narrow_gather_sum(gt.ptr_t, gt.perm, t_edge, N)
+    report("c3", "edge_softmax_bwd H=4 (row pass + transposed gather)", timeit(sm_bwd, iters),
+           E * H * (4 + 4 + 1 + 4) + E * (8 + 4 * H) + 8 * N * H, 6 * E * H)
+    x = torch.randn(N, H, C, device="cuda") / 8
+    g = torch.randn(N, H, C, device="cuda") / 8
+    report("c3", "spmm_multihead_fwd H=4 C=64", timeit(lambda: _ops.spmm(ptr, idx, x, N, val=ev), iters),
+           spmm_bytes(N, E, H * C, H), 2 * E * H * C)
+    report("c3", "spmm_multihead_bwd H=4 C=64",
+           timeit(lambda: _ops.spmm(gt.ptr_t, gt.idx_t, g, N, val=ev, val_perm=gt.perm), iters),
+           spmm_bytes(N, E, H * C, H) + 8 * E, 2 * E * H * C)
+    report("c3", "sddmm_csr (edge-value grad) H=4 C=64", timeit(lambda: _ops.sddmm_csr(ptr, idx, x, g, N), iters),
+           E * (4 * H * C + 8) + 4 * N * H * C + 4 * E * H, 2 * E * H * C)
+    dst = _ops.csr_row_ids(ptr, N, E)
+    out = torch.empty(E, H, device="cuda")
+    report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),
+           E * (8 * H * C + 16) + 4 * E * H, 2 * E * H * C)
+    del x, g
+
+
+def c4(iters):
+    import cxgnncomp
+    import cxgnncomp_backend as B
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _typed
+    N, E, R, K = 1000000, 20000000, 16, 128
+    ptr, idx, etype, _ = S.hetero_graph(N, E, num_rel=R, device="cuda")
+    x = torch.randn(N, K, device="cuda") / 8
+    w = torch.randn(R, K, K, device="cuda") * 0.02
+    rel32 = etype.int()
+    perm, seg = _typed.rel_segment(rel32, R)
+    rows = B._ops.csr_row_ids(ptr, N, E)
+    src, dst = idx[perm], rows[perm]
+    out = torch.zeros(N, K, device="cuda")
+    flops = 2.0 * E * K * K
+    fused_bytes = E * (4 * K + 8 + 8 + 4 * K) + 4 * R * K * K
+    report("c4", "rel_segment (stable sort by relation)", timeit(lambda: _typed.rel_segment(rel32, R), iters))
+
+    def fused(bf16):
+        out.zero_()
+        _typed.typed_gemm(x, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, bf16=bf16)
+    report("c4", "rgcn fused gather-GEMM-scatter fp32 MFMA", timeit(lambda: fused(False), iters), fused_bytes, flops,
+           MFMA_F32)
+    x16 = x.to(torch.bfloat16)
+
+    def fused16():
+        out.zero_()
+        _typed.typed_gemm(x16, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, bf16=True)
+    report("c4", "rgcn fused gather-GEMM-scatter bf16 MFMA", timeit(fused16, iters),
+           E * (2 * K + 16 + 4 * K) + 2 * R * K * K, flops, MFMA_BF16)
+    xe = torch.empty(E, K, device="cuda")
+    xe.normal_()
+    oe = torch.empty(E, K, device="cuda")
+    report("c4", "typed GEMM edge->edge fp32 (E x 128 x 128, sorted rows)",
+           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe), iters), E * 8 * K + 4 * R * K * K, flops, MFMA_F32)
+    xe16 = xe.to(torch.bfloat16)
+    report("c4", "typed GEMM edge->edge bf16",
+           timeit(lambda: _typed.typed_gemm(xe16, w, seg, E, out=oe, bf16=True), iters),
+           E * 6 * K + 2 * R * K * K, flops, MFMA_BF16)
+    del xe, oe, xe16
+    report("c4", "torch.mm [1M,128]x[128,128] x 20 (library GEMM of the same flops, no gather, for scale)",
+           (E / N) * timeit(lambda: torch.mm(x, w[0]), iters), E * 8 * K, flops, MFMA_F32)
+    layer = cxgnncomp.MyRGCNConv(K, K, R).cuda()
+    xg = x.clone().requires_grad_(True)
+
+    def layer_step():
+        xg.grad = None
+        o = layer(xg, ptr, idx, etype, N)
+        o.sum().backward()
+    report("c4", "MyRGCNConv layer fwd+bwd (gather, typed GEMM, aggregate, /deg)", timeit(layer_step, max(2, iters // 3)))
+
+
+def c5(iters):
+    import cxgnncomp
+    from cxgnncomp import synthetic as S
+    ptr, idx, nn, ne = S.sampled_batch(device="cuda")
+    n_src = nn[-1]
+    x = torch.randn(n_src, 128, device="cuda")
+    layers = [cxgnncomp.MySageConv(128, 256).cuda(), cxgnncomp.MySageConv(256, 256).cuda(),
+              cxgnncomp.MySageConv(256, 47).cuda()]
+    import cxgnncomp_backend as B
+    for li, (rows, edges) in enumerate(zip(nn[2::-1], ne[::-1])):
+        report("c5", "sage_mean_forward rows=%d edges=%d F=128" % (rows, edges),
+               timeit(lambda: B.sage_mean_forward(x, ptr, idx, rows), iters), spmm_bytes(rows, edges, 128), edges * 128)
+    xg = x.clone().requires_grad_(True)
+
+    def batch_step():
+        xg.grad = None
+        h = xg
+        for li, layer in enumerate(layers):
+            h = layer(h, ptr, idx, nn[2 - li])
+            if li < 2:
+                h = torch.relu(h)
+        h.sum().backward()
+    report("c5", "3-layer SAGE fwd+bwd per batch (%s nodes per layer)" % nn, timeit(batch_step, iters))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
+    ap.add_argument("--iters", type=int, default=10)
+    args = ap.parse_args()
+    table = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5}
+    for name in args.configs.split(","):
+        table[name](args.iters)
+        torch.cuda.empty_cache()
+
+
+if __name__ == "__main__":
+    main()

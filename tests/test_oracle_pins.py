@@ -357,3 +357,33 @@ def test_index_work_invariants_and_brute_force():
     assert np.array_equal(np.sort(indices), np.arange(len(buf)))
     for t in range(0, int((st < 6).sum()), thres):       # one relation per tile of thres rows
         assert len(set(st[t:t + thres])) == 1
+
+
+# ----------------------------------------------------------------------------- remaining pure-python restatements
+def test_small_hand_cases_for_row_filters_and_select_mm():
+    ptr = np.array([0, 2, 2, 5, 6])
+    idx = np.array([10, 11, 12, 13, 14, 15])
+    # rows 1 and 2 removed: rows 0 and 3 remain
+    p, i = pyref.remove_from_graph(ptr, idx, np.array([False, True, True, False]))
+    assert p.tolist() == [0, 2, 3] and i.tolist() == [10, 11, 15]
+    # edges 0, 1 (all of row 0) and 3 removed: row 0 disappears, row 1 was already empty
+    p, i = pyref.remove_from_graph_by_edge(ptr, idx, np.array([True, True, False, True, False, False]))
+    assert p.tolist() == [0, 2, 3] and i.tolist() == [12, 14, 15]
+    # coo -> csr keeps the input order inside a destination and agrees with scipy
+    src = np.array([5, 1, 7, 3, 9, 2])
+    dst = np.array([2, 0, 2, 1, 0, 2])
+    cp, ci = oracle.coo_to_csr(src, dst, 4)
+    assert cp.tolist() == [0, 2, 3, 6, 6] and ci.tolist() == [1, 9, 3, 5, 7, 2]
+    m = sp.coo_matrix((np.ones(6), (dst, src)), shape=(4, 10)).tocsr()
+    assert np.array_equal(m.indptr, cp)
+    # per-relation select + mm and the gathered-weight form against a direct loop over rows
+    x = torch.arange(12, dtype=torch.float64).reshape(4, 3)
+    w = torch.stack([torch.eye(3, dtype=torch.float64), 2 * torch.eye(3, dtype=torch.float64)])
+    eidx = torch.tensor([3, 0, 2, 1, 3])
+    types = torch.tensor([1, 0, 1, 1, 0])
+    parts = pyref.select_mm_s2e(x, w, eidx, types)
+    assert torch.equal(parts[0], x[[0, 3]]) and torch.equal(parts[1], 2 * x[[3, 2, 1]])
+    dstn = torch.tensor([0, 1, 0, 1, 1])
+    out = pyref.typed_linear_naive_s2d(x, w, types, eidx, dstn, 2, 5)
+    want = torch.stack([2 * x[3] + 2 * x[2], x[0] + 2 * x[1] + x[3]])
+    assert torch.equal(out, want)
