@@ -20,6 +20,19 @@ constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
 constexpr int kSpan = 256;
 
+#ifndef CXG_SDDMM_U
+#define CXG_SDDMM_U 16
+#endif
+#ifndef CXG_SDDMM_U_V4
+#define CXG_SDDMM_U_V4 8
+#endif
+#ifndef CXG_SDDMM_COO_U
+#define CXG_SDDMM_COO_U 8
+#endif
+#ifndef CXG_SDDMM_COO_U_V4
+#define CXG_SDDMM_COO_U_V4 4
+#endif
+
 template <int V> struct Vec;
 template <> struct Vec<1> { using type = float; };
 template <> struct Vec<2> { using type = float2; };
@@ -37,8 +50,20 @@ template <> __device__ __forceinline__ float4 vzero<4>() { return make_float4(0.
 
 // Sum over aligned groups of `group` lanes (power of two <= 64); every lane of a
 // group ends with the group's total.
+// The first four butterfly steps stay inside a 16-lane DPP row and use data-parallel
+// primitives (quad permutes and row mirrors, a few cycles each); only groups wider
+// than a row need the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float group_sum(float v, int group) {
-  for (int m = 1; m < group; m <<= 1) v += __shfl_xor(v, m, CXG_WAVE);
+  if (group >= 2) v += dpp_f32<0xB1>(v);    // quad_perm [1,0,3,2]: lane ^ 1
+  if (group >= 4) v += dpp_f32<0x4E>(v);    // quad_perm [2,3,0,1]: lane ^ 2
+  if (group >= 8) v += dpp_f32<0x141>(v);   // row_half_mirror: the other quad of 8
+  if (group >= 16) v += dpp_f32<0x140>(v);  // row_mirror: the other half of 16
+  if (group >= 32) v += __shfl_xor(v, 16, CXG_WAVE);
+  if (group >= 64) v += __shfl_xor(v, 32, CXG_WAVE);
   return v;
 }
 
@@ -61,7 +86,7 @@ struct SddmmArgs {
 template <int V>
 __global__ __launch_bounds__(kBlock) void sddmm_csr_packed_kernel(SddmmArgs a) {
   using vec_t = typename Vec<V>::type;
-  constexpr int U = (V == 4) ? 8 : 16;
+  constexpr int U = (V == 4) ? CXG_SDDMM_U_V4 : CXG_SDDMM_U;
   const int lane = lane_id();
   const int wave = uniform_i32(threadIdx.x >> 6);
   const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -127,7 +152,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_csr_packed_kernel(SddmmArgs a) {
 template <int V>
 __global__ __launch_bounds__(kBlock) void sddmm_coo_packed_kernel(SddmmArgs a) {
   using vec_t = typename Vec<V>::type;
-  constexpr int U = (V == 4) ? 4 : 8;
+  constexpr int U = (V == 4) ? CXG_SDDMM_COO_U_V4 : CXG_SDDMM_COO_U;
   const int lane = lane_id();
   const int wave = uniform_i32(threadIdx.x >> 6);
   const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;

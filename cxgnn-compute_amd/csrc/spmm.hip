@@ -21,6 +21,13 @@
 namespace cxg {
 namespace {
 
+#ifndef CXG_SPMM_U
+#define CXG_SPMM_U 1
+#endif
+#ifndef CXG_SPMM_U_V4
+#define CXG_SPMM_U_V4 8
+#endif
+
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
 
@@ -295,7 +302,12 @@ Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
 
 template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT>
 int launch_spmm(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
-  constexpr int U = (V == 4) ? 8 : 16;
+  // Gathers in flight per wave.  Measured on MI355X (61.9M-edge power-law graph):
+  // with 32 waves per CU the memory system is already saturated, and issuing more
+  // than one row gather per wave at a time only lengthens the queues and lowers
+  // the L2 hit rate (F=128: 16 in flight 5.56 ms, 8: 4.94, 4: 4.51, 1: 4.31 ms).
+  // 16-byte-per-lane gathers (V == 4) are flat from 1 to 8 and best at 8.
+  constexpr int U = (V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U;
   const int tile = CXG_WAVE * V;
   dim3 grid((unsigned)ceil_div(n_spans_cap, kWavesPerBlock), (unsigned)ceil_div(a.F, tile), 1);
   dim3 block(kBlock, 1, 1);
