@@ -151,11 +151,13 @@ def c4(iters):
     fused_bytes = E * (4 * K + 8 + 8 + 4 * K) + 4 * R * K * K
     report("c4", "rel_segment (stable sort by relation)", timeit(lambda: _typed.rel_segment(rel32, R), iters))
 
-    def fused(bf16):
+    def fused(precision):
         out.zero_()
-        _typed.typed_gemm(x, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, bf16=bf16)
-    report("c4", "rgcn fused gather-GEMM-scatter fp32 MFMA", timeit(lambda: fused(False), iters), fused_bytes, flops,
-           MFMA_F32)
+        _typed.typed_gemm(x, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, precision=precision)
+    report("c4", "rgcn fused gather-GEMM-scatter fp32 MFMA", timeit(lambda: fused("fp32"), iters), fused_bytes,
+           flops, MFMA_F32)
+    report("c4", "rgcn fused gather-GEMM-scatter fp32 as 3 bf16 products", timeit(lambda: fused("split"), iters),
+           fused_bytes, flops)
     x16 = x.to(torch.bfloat16)
 
     def fused16():
@@ -167,7 +169,11 @@ def c4(iters):
     xe.normal_()
     oe = torch.empty(E, K, device="cuda")
     report("c4", "typed GEMM edge->edge fp32 (E x 128 x 128, sorted rows)",
-           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe), iters), E * 8 * K + 4 * R * K * K, flops, MFMA_F32)
+           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="fp32"), iters),
+           E * 8 * K + 4 * R * K * K, flops, MFMA_F32)
+    report("c4", "typed GEMM edge->edge fp32 as 3 bf16 products",
+           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="split"), iters),
+           E * 8 * K + 4 * R * K * K, flops)
     xe16 = xe.to(torch.bfloat16)
     report("c4", "typed GEMM edge->edge bf16",
            timeit(lambda: _typed.typed_gemm(xe16, w, seg, E, out=oe, bf16=True), iters),

@@ -1,6 +1,8 @@
 """Typed GEMM, relation segmentation and the relational ops built on them
 (binding.cpp:45-54): pad_rel*, typed_linear*, aggr_rel_direct,
 aggr_rgcn_direct_func, seastar_*."""
+import os
+
 import torch
 
 from . import _lib, _ops
@@ -8,6 +10,11 @@ from ._ops import _req, _workspace, as_int
 
 GEMM_ACCUMULATE = 1
 GEMM_ATOMIC = 2
+GEMM_SPLIT_BF16 = 4
+
+# How fp32 typed GEMMs multiply: "split" (three bf16 partial products per fp32
+# product, HBM bound for K, N <= 128) or "fp32" (v_mfma_f32_32x32x2_f32).
+GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split")
 
 
 def rel_segment(types, num_rel):
@@ -31,11 +38,14 @@ def rel_segment(types, num_rel):
 
 
 def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n_out=None,
-               accumulate=False, atomic=False, bf16=False):
+               accumulate=False, atomic=False, bf16=False, precision=None):
     """out[dst(i)] (=|+=) a[src(i)] @ w[r] for rows i of segment r (see cxg_typed_gemm_f32).
 
-    a [*, K] fp32, w [R, K, N] fp32.  With bf16=True the operands are rounded to
-    bf16 (W transposed to [R, N, K]) and multiplied on the bf16 matrix cores."""
+    a [*, K] fp32, w [R, K, N] fp32.  precision "split" (the default, see
+    GEMM_PRECISION) lets the library form fp32 products from three bf16 partial
+    products (relative error per product < 2^-16, the reference's tl.dot is TF32);
+    "fp32" forces v_mfma_f32_32x32x2_f32.  With bf16=True the operands are rounded
+    to bf16 (W transposed to [R, N, K]) and multiplied on the bf16 matrix cores."""
     lib = _lib.load()
     _req(a, "a", torch.float32 if not (bf16 and a.dtype == torch.bfloat16) else torch.bfloat16, 2)
     if w.dim() != 3:
@@ -64,6 +74,11 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
     if dst_idx is None and out.shape[0] < m_rows:
         raise ValueError("output has fewer rows than M")
     flags = (GEMM_ACCUMULATE if accumulate else 0) | (GEMM_ATOMIC if atomic else 0)
+    precision = precision or GEMM_PRECISION
+    if precision not in ("split", "fp32"):
+        raise ValueError("precision must be 'split' or 'fp32'")
+    if precision == "split":
+        flags |= GEMM_SPLIT_BF16
     stream = _lib.current_stream(a.device)
     with torch.cuda.device(a.device):
         if bf16:

@@ -191,6 +191,7 @@ int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const floa
 
 #define CXG_GEMM_ACCUMULATE 1u /* C += A W instead of C = A W                      */
 #define CXG_GEMM_ATOMIC 2u     /* add with fp32 atomics (several rows share a dst) */
+#define CXG_GEMM_SPLIT_BF16 4u /* fp32 operands may be multiplied as 3 bf16 partial products */
 
 /*
  * C[dst(i), :] = A[src(i), :] @ W[r] for the rows i in [seg_ptr[r], seg_ptr[r+1]),
@@ -198,7 +199,12 @@ int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const floa
  * a negative src or dst skips the row.  A is [*, K] (row stride lda), W is
  * [R, K, N], C is [*, N] (row stride ldc), all fp32; seg_ptr is a device array of
  * R+1 row offsets (see cxg_rel_segment_*).  Computed with
- * v_mfma_f32_32x32x2_f32.  Replaces typed_matmul
+ * v_mfma_f32_32x32x2_f32; with CXG_GEMM_SPLIT_BF16 (and K <= 128, K and lda
+ * multiples of 4, A 16-byte aligned) every operand is split into two bf16 halves
+ * and a*b is formed as hi*hi + lo*hi + hi*lo on v_mfma_f32_32x32x16_bf16 with
+ * fp32 accumulation: relative error per product below 2^-16 (the reference's
+ * tl.dot runs in TF32, 2^-11), HBM bound instead of matrix-core bound.  Replaces
+ * typed_matmul
  * (cxgnncomp/codegen/triton_typed_matmul.py:752-860: src_idx only = its
  * "single index" kernel with dst = src, seq_output = dst NULL, both = double
  * index) and, with row maps and CXG_GEMM_ACCUMULATE / CXG_GEMM_ATOMIC, the
