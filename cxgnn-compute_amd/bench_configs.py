@@ -156,7 +156,7 @@ def c4(iters):
         _typed.typed_gemm(x, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, precision=precision)
     report("c4", "rgcn fused gather-GEMM-scatter fp32 MFMA", timeit(lambda: fused("fp32"), iters), fused_bytes,
            flops, MFMA_F32)
-    report("c4", "rgcn fused gather-GEMM-scatter fp32 as 3 bf16 products", timeit(lambda: fused("split"), iters),
+    report("c4", "rgcn fused gather-GEMM-scatter fp32 as 6 bf16 products", timeit(lambda: fused("split6"), iters),
            fused_bytes, flops)
     x16 = x.to(torch.bfloat16)
 
@@ -171,9 +171,10 @@ def c4(iters):
     report("c4", "typed GEMM edge->edge fp32 (E x 128 x 128, sorted rows)",
            timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="fp32"), iters),
            E * 8 * K + 4 * R * K * K, flops, MFMA_F32)
-    report("c4", "typed GEMM edge->edge fp32 as 3 bf16 products",
-           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="split"), iters),
-           E * 8 * K + 4 * R * K * K, flops)
+    for prec, nprod in (("split6", 6), ("split3", 3)):
+        report("c4", "typed GEMM edge->edge fp32 as %d bf16 products" % nprod,
+               timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision=prec), iters),
+               E * 8 * K + 4 * R * K * K, flops)
     xe16 = xe.to(torch.bfloat16)
     report("c4", "typed GEMM edge->edge bf16",
            timeit(lambda: _typed.typed_gemm(xe16, w, seg, E, out=oe, bf16=True), iters),

@@ -265,33 +265,48 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_kernel(GemmArgs g) {
 }
 
 // ----------------------------------------------------------------------------
-// fp32 operands, products on the bf16 matrix cores as three partial products
+// fp32 operands, products on the bf16 matrix cores as partial products
 // ----------------------------------------------------------------------------
-// x = hi + lo with hi = bf16(x), lo = bf16(x - hi) keeps 16 significant bits of
-// each operand; a*b ~= hi_a*hi_b + lo_a*hi_b + hi_a*lo_b (fp32 accumulate) has a
-// relative error below 2^-16 per product -- 30x tighter than the TF32 tl.dot of
-// the reference's Triton kernel -- at 3/16 of the fp32-MFMA cycles, which turns
-// the K, N <= 128 typed GEMM from matrix-core bound into HBM bound.
+// x = p0 + p1 (+ p2) with p0 = bf16(x), p1 = bf16(x - p0), p2 = bf16(x - p0 - p1):
+// NS parts keep 8*NS significant bits of each operand.  a*b is accumulated in fp32
+// from the partial products a_i*b_j with i + j < NS, smallest first:
+//   NS = 3: six products, every dropped term is below 2^-24 |ab| -- the result is
+//           as accurate as an fp32 FMA chain;
+//   NS = 2: three products, relative error per product below 2^-16 (the TF32
+//           tl.dot of the reference's Triton kernel is 2^-11).
+// Six bf16 MFMAs take 3/8 of the cycles of the fp32 MFMA for the same K, which
+// turns the K, N <= 128 typed GEMM from matrix-core bound into HBM bound.
 //
 // A block owns up to G consecutive 64-row tiles of ONE relation and keeps that
 // relation's weight slab in registers, already split and in MFMA operand layout
 // (wave w: columns 32w..32w+31), so W is fetched once per 64*G rows.  A tiles are
 // fetched as whole 16-byte-per-lane row segments, split on the way into LDS, and
-// the next tile's loads are in flight while the current one is multiplied.
-template <int KS>
+// the loads of the next two tiles are in flight while the current one is multiplied.
+template <int NS>
+__device__ __forceinline__ void split_bf16(float x, __bf16 (&p)[NS]) {
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    p[i] = (__bf16)x;
+    x -= (float)p[i];
+  }
+}
+
+template <int KS, int NS>
 __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, int G) {
   constexpr int KP = KS * 16 + 8;          // padded LDS row (bf16 elements)
   constexpr int LPR = KS * 4;              // lanes per A row, one float4 each
   constexpr int RPI = kThreads / LPR;      // rows per load instruction
   constexpr int NLD = kBM / RPI;           // load instructions per tile
-  __shared__ __attribute__((aligned(16))) uint16_t Ah[kBM][KP];
-  __shared__ __attribute__((aligned(16))) uint16_t Al[kBM][KP];
-  __shared__ int64_t s_src[2][kBM], s_dst[2][kBM];
+  __shared__ __attribute__((aligned(16))) uint16_t Ap[NS][kBM][KP];
+  __shared__ int64_t s_src[3][kBM], s_dst[3][kBM];
   const int64_t span = (int64_t)kBM * G;
   int rel = -1;
   int64_t row0 = 0, row_end = 0;
+  // Column tiles vary fastest over the block index, so the blocks that read the
+  // same A rows run at the same time and share them through the caches.
+  const int n_ct = (g.N + 127) / 128;
   {
-    int64_t t = blockIdx.x;
+    int64_t t = blockIdx.x / n_ct;
     for (int r = 0; r < g.R; ++r) {
       const int64_t b = g.seg[r], e = g.seg[r + 1];
       const int64_t nt = (e - b + span - 1) / span;
@@ -301,13 +316,13 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
   }
   if (rel < 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.y * 128;
+  const int n0 = (int)(blockIdx.x % n_ct) * 128;
   const int K = g.K, N = g.N;
   const int64_t rows_here = (row_end - row0) < span ? (row_end - row0) : span;
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
   // this wave's 32 columns of W[rel], split, in B-operand layout
-  v8bf bh[KS], bl[KS];
+  v8bf bw[NS][KS];
   {
     const float* W = reinterpret_cast<const float*>(g.w) + (int64_t)rel * K * N;
     const int col = n0 + wave * 32 + (lane & 31);
@@ -317,9 +332,10 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
       for (int j = 0; j < 8; ++j) {
         const int k = s * 16 + (lane >> 5) * 8 + j;
         const float w = (k < K && col < N) ? W[(int64_t)k * N + col] : 0.f;
-        const __bf16 hi = (__bf16)w;
-        bh[s][j] = hi;
-        bl[s][j] = (__bf16)(w - (float)hi);
+        __bf16 parts[NS];
+        split_bf16<NS>(w, parts);
+#pragma unroll
+        for (int q = 0; q < NS; ++q) bw[q][s][j] = parts[q];
       }
     }
   }
@@ -327,9 +343,8 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
   const int c4 = tid % LPR, rsub = tid / LPR;
   const bool k_ok = 4 * c4 < K;
   const float* A = reinterpret_cast<const float*>(g.a);
-  float4 areg[NLD];
-  auto load_maps = [&](int t, int buf) {
-    if (tid < kBM) {
+  auto load_maps = [&](int t) {
+    if (tid < kBM && t < n_tiles) {
       const int64_t gr = row0 + (int64_t)t * kBM + tid;
       int64_t sidx = -1, didx = -1;
       if (gr < row_end) {
@@ -337,44 +352,41 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
         didx = g.dst ? g.dst[gr] : gr;
         if (sidx < 0 || didx < 0) { sidx = -1; didx = -1; }
       }
-      s_src[buf][tid] = sidx;
-      s_dst[buf][tid] = didx;
+      s_src[t % 3][tid] = sidx;
+      s_dst[t % 3][tid] = didx;
     }
   };
-  auto gload = [&](int buf) {
+  auto gload = [&](float4 (&areg)[NLD], int t) {
+    if (t >= n_tiles) return;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int64_t sidx = s_src[buf][i * RPI + rsub];
+      const int64_t sidx = s_src[t % 3][i * RPI + rsub];
       areg[i] = (sidx >= 0 && k_ok) ? *reinterpret_cast<const float4*>(A + sidx * g.lda + 4 * c4)
                                     : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   };
-  auto sstore = [&]() {
+  // One tile: stage its rows (already in registers) into LDS, start the loads of
+  // tile t + 2 into the same registers, multiply, store.
+  auto tile_step = [&](float4 (&areg)[NLD], int t) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const float v[4] = {areg[i].x, areg[i].y, areg[i].z, areg[i].w};
       typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
-      v4bf h, l;
+      v4bf part[NS];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        h[j] = (__bf16)v[j];
-        l[j] = (__bf16)(v[j] - (float)h[j]);
+        __bf16 parts[NS];
+        split_bf16<NS>(v[j], parts);
+#pragma unroll
+        for (int q = 0; q < NS; ++q) part[q][j] = parts[q];
       }
       const int row = i * RPI + rsub;
-      *reinterpret_cast<v4bf*>(&Ah[row][4 * c4]) = h;
-      *reinterpret_cast<v4bf*>(&Al[row][4 * c4]) = l;
+#pragma unroll
+      for (int q = 0; q < NS; ++q) *reinterpret_cast<v4bf*>(&Ap[q][row][4 * c4]) = part[q];
     }
-  };
-
-  load_maps(0, 0);
-  __syncthreads();
-  gload(0);
-  for (int t = 0; t < n_tiles; ++t) {
-    const int cur = t & 1;
-    sstore();
-    if (t + 1 < n_tiles) load_maps(t + 1, cur ^ 1);
+    load_maps(t + 2);
     __syncthreads();
-    if (t + 1 < n_tiles) gload(cur ^ 1);
+    gload(areg, t + 2);
     v16f acc[2];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -385,22 +397,36 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         const int row = mt * 32 + (lane & 31), k = s * 16 + (lane >> 5) * 8;
-        const v8bf ah = *reinterpret_cast<const v8bf*>(&Ah[row][k]);
-        const v8bf al = *reinterpret_cast<const v8bf*>(&Al[row][k]);
-        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[s], acc[mt], 0, 0, 0);
-        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[s], acc[mt], 0, 0, 0);
-        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[s], acc[mt], 0, 0, 0);
+        v8bf ap[NS];
+#pragma unroll
+        for (int q = 0; q < NS; ++q) ap[q] = *reinterpret_cast<const v8bf*>(&Ap[q][row][k]);
+#pragma unroll
+        for (int order = NS - 1; order >= 0; --order)
+#pragma unroll
+          for (int i = 0; i <= order; ++i)
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[i], bw[order - i][s], acc[mt], 0, 0, 0);
       }
     }
-    store_tile<128, 2>(g, acc, s_dst[cur], 0, wave, lane, n0);
-    __syncthreads();   // every wave is done with Ah/Al and s_dst[cur]
+    store_tile<128, 2>(g, acc, s_dst[t % 3], 0, wave, lane, n0);
+    __syncthreads();   // every wave is done with Ap before the next tile is staged
+  };
+
+  float4 areg0[NLD], areg1[NLD];
+  load_maps(0);
+  load_maps(1);
+  __syncthreads();
+  gload(areg0, 0);
+  gload(areg1, 1);
+  for (int t = 0; t < n_tiles; t += 2) {
+    tile_step(areg0, t);
+    if (t + 1 < n_tiles) tile_step(areg1, t + 1);
   }
 }
 
 int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64_t M, int K, int N,
                int R, unsigned flags) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
-  CXG_REQUIRE((flags & ~7u) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE((flags & ~15u) == 0, CXG_ERR_ARG, "unknown flag");
   if (M == 0) return CXG_OK;
   CXG_REQUIRE(a && w && c && seg, CXG_ERR_ARG, "null pointer");
   return CXG_OK;
@@ -420,15 +446,25 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   cxg::GemmArgs g{a, lda, w, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
                   (int)(flags & 1u), (int)((flags >> 1) & 1u)};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if ((flags & CXG_GEMM_SPLIT_BF16) && K <= 128 && (K & 3) == 0 && (lda & 3) == 0 &&
+  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3)) && K <= 128 && (K & 3) == 0 && (lda & 3) == 0 &&
       ((uintptr_t)a & 15) == 0) {
-    // 64*G rows per block: 8 tiles when the launch still has a few thousand blocks
-    int G = (int)(M / ((int64_t)cxg::kBM * 2048));
-    G = G < 1 ? 1 : (G > 8 ? 8 : G);
-    const dim3 grid((unsigned)(cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R), (unsigned)cxg::ceil_div(N, 128));
-    if (K <= 32) hipLaunchKernelGGL(cxg::typed_gemm_split_kernel<2>, grid, dim3(cxg::kThreads), 0, st, g, G);
-    else if (K <= 64) hipLaunchKernelGGL(cxg::typed_gemm_split_kernel<4>, grid, dim3(cxg::kThreads), 0, st, g, G);
-    else hipLaunchKernelGGL(cxg::typed_gemm_split_kernel<8>, grid, dim3(cxg::kThreads), 0, st, g, G);
+    // 64*G rows per block: up to 32 tiles while the launch keeps a few thousand blocks
+    int G = (int)(M / ((int64_t)cxg::kBM * 4096));
+    G = G < 1 ? 1 : (G > 32 ? 32 : G);
+    const int64_t n_blocks = (cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R) * cxg::ceil_div(N, 128);
+    CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
+    const dim3 grid((unsigned)n_blocks);
+#define CXG_SPLIT(KS)                                                                          \
+  do {                                                                                         \
+    if (flags & CXG_GEMM_SPLIT_BF16X3)                                                         \
+      hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, 2>), grid, dim3(cxg::kThreads), 0, st, g, G); \
+    else                                                                                       \
+      hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, 3>), grid, dim3(cxg::kThreads), 0, st, g, G); \
+  } while (0)
+    if (K <= 32) CXG_SPLIT(2);
+    else if (K <= 64) CXG_SPLIT(4);
+    else CXG_SPLIT(8);
+#undef CXG_SPLIT
     CXG_LAUNCH_CHECK("typed_gemm_split_kernel");
     return CXG_OK;
   }

@@ -230,12 +230,11 @@ class MyRGCNConv(torch.nn.Module):
     def forward(self, x, ptr, idx, edge_types, num_node):
         if idx.shape[0] > 1e8:
             return RGCNOP.apply(x, self.linear, ptr, idx, edge_types, num_node)
-        if len(self.preprocessed) == 0:
-            self.preprocessed = TypedLinearE2EOP.preprocess(self.linear, edge_types)
-        out = run_rgcn4(x, ptr, idx, edge_types, self.linear, num_node, num_edge=edge_types.shape[0],
-                        preproccessed=self.preprocessed)
-        deg = ptr[1:] - ptr[:-1]
-        return out / deg.unsqueeze(-1)[:out.shape[0]]
+        # Upstream gathers x[idx], runs the edge-level typed linear and sums the edge
+        # rows of every destination (run_rgcn4, :309-326, :352-378); the same layer as
+        # one op that never materialises per-edge rows.  Rows without edges give 0
+        # (upstream divides 0 by 0 there).
+        return cxgnncomp_backend.aggr_rgcn_mean(x, ptr, idx, self.linear, edge_types, num_node)
 
 
 class MyGATConv(torch.nn.Module):

@@ -237,7 +237,7 @@ def gather(input, dest, num_node):
 
 from ._rel import (aggr_rel, selective_aggr, selective_aggr_bwd, target_aggr,  # noqa: E402,F401
                    target_aggr_backward)
-from ._typed import (aggr_rel_direct, aggr_rgcn_direct_func, pad_rel, pad_rel_idx,  # noqa: E402,F401
+from ._typed import (aggr_rel_direct, aggr_rgcn_direct_func, aggr_rgcn_mean, pad_rel, pad_rel_idx,  # noqa: E402,F401
                      seastar_backward, seastar_forward, typed_linear, typed_linear_s2d,
                      typed_linear_s2e)
 from ._schedule import (COMPUTEOP, REDUCEOP, GSpMM_u, GSpMM_u_e, gen_edge_type_mag240m,  # noqa: E402,F401

@@ -1,6 +1,7 @@
 """Typed GEMM, relation segmentation and the relational ops built on them
 (binding.cpp:45-54): pad_rel*, typed_linear*, aggr_rel_direct,
 aggr_rgcn_direct_func, seastar_*."""
+import collections
 import os
 
 import torch
@@ -10,11 +11,14 @@ from ._ops import _req, _workspace, as_int
 
 GEMM_ACCUMULATE = 1
 GEMM_ATOMIC = 2
-GEMM_SPLIT_BF16 = 4
+GEMM_SPLIT_BF16X6 = 4
+GEMM_SPLIT_BF16X3 = 8
 
-# How fp32 typed GEMMs multiply: "split" (three bf16 partial products per fp32
-# product, HBM bound for K, N <= 128) or "fp32" (v_mfma_f32_32x32x2_f32).
-GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split")
+# How fp32 typed GEMMs multiply: "split6" (six bf16 partial products per fp32
+# product: fp32-accurate and HBM bound for K <= 128), "split3" (three partial
+# products, relative error below 2^-16 per product) or "fp32" (v_mfma_f32_32x32x2_f32).
+GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split6")
+_PRECISION_FLAGS = {"fp32": 0, "split6": GEMM_SPLIT_BF16X6, "split3": GEMM_SPLIT_BF16X3}
 
 
 def rel_segment(types, num_rel):
@@ -41,10 +45,10 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
                accumulate=False, atomic=False, bf16=False, precision=None):
     """out[dst(i)] (=|+=) a[src(i)] @ w[r] for rows i of segment r (see cxg_typed_gemm_f32).
 
-    a [*, K] fp32, w [R, K, N] fp32.  precision "split" (the default, see
-    GEMM_PRECISION) lets the library form fp32 products from three bf16 partial
-    products (relative error per product < 2^-16, the reference's tl.dot is TF32);
-    "fp32" forces v_mfma_f32_32x32x2_f32.  With bf16=True the operands are rounded
+    a [*, K] fp32, w [R, K, N] fp32.  precision "split6" (the default, see
+    GEMM_PRECISION) forms every fp32 product from six bf16 partial products
+    (fp32-accurate), "split3" from three (relative error per product < 2^-16, the
+    reference's tl.dot is TF32); "fp32" forces v_mfma_f32_32x32x2_f32.  With bf16=True the operands are rounded
     to bf16 (W transposed to [R, N, K]) and multiplied on the bf16 matrix cores."""
     lib = _lib.load()
     _req(a, "a", torch.float32 if not (bf16 and a.dtype == torch.bfloat16) else torch.bfloat16, 2)
@@ -75,10 +79,9 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
         raise ValueError("output has fewer rows than M")
     flags = (GEMM_ACCUMULATE if accumulate else 0) | (GEMM_ATOMIC if atomic else 0)
     precision = precision or GEMM_PRECISION
-    if precision not in ("split", "fp32"):
-        raise ValueError("precision must be 'split' or 'fp32'")
-    if precision == "split":
-        flags |= GEMM_SPLIT_BF16
+    if precision not in _PRECISION_FLAGS:
+        raise ValueError("precision must be one of %s" % sorted(_PRECISION_FLAGS))
+    flags |= _PRECISION_FLAGS[precision]
     stream = _lib.current_stream(a.device)
     with torch.cuda.device(a.device):
         if bf16:
@@ -186,13 +189,67 @@ def _weight_grad(x, g, src, dst, seg, shape):
     return gw
 
 
+# Transform-first RGCN: out[d] = sum_e Y[idx[e], rel[e]] with Y[s, r] = x[s] @ W[r]
+# computed for every (source, relation) pair by one dense GEMM against the
+# concatenated weights.  2 * n_src * R * K * N flops instead of 2 * E * K * N, no
+# atomics, deterministic; the aggregation is the plain SpMM over a combined index.
+# Chosen when the graph has at least half as many edges as (source, relation)
+# pairs and Y fits the memory budget; sparser inputs (sampled blocks with many
+# relations) use the fused gather-GEMM-scatter launch.
+RGCN_DENSE_MAX_BYTES = 64 << 30
+
+
+class _RelGraph:
+    """Index structures of the transform-first path for one (ptr, idx, rel):
+    key_fwd[e] = idx[e] * R + rel[e]; the CSR of the reversed graph with one row
+    per (source, relation) pair (ptr_key, idx_key = destinations); ptr_src =
+    its coarsening to one row per source; key_bwd[k] = idx_key[k] * R + rel."""
+    __slots__ = ("key_fwd", "ptr_key", "idx_key", "ptr_src", "key_bwd", "n_edges", "_keep")
+
+
+_REL_CACHE = collections.OrderedDict()
+_REL_CACHE_CAP = 4
+
+
+def _rel_graph(ptr, idx, rel, n, n_src, R):
+    key = (ptr.data_ptr(), idx.data_ptr(), rel.data_ptr(), ptr.shape[0], idx.shape[0], n, n_src, R,
+           ptr._version, idx._version, rel._version, ptr.device.index)
+    rg = _REL_CACHE.get(key)
+    if rg is not None:
+        _REL_CACHE.move_to_end(key)
+        return rg
+    rg = _RelGraph()
+    rg.n_edges = int(ptr[n].item())
+    rel64 = rel[:rg.n_edges].to(torch.int64)
+    if rg.n_edges and (int(rel64.min()) < 0 or int(rel64.max()) >= R):
+        raise ValueError("relation ids must lie in [0, %d)" % R)
+    rg.key_fwd = idx[:rg.n_edges] * R + rel64
+    rg.ptr_key, rg.idx_key, perm, _ = _ops.csr_transpose(ptr, rg.key_fwd, n, n_src * R)
+    rg.ptr_src = rg.ptr_key[::R].contiguous()
+    rg.key_bwd = rg.idx_key * R + rel64[perm]
+    rg._keep = (ptr, idx, rel)
+    _REL_CACHE[key] = rg
+    while len(_REL_CACHE) > _REL_CACHE_CAP:
+        _REL_CACHE.popitem(last=False)
+    return rg
+
+
+def _dense_seg(n_rows, device):
+    return torch.tensor([0, n_rows], dtype=torch.int64, device=device)
+
+
+def _use_dense(n_edges, n_src, R, N):
+    return 2 * n_edges >= n_src * R and 4 * n_src * R * N <= RGCN_DENSE_MAX_BYTES
+
+
 class _RgcnFusedFunction(torch.autograd.Function):
     """out[r] = sum_e x[idx[e]] @ W[rel[e]] (aggr_rgcn_direct_kernel,
-    src/cpp/src/rel_spmm.cu:138-181).  The reference's backward returns zeros
-    (rel_spmm.cu:400-432); the true gradients are computed here."""
+    src/cpp/src/rel_spmm.cu:138-181), optionally divided by the row's edge count.
+    The reference's backward returns zeros (rel_spmm.cu:400-432); the true
+    gradients are computed here."""
 
     @staticmethod
-    def forward(ctx, x, ptr, idx, weights, rel, num_node):
+    def forward(ctx, x, ptr, idx, weights, rel, num_node, mean=False):
         n = as_int(num_node)
         if n == 0:
             n = ptr.shape[0] - 1
@@ -200,25 +257,63 @@ class _RgcnFusedFunction(torch.autograd.Function):
             raise ValueError("feat_len weight size %d %d" % (x.shape[1], weights.shape[1]))
         x = x.contiguous()
         weights = weights.contiguous()
-        n_edges, src, dst, seg = _edge_segments(ptr, idx, rel, n, weights.shape[0])
-        out = torch.zeros((n, weights.shape[2]), dtype=torch.float32, device=x.device)
+        R, K, N = weights.shape
+        n_src = x.shape[0]
+        ctx.n, ctx.mean = n, mean
+        n_edges = int(ptr[n].item())
+        ctx.dense = _use_dense(n_edges, n_src, R, N)
+        if ctx.dense:
+            rg = _rel_graph(ptr, idx, rel, n, n_src, R)
+            wcat = weights.permute(1, 0, 2).reshape(1, K, R * N).contiguous()
+            y = typed_gemm(x, wcat, _dense_seg(n_src, x.device), n_src)          # [n_src, R*N]
+            out = _ops.spmm(ptr, rg.key_fwd, y.view(n_src * R, N), n, mean=mean)
+            ctx.rg = rg
+            ctx.save_for_backward(x, weights, ptr)
+            return out
+        n_edges, src, dst, seg = _edge_segments(ptr, idx, rel, n, R)
+        out = torch.zeros((n, N), dtype=torch.float32, device=x.device)
         typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=dst, out=out, atomic=True)
-        ctx.save_for_backward(x, weights, src, dst, seg)
+        if mean:
+            out *= _inv_degree(ptr, n).unsqueeze(1)
+        ctx.save_for_backward(x, weights, ptr, src, dst, seg)
         ctx.n_edges = n_edges
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, weights, src, dst, seg = ctx.saved_tensors
         grad_out = grad_out.contiguous()
+        x, weights, ptr = ctx.saved_tensors[:3]
+        R, K, N = weights.shape
+        n, n_src = ctx.n, x.shape[0]
+        if ctx.mean:
+            grad_out = grad_out * _inv_degree(ptr, n).unsqueeze(1)
         gx = gw = None
+        if ctx.dense:
+            rg = ctx.rg
+            if ctx.needs_input_grad[0]:
+                # Z[d, r] = g[d] @ W[r]^T for every (destination, relation), then the
+                # plain SpMM over the reversed graph
+                wcat_t = weights.permute(2, 0, 1).reshape(1, N, R * K).contiguous()
+                z = typed_gemm(grad_out, wcat_t, _dense_seg(n, x.device), n)      # [n, R*K]
+                gx = _ops.spmm(rg.ptr_src, rg.key_bwd, z.view(n * R, K), n_src)
+            if ctx.needs_input_grad[3]:
+                # gY[s, r] = sum of g over the edges (s -> d) of relation r; gW[r] = x^T gY[:, r]
+                gy = _ops.spmm(rg.ptr_key, rg.idx_key, grad_out, n_src * R)      # [n_src*R, N]
+                gw = torch.mm(x.t(), gy.view(n_src, R * N)).view(K, R, N).permute(1, 0, 2).contiguous()
+            return gx, None, None, gw, None, None, None
+        src, dst, seg = ctx.saved_tensors[3:]
         if ctx.needs_input_grad[0]:
             gx = torch.zeros_like(x)
             typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), seg, ctx.n_edges, src_idx=dst,
                        dst_idx=src, out=gx, atomic=True)
         if ctx.needs_input_grad[3]:
             gw = _weight_grad(x, grad_out, src, dst, seg, weights.shape)
-        return gx, None, None, gw, None, None
+        return gx, None, None, gw, None, None, None
+
+
+def _inv_degree(ptr, n):
+    deg = (ptr[1:n + 1] - ptr[:n]).to(torch.float32)
+    return torch.where(deg > 0, 1.0 / deg, torch.zeros_like(deg))
 
 
 def aggr_rgcn_direct_func(input, ptr, idx, weights, rel, num_node):
@@ -226,6 +321,13 @@ def aggr_rgcn_direct_func(input, ptr, idx, weights, rel, num_node):
     if weights.dim() != 3:
         raise ValueError("weights must be [num_rel, in, out]")
     return _RgcnFusedFunction.apply(input, ptr, idx, weights, rel, num_node)
+
+
+def aggr_rgcn_mean(input, ptr, idx, weights, rel, num_node):
+    """aggr_rgcn_direct_func divided by each row's edge count (rows without edges
+    give 0): the whole relational layer of MyRGCNConv
+    (cxgnncomp/graph_conv.py:352-378) in one differentiable op."""
+    return _RgcnFusedFunction.apply(input, ptr, idx, weights, rel, num_node, True)
 
 
 def aggr_rel_direct(input, ptr, idx, weights, etype, num_node, num_rel):

@@ -191,7 +191,8 @@ int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const floa
 
 #define CXG_GEMM_ACCUMULATE 1u /* C += A W instead of C = A W                      */
 #define CXG_GEMM_ATOMIC 2u     /* add with fp32 atomics (several rows share a dst) */
-#define CXG_GEMM_SPLIT_BF16 4u /* fp32 operands may be multiplied as 3 bf16 partial products */
+#define CXG_GEMM_SPLIT_BF16X6 4u /* fp32 products as 6 bf16 partial products (fp32-accurate) */
+#define CXG_GEMM_SPLIT_BF16X3 8u /* fp32 products as 3 bf16 partial products (2^-16 / product) */
 
 /*
  * C[dst(i), :] = A[src(i), :] @ W[r] for the rows i in [seg_ptr[r], seg_ptr[r+1]),
@@ -199,11 +200,13 @@ int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const floa
  * a negative src or dst skips the row.  A is [*, K] (row stride lda), W is
  * [R, K, N], C is [*, N] (row stride ldc), all fp32; seg_ptr is a device array of
  * R+1 row offsets (see cxg_rel_segment_*).  Computed with
- * v_mfma_f32_32x32x2_f32; with CXG_GEMM_SPLIT_BF16 (and K <= 128, K and lda
- * multiples of 4, A 16-byte aligned) every operand is split into two bf16 halves
- * and a*b is formed as hi*hi + lo*hi + hi*lo on v_mfma_f32_32x32x16_bf16 with
- * fp32 accumulation: relative error per product below 2^-16 (the reference's
- * tl.dot runs in TF32, 2^-11), HBM bound instead of matrix-core bound.  Replaces
+ * v_mfma_f32_32x32x2_f32; with CXG_GEMM_SPLIT_BF16X6 or _X3 (and K <= 128, K and
+ * lda multiples of 4, A 16-byte aligned) every operand is split into three (two)
+ * bf16 parts and a*b is accumulated in fp32 on v_mfma_f32_32x32x16_bf16 from the
+ * six (three) partial products whose magnitude is above 2^-24 (2^-16) of |ab|:
+ * X6 is as accurate as an fp32 FMA chain, X3 is off by at most 2^-16 per product
+ * (the reference's tl.dot runs in TF32, 2^-11); both are HBM bound instead of
+ * matrix-core bound.  Other shapes ignore the two flags.  Replaces
  * typed_matmul
  * (cxgnncomp/codegen/triton_typed_matmul.py:752-860: src_idx only = its
  * "single index" kernel with dst = src, seq_output = dst NULL, both = double

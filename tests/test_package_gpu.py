@@ -326,7 +326,10 @@ def test_rgcn_conv_layer():
     ref.backward(g.double())
     assert_close(_np(out), ref.detach().numpy(), RTOL, 2 * ATOL, "rgcn conv fwd")
     assert_close(_np(xg.grad), x64.grad.numpy(), RTOL, 2 * ATOL, "rgcn conv grad x")
-    assert len(layer.preprocessed) == 4
+    w64 = w.double().requires_grad_(True)
+    (pyref.typed_linear_s2d_sort(x.double(), w64, ptr, idx, etype, n) / deg).backward(g.double())
+    sc = float(w64.grad.abs().max())
+    assert_close(_np(layer.linear.grad) / sc, w64.grad.numpy() / sc, RTOL, 2 * ATOL, "rgcn conv grad w")
 
 
 def test_schedule_helpers_on_gpu_tensors():

@@ -1,12 +1,13 @@
 """Typed GEMM (MFMA), relation segmentation, pad_rel and the fused RGCN op
 through cxgnncomp_backend vs the oracle.
 
-Every fp32 test runs twice: with the exact fp32 MFMA kernel ("fp32": 1e-4
-relative / 1e-5 absolute at O(1) output scale) and with the default three-way
-bf16 split ("split": operands keep 16 significant bits and the lo*lo partial
-product is dropped, so each product is off by at most 3 * 2^-18 = 1.1e-5
-relative; over K <= 256 terms of an O(1) row that is 1e-4 relative / 4e-5
-absolute, stated here and checked below).
+Every fp32 test runs three times: with the fp32 MFMA kernel ("fp32") and with
+the default six-product bf16 split ("split6", fp32-accurate) at 1e-4 relative /
+1e-5 absolute at O(1) output scale, and with the three-product split ("split3":
+operands keep 16 significant bits and the lo*lo product is dropped, so each
+product is off by at most 3 * 2^-18 = 1.1e-5 relative; over K <= 256 terms of
+an O(1) row that is 1e-4 relative / 4e-5 absolute, stated here and checked
+below).
 bf16 MFMA path (stated tolerance): operands are rounded to bf16 (8 significant
 bits), products accumulate in fp32; against the oracle run on the same
 bf16-rounded operands the bound is the fp32 one, against the unrounded fp32
@@ -22,14 +23,14 @@ pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-4, 1e-5
 
 
-@pytest.fixture(autouse=True, params=["fp32", "split"])
+@pytest.fixture(autouse=True, params=["fp32", "split6", "split3"])
 def gemm_precision(request):
     """Runs every test of this file under both multiplication modes; ATOL follows."""
     from cxgnncomp_backend import _typed
     global ATOL
     old = _typed.GEMM_PRECISION
     _typed.GEMM_PRECISION = request.param
-    ATOL = 1e-5 if request.param == "fp32" else 4e-5
+    ATOL = 4e-5 if request.param == "split3" else 1e-5
     yield request.param
     _typed.GEMM_PRECISION = old
     ATOL = 1e-5
@@ -164,10 +165,15 @@ def test_rgcn_fused_toy_all_ones():
     assert torch.all(out.cpu() == 3968.0)
 
 
+@pytest.mark.parametrize("strategy", ["transform_first", "gather_gemm_scatter"])
 @pytest.mark.parametrize("K,N,R", [(128, 128, 16), (64, 32, 3)])
-def test_rgcn_fused_forward_backward(K, N, R):
+def test_rgcn_fused_forward_backward(K, N, R, strategy, monkeypatch):
     import cxgnncomp_backend as B
     from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _typed
+    if strategy == "gather_gemm_scatter":
+        monkeypatch.setattr(_typed, "RGCN_DENSE_MAX_BYTES", 0)    # rules the dense path out
+    assert _typed._use_dense(40000, 3000, R, N) == (strategy == "transform_first")
     ptr, idx, etype, _ = S.hetero_graph(3000, 40000, num_rel=R, seed=4)
     n = ptr.shape[0] - 1
     torch.manual_seed(14)
@@ -177,7 +183,7 @@ def test_rgcn_fused_forward_backward(K, N, R):
     xg = x.cuda().requires_grad_(True)
     wg = w.cuda().requires_grad_(True)
     rel = etype.int()
-    announce("aggr_rel_direct K=%d N=%d R=%d" % (K, N, R))
+    announce("aggr_rel_direct K=%d N=%d R=%d %s" % (K, N, R, strategy))
     out = B.aggr_rel_direct(xg, ptr.cuda(), idx.cuda(), wg, rel.cuda(), n, R)
     out.backward(g.cuda())
     torch.cuda.synchronize()
