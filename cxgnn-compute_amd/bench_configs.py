@@ -6,7 +6,15 @@ has in each configuration, as milliseconds, effective GB/s (algorithmic bytes of
 the gather model / time), GFLOP/s and fraction of the 8 TB/s HBM peak (or of the
 matrix-core peak for the typed GEMM).
 
-Usage: python bench_configs.py [--configs c1,c2,c3,c4,c5] [--iters 10]
+Timing: HIP events around every call; ``ms`` is the median of the timed calls,
+``p20_ms`` / ``p80_ms`` the spread.  ``--cold`` overwrites a 1 GiB buffer before
+every timed call so that nothing of the previous call is left in the L2 or the
+256 MB last-level cache; the default is warm (back-to-back calls).
+``--cpu-baseline`` adds, per configuration, the same ops in plain PyTorch on the
+host cores (the restatements of the reference's own PyTorch paths kept with the
+CPU oracle), on bounded samples of the same graphs.
+
+Usage: python bench_configs.py [--configs c1,c2,c3,c4,c5] [--iters 10] [--cold] [--cpu-baseline]
 """
 import argparse
 import json
@@ -23,21 +31,42 @@ MFMA_F32 = 157300.0   # GFLOP/s
 MFMA_BF16 = 2500000.0
 
 
+COLD = False
+CPU_BASELINE = False
+_flush = None
+_last_spread = None
+
+
 def timeit(fn, iters, warm=3):
+    """Median milliseconds of ``iters`` calls, each bracketed by its own HIP events."""
+    global _flush, _last_spread
     for _ in range(warm):
         fn()
+    if COLD and _flush is None:
+        _flush = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
     torch.cuda.synchronize()
-    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    s.record()
+    evs = []
     for _ in range(iters):
+        if COLD:
+            _flush.zero_()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
         fn()
-    e.record()
+        e.record()
+        evs.append((s, e))
     torch.cuda.synchronize()
-    return s.elapsed_time(e) / iters
+    ts = sorted(s.elapsed_time(e) for s, e in evs)
+    _last_spread = (ts[int(0.2 * (len(ts) - 1))], ts[int(round(0.8 * (len(ts) - 1)))])
+    return ts[len(ts) // 2]
 
 
 def report(cfg, op, ms, nbytes=None, flops=None, peak_flops=None, note=""):
+    global _last_spread
     rec = {"config": cfg, "op": op, "ms": round(ms, 4)}
+    if _last_spread is not None:
+        rec["p20_ms"], rec["p80_ms"] = round(_last_spread[0], 4), round(_last_spread[1], 4)
+        _last_spread = None
+    rec["cache"] = "cold" if COLD else "warm"
     if nbytes:
         gbs = nbytes / ms / 1e6
         rec["eff_GBps"] = round(gbs, 1)
@@ -49,6 +78,24 @@ def report(cfg, op, ms, nbytes=None, flops=None, peak_flops=None, note=""):
             rec["frac_mfma"] = round(gf / peak_flops, 4)
     if note:
         rec["note"] = note
+    print(json.dumps(rec), flush=True)
+
+
+def cpu_report(cfg, op, fn, sample, nbytes=None, repeats=3):
+    """One warm-up call and ``repeats`` timed calls of a host-side PyTorch restatement."""
+    import time
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    fn()
+    ts = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        fn()
+        ts.append((time.perf_counter() - t0) * 1e3)
+    ms = sorted(ts)[len(ts) // 2]
+    rec = {"config": cfg, "op": op, "cpu_ms": round(ms, 3), "cores": cores, "sample": sample}
+    if nbytes:
+        rec["cpu_eff_GBps"] = round(nbytes / ms / 1e6, 2)
     print(json.dumps(rec), flush=True)
 
 
@@ -81,10 +128,22 @@ def bench_aggregation(cfg, ptr, idx, n_dst, n_src, feat, iters, weighted=True):
                spmm_bytes(n_src, E, feat, 1) + 8 * E, 2 * E * feat)
 
 
+def cpu_spmm(cfg, ptr, idx, n_src, feat, rows):
+    """torch.sparse.mm on the first ``rows`` rows (cxgnncomp/codegen/torch_spmm.py:4-9)."""
+    from oracle import pyref
+    p, i = ptr[:rows + 1].cpu(), idx[:int(ptr[rows])].cpu()
+    x = torch.randn(n_src, feat)
+    e = int(p[-1])
+    cpu_report(cfg, "spmm_sum_fwd F=%d torch.sparse.mm" % feat, lambda: pyref.spmm_torch(x, p, i, rows),
+               "first %d rows, %d edges" % (rows, e), spmm_bytes(rows, e, feat))
+
+
 def c1(iters):
     from cxgnncomp import synthetic as S
     ptr, idx = S.uniform_graph(10000, 100000, device="cuda")
     bench_aggregation("c1", ptr, idx, 10000, 10000, 64, iters)
+    if CPU_BASELINE:
+        cpu_spmm("c1", ptr, idx, 10000, 64, 10000)
 
 
 def c2(iters):
@@ -92,6 +151,8 @@ def c2(iters):
     ptr, idx = S.powerlaw_directed_symmetrised(169343, 1166243, device="cuda")
     for f in (128, 256):
         bench_aggregation("c2", ptr, idx, 169343, 169343, f, iters)
+        if CPU_BASELINE:
+            cpu_spmm("c2", ptr, idx, 169343, f, 169343)
 
 
 def c3(iters):
@@ -131,6 +192,21 @@ def c3(iters):
     report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),
            E * (8 * H * C + 16) + 4 * E * H, 2 * E * H * C)
     del x, g
+    if CPU_BASELINE:
+        from oracle import pyref
+        cpu_spmm("c3", ptr, idx, N, 128, N // 8)
+        rows = N // 16
+        p, i = ptr[:rows + 1].cpu(), idx[:int(ptr[rows])].cpu()
+        e = int(p[-1])
+        a_s, a_d = att_s.cpu(), att_d.cpu()[:rows]
+        cpu_report("c3", "edge_softmax_fwd H=4 op-wise torch",
+                   lambda: pyref.edge_softmax_opwise(p, i, a_s, a_d, e, 0.2), "first %d rows, %d edges" % (rows, e),
+                   e * (8 + 4 * H) + 5 * e * H + 4 * rows * H + 8 * (rows + 1))
+        ne = 1 << 20
+        xs, gs = torch.randn(N, H, C) / 8, torch.randn(rows, H, C) / 8
+        d = torch.repeat_interleave(torch.arange(rows), p[1:] - p[:-1])[:ne]
+        cpu_report("c3", "sddmm H=4 C=64 gathered einsum", lambda: pyref.sddmm_einsum(i[:ne], d, xs, gs),
+                   "first %d edges" % ne, ne * (8 * H * C + 16) + 4 * ne * H)
 
 
 def c4(iters):
@@ -180,8 +256,11 @@ def c4(iters):
            timeit(lambda: _typed.typed_gemm(xe16, w, seg, E, out=oe, bf16=True), iters),
            E * 6 * K + 2 * R * K * K, flops, MFMA_BF16)
     del xe, oe, xe16
+    global _last_spread
+    t_mm = (E / N) * timeit(lambda: torch.mm(x, w[0]), iters)
+    _last_spread = tuple((E / N) * v for v in _last_spread)
     report("c4", "torch.mm [1M,128]x[128,128] x 20 (library GEMM of the same flops, no gather, for scale)",
-           (E / N) * timeit(lambda: torch.mm(x, w[0]), iters), E * 8 * K, flops, MFMA_F32)
+           t_mm, E * 8 * K, flops, MFMA_F32)
     layer = cxgnncomp.MyRGCNConv(K, K, R).cuda()
     xg = x.clone().requires_grad_(True)
 
@@ -189,7 +268,16 @@ def c4(iters):
         xg.grad = None
         o = layer(xg, ptr, idx, etype, N)
         o.sum().backward()
-    report("c4", "MyRGCNConv layer fwd+bwd (gather, typed GEMM, aggregate, /deg)", timeit(layer_step, max(2, iters // 3)))
+    report("c4", "MyRGCNConv layer fwd+bwd (typed transform, relational aggregate, /deg)",
+           timeit(layer_step, max(2, iters // 3)))
+    if CPU_BASELINE:
+        from oracle import pyref
+        rows = N // 32
+        p, i, t = ptr[:rows + 1].cpu(), idx[:int(ptr[rows])].cpu(), etype[:int(ptr[rows])].cpu()
+        xc, wc = x.cpu(), w.cpu()
+        cpu_report("c4", "rgcn forward, relation-sorted torch (TypedLinearS2DSort)",
+                   lambda: pyref.typed_linear_s2d_sort(xc, wc, p, i, t, rows),
+                   "first %d rows, %d edges" % (rows, int(p[-1])))
 
 
 def c5(iters):
@@ -215,13 +303,20 @@ def c5(iters):
                 h = torch.relu(h)
         h.sum().backward()
     report("c5", "3-layer SAGE fwd+bwd per batch (%s nodes per layer)" % nn, timeit(batch_step, iters))
+    if CPU_BASELINE:
+        cpu_spmm("c5", ptr, idx, n_src, 128, nn[2])
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
     ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--cold", action="store_true", help="flush the caches before every timed call")
+    ap.add_argument("--cpu-baseline", action="store_true", help="also time the host-side PyTorch restatements")
     args = ap.parse_args()
+    global COLD, CPU_BASELINE
+    COLD, CPU_BASELINE = args.cold, args.cpu_baseline
+    sys.path.insert(0, os.path.dirname(HERE))
     table = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5}
     for name in args.configs.split(","):
         table[name](args.iters)

@@ -449,7 +449,7 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3)) && K <= 128 && (K & 3) == 0 && (lda & 3) == 0 &&
       ((uintptr_t)a & 15) == 0) {
     // 64*G rows per block: up to 32 tiles while the launch keeps a few thousand blocks
-    int G = (int)(M / ((int64_t)cxg::kBM * 4096));
+    int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));
     G = G < 1 ? 1 : (G > 32 ? 32 : G);
     const int64_t n_blocks = (cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R) * cxg::ceil_div(N, 128);
     CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
