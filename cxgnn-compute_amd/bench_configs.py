@@ -192,6 +192,18 @@ def c3(iters):
     report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),
            E * (8 * H * C + 16) + 4 * E * H, 2 * E * H * C)
     del x, g
+    # scheduling helpers (index work): bytes = arrays read + written once
+    import cxgnncomp
+    new_ptr, _ = cxgnncomp.neighbor_grouping(ptr, 32)
+    n_groups = new_ptr.shape[0] - 1
+    report("c3", "neighbor_grouping thres=32 (%d groups)" % n_groups,
+           timeit(lambda: cxgnncomp.neighbor_grouping(ptr, 32), iters), 8 * (N + 1) * 2 + 16 * n_groups)
+    eflag = torch.rand(E, device="cuda") < 0.5
+    report("c3", "remove_from_graph_by_edge (half of the edges flagged)",
+           timeit(lambda: cxgnncomp.remove_from_graph_by_edge(ptr, idx, eflag), iters),
+           E * (1 + 8 + 8) + 8 * E // 2 + 8 * 3 * N)
+    report("c3", "csr transpose (stable sort by source + fills)",
+           timeit(lambda: _ops.csr_transpose(ptr, idx, N, N), max(2, iters // 4)), E * 8 * 4 + 16 * N)
     if CPU_BASELINE:
         from oracle import pyref
         cpu_spmm("c3", ptr, idx, N, 128, N // 8)
@@ -226,6 +238,9 @@ def c4(iters):
     flops = 2.0 * E * K * K
     fused_bytes = E * (4 * K + 8 + 8 + 4 * K) + 4 * R * K * K
     report("c4", "rel_segment (stable sort by relation)", timeit(lambda: _typed.rel_segment(rel32, R), iters))
+    layers = torch.tensor([N // 100, N // 10, N, N])
+    report("c4", "rel_schedule (16 per-relation sub-graphs + layer table)",
+           timeit(lambda: B.rel_schedule(ptr, idx, rel32, layers, R), max(2, iters // 4)))
 
     def fused(precision):
         out.zero_()

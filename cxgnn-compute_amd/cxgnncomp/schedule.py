@@ -1,8 +1,11 @@
-"""Degree bucketing and row filtering of CSR graphs (cxgnncomp/schedule.py:6-144),
-as vectorised index arithmetic on the tensors' own device instead of Python loops
-over rows.  Results are identical to the upstream loops (bit-exact index work).
+"""Degree bucketing and row filtering of CSR graphs (cxgnncomp/schedule.py:6-144).
+Graphs on the GPU go through the library's scan + fill kernels; host tensors are
+handled with vectorised index arithmetic instead of upstream's Python loops over
+rows.  Results are identical to the upstream loops (bit-exact index work).
 """
 import torch
+
+from cxgnncomp_backend import _ops
 
 
 def _degrees(ptr):
@@ -23,6 +26,8 @@ def neighbor_grouping(ptr, neighbor_thres=32):
     if not isinstance(ptr, torch.Tensor):
         ptr = torch.as_tensor(ptr)
     ptr = ptr.to(torch.int64)
+    if ptr.is_cuda:
+        return _ops.neighbor_group(ptr.contiguous(), neighbor_thres)
     n = ptr.shape[0] - 1
     deg = _degrees(ptr)
     groups = torch.clamp((deg + neighbor_thres - 1) // neighbor_thres, min=1)
@@ -42,6 +47,8 @@ def neighbor_grouping_gpu(ptr, neighbor_thres=32):
 
 def remove_from_graph(ptr, idx, remove_flag):
     """Keep the rows whose flag is false (upstream :106-121)."""
+    if ptr.is_cuda:
+        return _ops.filter_rows(ptr, idx, remove_flag)
     keep = ~remove_flag.to(torch.bool)
     deg = _degrees(ptr)
     new_ptr = torch.cat([ptr[:1] * 0, torch.cumsum(deg[keep], 0)])
@@ -53,6 +60,8 @@ def remove_from_graph_by_edge(ptr, idx, remove_flag):
     """Drop flagged edges, then drop rows left without edges (upstream :124-144)."""
     assert remove_flag.shape == idx.shape, \
         f"remove_flag.shape != idx.shape {remove_flag.shape} {idx.shape}"
+    if ptr.is_cuda:
+        return _ops.filter_edges(ptr, idx, remove_flag)[:2]
     keep = ~remove_flag.to(torch.bool)
     n = ptr.shape[0] - 1
     rows = _row_of_edge(ptr)

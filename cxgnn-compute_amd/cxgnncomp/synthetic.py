@@ -21,6 +21,9 @@ def _gen(seed, device):
 
 def csr_from_coo(src, dst, num_dst):
     """CSR by destination, edges of one destination kept in input order."""
+    if src.is_cuda:
+        from cxgnncomp_backend import _ops
+        return _ops.coo_to_csr(src.contiguous(), dst.contiguous(), num_dst)[:2]
     dst_sorted, order = torch.sort(dst, stable=True)
     idx = src[order].contiguous()
     counts = torch.bincount(dst_sorted, minlength=num_dst)

@@ -50,6 +50,15 @@ SIGNATURES = {
     "cxg_csr_row_ids_i64": (_I32, [_P, _I64, _I64, _P, _P]),
     "cxg_edge_value_degree_f32": (_I32, [_P, _I64, _P, _P]),
     "cxg_pad_rel_i64": (_I32, [_P, _P, _P, _I32, _I32, _I64, _P]),
+    "cxg_scan_workspace_bytes": (_SZ, [_I64]),
+    "cxg_neighbor_group_plan_i64": (_I32, [_P, _I64, _I64, _P, _P, _SZ, _P]),
+    "cxg_neighbor_group_fill_i64": (_I32, [_P, _P, _I64, _I64, _I64, _P, _P, _P]),
+    "cxg_filter_rows_plan_i64": (_I32, [_P, _I64, _P, _P, _P, _P, _SZ, _P]),
+    "cxg_filter_rows_fill_i64": (_I32, [_P, _P, _I64, _P, _P, _I64, _P, _P, _P]),
+    "cxg_filter_edges_plan_i64": (_I32, [_P, _I64, _I64, _P, _P, _I32, _P, _P, _P, _SZ, _P]),
+    "cxg_filter_edges_fill_i64": (_I32, [_P, _P, _I64, _I64, _P, _P, _P, _P, _P, _P]),
+    "cxg_coo_to_csr_workspace_bytes": (_SZ, [_I64, _I64]),
+    "cxg_coo_to_csr_i64": (_I32, [_P, _P, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
 }
 
 _lib = None

@@ -383,3 +383,114 @@ def gather_rows(inp, sel):
                                      inp.shape[1], _lib.current_stream(inp.device))
     _lib.check(st)
     return out
+
+
+# --------------------------------------------------------------------------- #
+# scheduling helpers as device index work
+# --------------------------------------------------------------------------- #
+def _scan_ws(lib, n, dev):
+    return _workspace(lib.cxg_scan_workspace_bytes(int(n)), dev)
+
+
+def neighbor_group(ptr, thres):
+    """(new_ptr, new_target) of cxg_neighbor_group_*: rows cut into chunks of ``thres`` edges."""
+    lib = _lib.load()
+    _req(ptr, "ptr", torch.int64, 1)
+    dev, n = ptr.device, ptr.shape[0] - 1
+    off = torch.empty(n + 1, dtype=torch.int64, device=dev)
+    ws = _scan_ws(lib, n, dev)
+    with torch.cuda.device(dev):
+        stream = _lib.current_stream(dev)
+        _lib.check(lib.cxg_neighbor_group_plan_i64(ptr.data_ptr(), n, int(thres), off.data_ptr(),
+                                                   ws.data_ptr(), ws.numel(), stream))
+        n_groups = int(off[n].item())
+        new_ptr = torch.empty(n_groups + 1, dtype=torch.int64, device=dev)
+        new_target = torch.empty(n_groups, dtype=torch.int64, device=dev)
+        _lib.check(lib.cxg_neighbor_group_fill_i64(ptr.data_ptr(), off.data_ptr(), n, int(thres), n_groups,
+                                                   new_ptr.data_ptr(), _lib.ptr(new_target), stream))
+    return new_ptr, new_target
+
+
+def filter_rows(ptr, idx, remove_flag):
+    """Keep the rows whose flag is false: (new_ptr, new_idx)."""
+    lib = _lib.load()
+    n = ptr.shape[0] - 1
+    _check_graph(ptr, idx, n)
+    flag = remove_flag.to(torch.uint8).contiguous()
+    if flag.shape[0] < n or flag.device != ptr.device:
+        raise ValueError("remove_flag must have one entry per row on the graph's device")
+    dev = ptr.device
+    row_off = torch.empty(n + 1, dtype=torch.int64, device=dev)
+    edge_off = torch.empty(n + 1, dtype=torch.int64, device=dev)
+    ws = _scan_ws(lib, n, dev)
+    with torch.cuda.device(dev):
+        stream = _lib.current_stream(dev)
+        _lib.check(lib.cxg_filter_rows_plan_i64(ptr.data_ptr(), n, _lib.ptr(flag), row_off.data_ptr(),
+                                                edge_off.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+        n_rows_out, n_edges_out = int(row_off[n].item()), int(edge_off[n].item())
+        new_ptr = torch.empty(n_rows_out + 1, dtype=torch.int64, device=dev)
+        new_idx = torch.empty(n_edges_out, dtype=torch.int64, device=dev)
+        _lib.check(lib.cxg_filter_rows_fill_i64(ptr.data_ptr(), _lib.ptr(idx), n, row_off.data_ptr(),
+                                                edge_off.data_ptr(), n_edges_out, new_ptr.data_ptr(),
+                                                _lib.ptr(new_idx), stream))
+    return new_ptr, new_idx
+
+
+def filter_edges(ptr, idx, remove_flag=None, rel=None, keep_rel=0, want_target=False):
+    """Keep edge e if ``rel[e] == keep_rel`` (rel given) or ``not remove_flag[e]``, drop the
+    rows left empty.  Returns (new_ptr, new_idx, new_target or None, row_off); row_off[i]
+    is the number of kept rows among the first i rows."""
+    lib = _lib.load()
+    n = ptr.shape[0] - 1
+    _check_graph(ptr, idx, n)
+    dev = ptr.device
+    n_edges = int(ptr[n].item())
+    if int(ptr[0].item()) != 0:
+        raise ValueError("ptr[0] must be 0")
+    if idx.shape[0] < n_edges:
+        raise ValueError("idx shorter than ptr[-1]")
+    flag = None
+    if rel is not None:
+        _req(rel, "rel", torch.int32, 1)
+        if rel.shape[0] < n_edges:
+            raise ValueError("rel shorter than the number of edges")
+    else:
+        flag = remove_flag.to(torch.uint8).contiguous()
+        if flag.shape[0] < n_edges or flag.device != dev:
+            raise ValueError("remove_flag must have one entry per edge on the graph's device")
+    edge_pos = torch.empty(n_edges + 1, dtype=torch.int64, device=dev)
+    row_off = torch.empty(n + 1, dtype=torch.int64, device=dev)
+    ws = _scan_ws(lib, max(n, n_edges), dev)
+    with torch.cuda.device(dev):
+        stream = _lib.current_stream(dev)
+        _lib.check(lib.cxg_filter_edges_plan_i64(ptr.data_ptr(), n, n_edges, _lib.ptr(flag), _lib.ptr(rel),
+                                                 int(keep_rel), edge_pos.data_ptr(), row_off.data_ptr(),
+                                                 ws.data_ptr(), ws.numel(), stream))
+        n_rows_out, n_edges_out = int(row_off[n].item()), int(edge_pos[n_edges].item())
+        new_ptr = torch.empty(n_rows_out + 1, dtype=torch.int64, device=dev)
+        new_idx = torch.empty(n_edges_out, dtype=torch.int64, device=dev)
+        new_target = torch.empty(n_rows_out, dtype=torch.int64, device=dev) if want_target else None
+        _lib.check(lib.cxg_filter_edges_fill_i64(ptr.data_ptr(), _lib.ptr(idx), n, n_edges, edge_pos.data_ptr(),
+                                                 row_off.data_ptr(), new_ptr.data_ptr(), _lib.ptr(new_idx),
+                                                 _lib.ptr(new_target), stream))
+    return new_ptr, new_idx, new_target, row_off
+
+
+def coo_to_csr(src, dst, n_rows):
+    """CSR by destination of the edge list (src, dst), stable: (ptr, idx, perm)."""
+    lib = _lib.load()
+    _req(src, "src", torch.int64, 1)
+    _req(dst, "dst", torch.int64, 1)
+    if src.shape != dst.shape or src.device != dst.device:
+        raise ValueError("src and dst must have the same length and device")
+    dev, e = src.device, src.shape[0]
+    if e and (int(dst.min()) < 0 or int(dst.max()) >= n_rows):
+        raise ValueError("destination ids must lie in [0, %d)" % n_rows)
+    ptr = torch.empty(n_rows + 1, dtype=torch.int64, device=dev)
+    idx = torch.empty(e, dtype=torch.int64, device=dev)
+    perm = torch.empty(e, dtype=torch.int64, device=dev)
+    ws = _workspace(lib.cxg_coo_to_csr_workspace_bytes(e, n_rows), dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.cxg_coo_to_csr_i64(_lib.ptr(src), _lib.ptr(dst), e, n_rows, ptr.data_ptr(), _lib.ptr(idx),
+                                          _lib.ptr(perm), ws.data_ptr(), ws.numel(), _lib.current_stream(dev)))
+    return ptr, idx, perm

@@ -18,9 +18,12 @@ def rel_schedule(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel):
     target_r (original row ids); then a [num_rel, L] table, L = len(num_node_in_layer)-1,
     whose entry [r, l] is the number of kept rows among the first num_node_in_layer[l]
     rows.  Returns the 3*num_rel + 1 tensors in that order, on the inputs' device
-    (upstream works on CPU tensors)."""
+    (upstream works on CPU tensors); graphs on the GPU use the library's edge filter
+    once per relation."""
     n = csr_ptr.shape[0] - 1
     num_rel = int(num_rel)
+    if csr_ptr.is_cuda:
+        return _rel_schedule_device(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel, n)
     rows = _rows_of_edges(csr_ptr, n)
     e = rows.shape[0]
     idx = csr_idx[:e]
@@ -46,6 +49,32 @@ def rel_schedule(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel):
                 break
             table[r, l] = kept_before[i]
             pos = i
+    out.append(table)
+    return out
+
+
+def _rel_schedule_device(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel, n):
+    layers = [int(v) for v in num_node_in_layer.tolist()]
+    num_layer = len(layers) - 1
+    # upstream walks rows in order and records layer l when it reaches row
+    # num_node_in_layer[l]-1; a boundary that lies behind the walk is never met
+    reached, pos = [], -1
+    for l in range(num_layer):
+        i = layers[l] - 1
+        if i <= pos or i >= n:
+            break
+        reached.append(i + 1)
+        pos = i
+    at = torch.tensor(reached, dtype=torch.int64, device=csr_ptr.device)
+    table = torch.zeros((num_rel, max(num_layer, 0)), dtype=torch.int64, device=csr_ptr.device)
+    rel32 = rel.to(torch.int32).contiguous()
+    out = []
+    for r in range(num_rel):
+        sub_ptr, sub_idx, target, row_off = _ops.filter_edges(csr_ptr, csr_idx, rel=rel32, keep_rel=r,
+                                                              want_target=True)
+        out += [sub_ptr, sub_idx, target]
+        if reached:
+            table[r, :len(reached)] = row_off[at]
     out.append(table)
     return out
 

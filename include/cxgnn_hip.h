@@ -302,6 +302,76 @@ int cxg_edge_value_degree_f32(const int64_t* ptr, int64_t n_rows, float* out,
 int cxg_pad_rel_i64(int64_t* rel, int64_t* idx, const int64_t* count, int thres,
                     int num_rel, int64_t base, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* Scheduling helpers as device index work (bit-exact)                          */
+/* ------------------------------------------------------------------------- */
+/* Output sizes depend on the data: a "plan" call leaves exclusive-scan offsets
+ * on the device (n+1 entries; the last one is the output size, which the caller
+ * copies back to allocate the outputs), a "fill" call writes the outputs.      */
+
+/* Scratch bytes for the plan calls on arrays of up to n elements. */
+size_t cxg_scan_workspace_bytes(int64_t n);
+
+/*
+ * Neighbor grouping (degree bucketing): every row is cut into consecutive chunks
+ * of `thres` edges, the last chunk holds the remainder, an empty row gives one
+ * empty chunk.  plan: group_off[r] = number of chunks of rows < r (n_rows+1
+ * entries).  fill: new_ptr[n_groups+1] (new_ptr[0] = 0, then the chunk ends as
+ * positions in idx) and new_target[g] = row of chunk g.  Replaces
+ * neighbor_grouping / neighbor_grouping_gpu (cxgnncomp/schedule.py:6-35).
+ */
+int cxg_neighbor_group_plan_i64(const int64_t* ptr, int64_t n_rows, int64_t thres,
+                                int64_t* group_off, void* workspace, size_t workspace_bytes,
+                                void* stream);
+int cxg_neighbor_group_fill_i64(const int64_t* ptr, const int64_t* group_off, int64_t n_rows,
+                                int64_t thres, int64_t n_groups, int64_t* new_ptr,
+                                int64_t* new_target, void* stream);
+
+/*
+ * Row filter: keep the rows r with remove_flag[r] == 0, edges unchanged.
+ * plan: row_off / edge_off = kept rows / kept edges before row r (n_rows+1
+ * entries each).  fill: new_ptr[row_off[n_rows]+1], new_idx[edge_off[n_rows]].
+ * Replaces remove_from_graph (cxgnncomp/schedule.py:106-121).
+ */
+int cxg_filter_rows_plan_i64(const int64_t* ptr, int64_t n_rows, const uint8_t* remove_flag,
+                             int64_t* row_off, int64_t* edge_off, void* workspace,
+                             size_t workspace_bytes, void* stream);
+int cxg_filter_rows_fill_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows,
+                             const int64_t* row_off, const int64_t* edge_off,
+                             int64_t n_edges_out, int64_t* new_ptr, int64_t* new_idx,
+                             void* stream);
+
+/*
+ * Edge filter: keep edge e if rel ? rel[e] == keep_rel : !remove_flag[e], then
+ * drop the rows left without edges; edge order is preserved.  ptr[0] must be 0
+ * and ptr[n_rows] == n_edges.  plan: edge_pos (n_edges+1) = kept edges before e,
+ * row_off (n_rows+1) = kept rows before r.  fill: new_ptr[row_off[n_rows]+1],
+ * new_idx[edge_pos[n_edges]] and, if not NULL, new_target[k] = original id of
+ * kept row k.  Replaces remove_from_graph_by_edge (cxgnncomp/schedule.py:124-144)
+ * and, called once per relation with rel/keep_rel, the per-relation sub-graphs
+ * (ptr_r, idx_r, target_r) of rel_schedule (src/cpp/src/schedule.cu:5-63); the
+ * cumulative row counts of its layer table are entries of row_off.
+ */
+int cxg_filter_edges_plan_i64(const int64_t* ptr, int64_t n_rows, int64_t n_edges,
+                              const uint8_t* remove_flag, const int32_t* rel, int32_t keep_rel,
+                              int64_t* edge_pos, int64_t* row_off, void* workspace,
+                              size_t workspace_bytes, void* stream);
+int cxg_filter_edges_fill_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows,
+                              int64_t n_edges, const int64_t* edge_pos, const int64_t* row_off,
+                              int64_t* new_ptr, int64_t* new_idx, int64_t* new_target,
+                              void* stream);
+
+/*
+ * COO -> CSR by destination: edges sorted by dst (stable: edges of one
+ * destination keep their input order), ptr[n_rows+1], idx = src in that order,
+ * perm[k] = input position of the k-th CSR edge.  The relation the reference
+ * builds in cxgnncomp/data_preparation.py:97-104.
+ */
+size_t cxg_coo_to_csr_workspace_bytes(int64_t n_edges, int64_t n_rows);
+int cxg_coo_to_csr_i64(const int64_t* src, const int64_t* dst, int64_t n_edges, int64_t n_rows,
+                       int64_t* ptr, int64_t* idx, int64_t* perm, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,130 @@
+"""Scheduling helpers on the GPU (neighbor grouping, row / edge filters, the
+per-relation sub-graphs of rel_schedule, COO -> CSR) against the CPU oracle:
+index work, so every comparison is bit-exact.  Edge cases: empty graph, empty
+rows, thresholds 1 and larger than any degree, everything removed, nothing
+removed, relations that never occur, layer boundaries the reference's walk never
+reaches.  A benchmark-sized case checks the invariants the outputs must satisfy."""
+import io
+from contextlib import redirect_stdout
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import announce
+from oracle import pyref
+
+pytestmark = pytest.mark.gpu
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+def _random_ptr(rng, n, hi):
+    deg = rng.integers(0, hi, n)
+    deg[::6] = 0
+    return np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+
+
+@pytest.mark.parametrize("n,hi", [(0, 5), (1, 1), (1, 9), (500, 120), (20000, 40)])
+@pytest.mark.parametrize("thres", [1, 4, 32, 1000])
+def test_neighbor_grouping_bit_exact(n, hi, thres):
+    import cxgnncomp
+    rng = np.random.default_rng(n + thres)
+    ptr = _random_ptr(rng, n, hi)
+    want_ptr, want_target = oracle.neighbor_grouping(ptr, thres)
+    announce("neighbor_grouping n=%d thres=%d" % (n, thres))
+    got_ptr, got_target = cxgnncomp.neighbor_grouping(torch.from_numpy(ptr).cuda(), thres)
+    assert got_ptr.is_cuda and got_ptr.dtype == torch.int64 and got_target.dtype == torch.int64
+    assert np.array_equal(_np(got_ptr), want_ptr) and np.array_equal(_np(got_target), want_target)
+    assert np.array_equal(_np(cxgnncomp.neighbor_grouping_gpu(torch.from_numpy(ptr).cuda(), thres)), want_ptr)
+
+
+@pytest.mark.parametrize("n,hi,p", [(0, 3, 0.5), (1, 4, 0.0), (200, 15, 0.3), (200, 15, 1.0), (200, 15, 0.0),
+                                    (30000, 30, 0.5)])
+def test_row_and_edge_filters_bit_exact(n, hi, p):
+    import cxgnncomp
+    rng = np.random.default_rng(n + int(10 * p))
+    ptr = _random_ptr(rng, n, hi)
+    E = int(ptr[-1])
+    idx = rng.integers(0, 1000, E)
+    tp, ti = torch.from_numpy(ptr).cuda(), torch.from_numpy(idx).cuda()
+    flag = rng.random(n) < p
+    with redirect_stdout(io.StringIO()):
+        want = pyref.remove_from_graph(ptr, idx, flag)
+    announce("remove_from_graph n=%d p=%.1f" % (n, p))
+    got = cxgnncomp.remove_from_graph(tp, ti, torch.from_numpy(flag).cuda())
+    assert np.array_equal(_np(got[0]), want[0]) and np.array_equal(_np(got[1]), want[1])
+    eflag = rng.random(E) < p
+    want = pyref.remove_from_graph_by_edge(ptr, idx, eflag)
+    announce("remove_from_graph_by_edge n=%d p=%.1f" % (n, p))
+    got = cxgnncomp.remove_from_graph_by_edge(tp, ti, torch.from_numpy(eflag).cuda())
+    assert np.array_equal(_np(got[0]), want[0]) and np.array_equal(_np(got[1]), want[1])
+
+
+@pytest.mark.parametrize("layers", [[20, 70, 150, 150], [150, 150], [70, 20, 150], [10, 151, 150], [150]])
+def test_rel_schedule_bit_exact(layers):
+    import cxgnncomp_backend as B
+    rng = np.random.default_rng(4)
+    ptr = _random_ptr(rng, 150, 12)
+    E = int(ptr[-1])
+    idx = rng.integers(0, 400, E)
+    rel = rng.integers(0, 5, E).astype(np.int32)
+    rel[rel == 3] = 2                                   # relation 3 never occurs
+    want = oracle.rel_schedule(ptr, idx, rel, layers, 5)
+    announce("rel_schedule layers=%s" % layers)
+    got = B.rel_schedule(torch.from_numpy(ptr).cuda(), torch.from_numpy(idx).cuda(), torch.from_numpy(rel).cuda(),
+                         torch.tensor(layers), 5)
+    assert len(got) == len(want) == 16
+    for g, w in zip(got, want):
+        assert g.is_cuda and g.dtype == torch.int64 and np.array_equal(_np(g), w)
+
+
+@pytest.mark.parametrize("n,e", [(1, 0), (5, 1), (300, 4000), (100000, 1500000)])
+def test_coo_to_csr_bit_exact(n, e):
+    from cxgnncomp import synthetic
+    from cxgnncomp_backend import _ops
+    rng = np.random.default_rng(e)
+    src = rng.integers(0, 5 * n, e)
+    dst = rng.integers(0, n, e)
+    want_ptr, want_idx = oracle.coo_to_csr(src, dst, n)
+    announce("coo_to_csr n=%d e=%d" % (n, e))
+    ptr, idx, perm = _ops.coo_to_csr(torch.from_numpy(src).cuda(), torch.from_numpy(dst).cuda(), n)
+    assert np.array_equal(_np(ptr), want_ptr) and np.array_equal(_np(idx), want_idx)
+    assert np.array_equal(_np(perm), np.argsort(dst, kind="stable"))
+    p2, i2 = synthetic.csr_from_coo(torch.from_numpy(src).cuda(), torch.from_numpy(dst).cuda(), n)
+    assert torch.equal(p2, ptr) and torch.equal(i2, idx)
+    with pytest.raises(ValueError):
+        _ops.coo_to_csr(torch.tensor([0]).cuda(), torch.tensor([n]).cuda(), n)
+
+
+def test_schedule_helpers_at_benchmark_size():
+    """2.45M rows / 61.9M edges: the outputs' defining invariants, checked on the device."""
+    import cxgnncomp
+    from cxgnncomp import synthetic
+    N = 2449029
+    ptr, idx = synthetic.powerlaw_symmetric_graph(N, 30929570, device="cuda")
+    E = idx.shape[0]
+    deg = ptr[1:] - ptr[:-1]
+    announce("neighbor_grouping at 61.9M edges")
+    new_ptr, new_target = cxgnncomp.neighbor_grouping(ptr, 32)
+    sizes = new_ptr[1:] - new_ptr[:-1]
+    groups = torch.clamp((deg + 31) // 32, min=1)
+    assert int(new_ptr[0]) == 0 and int(new_ptr[-1]) == E and new_target.shape[0] == int(groups.sum())
+    assert int(sizes.max()) <= 32 and int(sizes.min()) >= 0
+    assert torch.equal(torch.bincount(new_target, minlength=N), groups)
+    assert bool((new_target[1:] >= new_target[:-1]).all())
+    assert torch.equal(torch.zeros(N, dtype=torch.int64, device="cuda").index_add_(0, new_target, sizes), deg)
+    announce("remove_from_graph_by_edge at 61.9M edges")
+    g = torch.Generator(device="cuda").manual_seed(3)
+    eflag = torch.rand(E, generator=g, device="cuda") < 0.7
+    p2, i2 = cxgnncomp.remove_from_graph_by_edge(ptr, idx, eflag)
+    assert torch.equal(i2, idx[~eflag]) and int(p2[-1]) == i2.shape[0]
+    assert bool(((p2[1:] - p2[:-1]) > 0).all())
+    announce("remove_from_graph at 61.9M edges")
+    rflag = torch.rand(N, generator=g, device="cuda") < 0.5
+    p3, i3 = cxgnncomp.remove_from_graph(ptr, idx, rflag)
+    assert torch.equal(p3[1:] - p3[:-1], deg[~rflag])
+    assert torch.equal(i3, idx[torch.repeat_interleave(~rflag, deg)])
