@@ -5,7 +5,7 @@ import enum
 
 import torch
 
-from . import _ops
+from . import _lib, _ops
 
 
 def _rows_of_edges(ptr, n):
@@ -118,24 +118,45 @@ class REDUCEOP(enum.IntEnum):
 
 
 class COMPUTEOP(enum.IntEnum):
+    """Names in the order the reference exports them (binding.cpp:114-119), values
+    of its C enum (dgsparse.h:14)."""
     ADD = 0
-    MUL = 1
-    DIV = 2
-    SUB = 3
+    MUL = 2
+    DIV = 3
+    SUB = 1
+
+
+def _gspmm(rowptr, colind, val, b, red, comp):
+    lib = _lib.load()
+    for t, name in ((rowptr, "A_rowptr"), (colind, "A_colind")):
+        _ops._req(t, name, torch.int32, 1)
+    _ops._req(b, "B", torch.float32, 2)
+    n = rowptr.shape[0] - 1
+    if val is not None:
+        _ops._req(val, "A_csrVal", torch.float32, 1)
+        if val.shape[0] < colind.shape[0]:
+            raise ValueError("A_csrVal shorter than A_colind")
+    out = torch.empty((n, b.shape[1]), dtype=torch.float32, device=b.device)
+    with torch.cuda.device(b.device):
+        st = lib.cxg_gspmm_i32_f32(rowptr.data_ptr(), _lib.ptr(colind), _lib.ptr(val), _lib.ptr(b), _lib.ptr(out),
+                                   n, b.shape[1], int(red), int(comp), _lib.current_stream(b.device))
+    _lib.check(st)
+    return out
 
 
 def GSpMM_u(A_rowptr, A_colind, B, op):
-    """int32-CSR SpMM without edge values (binding.cpp:97-104); SUM and MEAN."""
+    """int32-CSR SpMM without edge values (binding.cpp:97-104): sum / max / min / mean of
+    the gathered rows; empty rows give 0."""
     op = REDUCEOP(int(op))
-    if op not in (REDUCEOP.SUM, REDUCEOP.MEAN):
-        raise NotImplementedError("GSpMM_u supports SUM and MEAN")
     if A_rowptr.dtype != torch.int32 or A_colind.dtype != torch.int32:
         raise ValueError("GSpMM_u takes int32 rowptr/colind")
-    return _ops.spmm(A_rowptr, A_colind, B, A_rowptr.shape[0] - 1, mean=(op == REDUCEOP.MEAN))
+    if op in (REDUCEOP.SUM, REDUCEOP.MEAN):
+        return _ops.spmm(A_rowptr, A_colind, B, A_rowptr.shape[0] - 1, mean=(op == REDUCEOP.MEAN))
+    return _gspmm(A_rowptr, A_colind, None, B, op, COMPUTEOP.MUL)
 
 
 def GSpMM_u_e(A_rowptr, A_colind, A_csrVal, B, re_op, comp_op):
-    """int32-CSR SpMM with edge values (binding.cpp:86-95); SUM of MUL."""
-    if REDUCEOP(int(re_op)) != REDUCEOP.SUM or COMPUTEOP(int(comp_op)) != COMPUTEOP.MUL:
-        raise NotImplementedError("GSpMM_u_e supports REDUCEOP.SUM with COMPUTEOP.MUL")
-    return _ops.spmm(A_rowptr.long(), A_colind.long(), B, A_rowptr.shape[0] - 1, val=A_csrVal)
+    """int32-CSR SpMM with edge values (binding.cpp:86-95):
+    out[r] = REDUCE_e COMPUTE(val[e], B[col[e]]) with COMPUTE add val+b, sub b-val,
+    mul val*b, div b/val (dgsparse.h:53-79)."""
+    return _gspmm(A_rowptr, A_colind, A_csrVal, B, REDUCEOP(int(re_op)), COMPUTEOP(int(comp_op)))

@@ -302,6 +302,20 @@ int cxg_edge_value_degree_f32(const int64_t* ptr, int64_t n_rows, float* out,
 int cxg_pad_rel_i64(int64_t* rel, int64_t* idx, const int64_t* count, int thres,
                     int num_rel, int64_t base, void* stream);
 
+/*
+ * Generalised CSR SpMM with int32 indices:
+ *   out[r, c] = REDUCE_{e in row r} COMPUTE(val[e], b[colind[e], c]),  out [n_rows, feat].
+ * reduce_op: 0 sum, 1 max, 2 min, 3 mean; compute_op: 0 val+b, 1 b-val, 2 val*b,
+ * 3 b/val (the enum values of src/cpp/include/dgsparse.h:13-14); val == NULL: the
+ * operand is b itself and compute_op is ignored.  A non-empty row's accumulator
+ * starts at 0 / (float)INT_MIN / (float)INT_MAX / 0, empty rows give 0, mean
+ * divides by the row length.  Replaces GSpMM_u / GSpMM_u_e
+ * (src/cpp/python_bindings/binding.cpp:87-107, src/cpp/src/dgsparse.cu:444-474).
+ */
+int cxg_gspmm_i32_f32(const int32_t* rowptr, const int32_t* colind, const float* val,
+                      const float* b, float* out, int64_t n_rows, int feat, int reduce_op,
+                      int compute_op, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Scheduling helpers as device index work (bit-exact)                          */
 /* ------------------------------------------------------------------------- */

@@ -176,6 +176,18 @@ def spmv(ptr, idx, x, n_dst):
     return out
 
 
+def gspmm(rowptr, colind, b, red, comp=2, val=None):
+    """dgSPARSE-style generalised SpMM; red 0 sum / 1 max / 2 min / 3 mean,
+    comp 0 add / 1 sub / 2 mul / 3 div (the C enum values of dgsparse.h:13-14)."""
+    rowptr, colind, b = _i32(rowptr), _i32(colind), _f32(b)
+    val = None if val is None else _f32(val)
+    n = rowptr.shape[0] - 1
+    out = np.zeros((n, b.shape[1]), dtype=np.float32)
+    _load().orc_gspmm(_p(rowptr), _p(colind), _p(val), _p(b), _p(out), _L(n), _I(b.shape[1]), _I(int(red)),
+                      _I(int(comp)))
+    return out
+
+
 def gather_fwd(x, dest, n_nodes):
     x, dest = _f32(x), _i64(dest)
     out = np.zeros((n_nodes, x.shape[1]), dtype=np.float32)

@@ -233,6 +233,40 @@ void orc_spmv(const Index* ptr, const Index* idx, const float* in, float* out, I
 }
 
 /* ------------------------------------------------------------------------- */
+/* GSpMM_u / GSpMM_u_e: generalised CSR SpMM of the dgSPARSE kernels           */
+/* src/cpp/include/dgsparse.h:14-131, src/cpp/src/dgsparse.cu:6-125,444-474:   */
+/*   out[r,c] = REDUCE_{e in row r} COMPUTE(val[e], b[col[e], c]);             */
+/*   REDUCE 0 sum, 1 max, 2 min, 3 mean; COMPUTE 0 val+b, 1 b-val, 2 val*b,    */
+/*   3 b/val (dgsparse.h:13-14,53-79); val == NULL: the operand is b itself.   */
+/*   The accumulator of a non-empty row starts at init(op): 0, (float)INT_MIN, */
+/*   (float)INT_MAX, 0 (dgsparse.h:117-130); empty rows give 0                 */
+/*   (dgsparse.cu:23-24); mean divides by the row length.  int32 indices.      */
+/* ------------------------------------------------------------------------- */
+void orc_gspmm(const int32_t* rowptr, const int32_t* colind, const float* val, const float* b,
+               float* out, Index n_rows, int feat, int red, int comp) {
+  for (Index r = 0; r < n_rows; ++r) {
+    const int lb = rowptr[r], hb = rowptr[r + 1];
+    for (int c = 0; c < feat; ++c) {
+      if (hb <= lb) { out[r * feat + c] = 0.f; continue; }
+      double acc = red == 1 ? (double)(float)INT32_MIN : red == 2 ? (double)(float)INT32_MAX : 0.0;
+      for (int k = lb; k < hb; ++k) {
+        const float f = b[(Index)colind[k] * feat + c];
+        float t = f;
+        if (val) {
+          const float v = val[k];
+          t = comp == 0 ? v + f : comp == 1 ? f - v : comp == 2 ? v * f : f / v;
+        }
+        if (red == 1) acc = (double)t > acc ? (double)t : acc;
+        else if (red == 2) acc = (double)t < acc ? (double)t : acc;
+        else acc += (double)t;
+      }
+      if (red == 3) acc /= (double)(hb - lb);
+      out[r * feat + c] = (float)acc;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------- */
 /* gather_fwd / gather_bwd src/cpp/src/aggr.cu:42-62                           */
 /*   fwd: out[dest[e]] += in[e] (out zeroed first, aggr.cu:406);               */
 /*   bwd: gin[e] = gout[dest[e]]                                               */

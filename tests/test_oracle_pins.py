@@ -387,3 +387,46 @@ def test_small_hand_cases_for_row_filters_and_select_mm():
     out = pyref.typed_linear_naive_s2d(x, w, types, eidx, dstn, 2, 5)
     want = torch.stack([2 * x[3] + 2 * x[2], x[0] + 2 * x[1] + x[3]])
     assert torch.equal(out, want)
+
+
+# ----------------------------------------------------------------------------- dgSPARSE-style GSpMM
+@pytest.mark.parametrize("comp", [None, 0, 1, 2, 3])
+def test_gspmm_matches_scipy_and_reduceat(comp):
+    """REDUCE x COMPUTE of the generalised SpMM against closed forms: sparse products for
+    sum / mean (val+b = rowsum(val) + A1 b, b-val = A1 b - rowsum(val), val*b = A_val b,
+    b/val = A_{1/val} b), numpy's segmented ufunc.reduceat for max / min."""
+    n_dst, n_src, F = 90, 70, 5
+    ptr, idx = rand_graph(n_dst, n_src, 600, 21)
+    rng = np.random.default_rng(22)
+    b = rng.standard_normal((n_src, F)).astype(np.float32)
+    E = idx.shape[0]
+    val = (rng.random(E) + 0.5).astype(np.float32) * rng.choice([-1.0, 1.0], E).astype(np.float32)
+    deg = np.diff(ptr)
+    ones = as_scipy(ptr, idx, np.ones(E), n_src)
+    b64 = b.astype(np.float64)
+    if comp is None:
+        want_sum, terms = ones @ b64, b64[idx]
+    else:
+        v = val.astype(np.float64)
+        rowsum = np.add.reduceat(np.concatenate([v, [0.0]]), np.minimum(ptr[:-1], E))
+        rowsum = np.where(deg > 0, rowsum, 0.0)[:, None]
+        want_sum = [rowsum + ones @ b64, ones @ b64 - rowsum, as_scipy(ptr, idx, v, n_src) @ b64,
+                    as_scipy(ptr, idx, 1.0 / v, n_src) @ b64][comp]
+        g = b64[idx]
+        terms = [v[:, None] + g, g - v[:, None], v[:, None] * g, g / v[:, None]][comp]
+    kw = {} if comp is None else {"val": val}
+    c = 2 if comp is None else comp
+    assert np.allclose(oracle.gspmm(ptr, idx, b, 0, c, **kw), want_sum, rtol=1e-5, atol=1e-5)
+    want_mean = np.where(deg[:, None] > 0, want_sum / np.maximum(deg, 1)[:, None], 0.0)
+    assert np.allclose(oracle.gspmm(ptr, idx, b, 3, c, **kw), want_mean, rtol=1e-5, atol=1e-5)
+    nonempty = deg > 0
+    starts = ptr[:-1][nonempty]
+    for red, uf in ((1, np.maximum), (2, np.minimum)):
+        want = np.zeros((n_dst, F))
+        want[nonempty] = uf.reduceat(terms, starts, axis=0)
+        got = oracle.gspmm(ptr, idx, b, red, c, **kw)
+        assert np.allclose(got, want.astype(np.float32), rtol=1e-6, atol=0)
+    # the accumulator of max / min starts at (float)INT_MIN / (float)INT_MAX (dgsparse.h:117-130)
+    big = np.full((1, 1), -3e9, dtype=np.float32)
+    assert oracle.gspmm([0, 1], [0], big, 1)[0, 0] == np.float32(-2147483648.0)
+    assert oracle.gspmm([0, 1], [0], -big, 2)[0, 0] == np.float32(2147483648.0)
