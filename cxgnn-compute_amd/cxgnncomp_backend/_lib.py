@@ -51,6 +51,7 @@ SIGNATURES = {
     "cxg_edge_value_degree_f32": (_I32, [_P, _I64, _P, _P]),
     "cxg_pad_rel_i64": (_I32, [_P, _P, _P, _I32, _I32, _I64, _P]),
     "cxg_gspmm_i32_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "cxg_topo_sort_host_i64": (_I64, [_P, _P, _P, _I64, _P]),
     "cxg_scan_workspace_bytes": (_SZ, [_I64]),
     "cxg_neighbor_group_plan_i64": (_I32, [_P, _I64, _I64, _P, _P, _SZ, _P]),
     "cxg_neighbor_group_fill_i64": (_I32, [_P, _P, _I64, _I64, _I64, _P, _P, _P]),

@@ -106,8 +106,27 @@ def gen_edge_type_mag240m(ptr, idx, sub_to_full):
 
 
 def topo_sort(csr_ptr, csr_idx, degree):
-    raise NotImplementedError("topo_sort (src/cpp/src/schedule.cu:72-128) is not used by any "
-                              "aggregation path and is not provided")
+    """Topological order of the nodes of a successor-list CSR on CPU tensors
+    (src/cpp/src/schedule.cu:71-128): FIFO from the nodes with degree 0; cycles are
+    broken by releasing the nodes with counter 1 and the first running-minimum node.
+    Entries of nodes never reached are left uninitialised, as upstream does."""
+    for t, name in ((csr_ptr, "csr_ptr"), (csr_idx, "csr_idx"), (degree, "degree")):
+        if t.is_cuda or t.dtype != torch.int64 or t.dim() != 1:
+            raise ValueError("%s must be a 1-D int64 CPU tensor" % name)
+    n = degree.shape[0]
+    if csr_ptr.shape[0] < n + 1:
+        raise ValueError("csr_ptr needs %d entries" % (n + 1))
+    ptr, idx, deg = csr_ptr.contiguous(), csr_idx.contiguous(), degree.contiguous()
+    n_edges = int(ptr[n]) if n else 0
+    if n_edges > idx.shape[0] or (n_edges and (int(idx[:n_edges].min()) < 0 or int(idx[:n_edges].max()) >= n)):
+        raise ValueError("csr_idx does not match csr_ptr / the number of nodes")
+    out = torch.empty(n, dtype=torch.int64)
+    cnt = _lib.load().cxg_topo_sort_host_i64(ptr.data_ptr(), idx.data_ptr(), deg.data_ptr(), n, out.data_ptr())
+    if cnt < 0:
+        _lib.check(int(cnt))
+    if cnt != n:
+        print("Error: graph is not a DAG, %d %d" % (cnt, n))
+    return out
 
 
 class REDUCEOP(enum.IntEnum):

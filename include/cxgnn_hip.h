@@ -386,6 +386,18 @@ int cxg_coo_to_csr_i64(const int64_t* src, const int64_t* dst, int64_t n_edges, 
                        int64_t* ptr, int64_t* idx, int64_t* perm, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/*
+ * Host-side (CPU memory, sequential) topological order of a graph given as CSR
+ * successor lists: FIFO queue seeded with the nodes whose `degree` counter is 0
+ * in id order; when the queue runs dry early, every node with counter 1 and the
+ * first node holding the running minimum counter above 1 are released.  Writes
+ * the emitted node ids to order[0..ret) and returns their number (< n_nodes for
+ * inputs the release rule cannot finish), or a negative status.  Replaces
+ * topo_sort (src/cpp/src/schedule.cu:71-128).
+ */
+int64_t cxg_topo_sort_host_i64(const int64_t* ptr, const int64_t* idx, const int64_t* degree,
+                               int64_t n_nodes, int64_t* order);
+
 #ifdef __cplusplus
 }
 #endif

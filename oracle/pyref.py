@@ -192,3 +192,35 @@ def reorder_by(ptr, idx, metric):
         new_ptr.append(new_ptr[-1] + int(ptr[c + 1] - ptr[c]))
         new_idx += [int(v) for v in idx[ptr[c]:ptr[c + 1]]]
     return np.array(new_ptr, dtype=np.int64), np.array(new_idx, dtype=np.int64)
+
+
+def topo_sort(ptr, idx, degree):
+    """src/cpp/src/schedule.cu:71-128 restated with a deque (small inputs only).
+    Returns (order list, number emitted)."""
+    from collections import deque
+    n = len(degree)
+    deg = [int(d) for d in degree]
+    q = deque(i for i in range(n) if deg[i] == 0)
+    out = []
+    while len(out) < n:
+        while q:
+            cur = q.popleft()
+            out.append(cur)
+            for k in range(int(ptr[cur]), int(ptr[cur + 1])):
+                nxt = int(idx[k])
+                deg[nxt] -= 1
+                if deg[nxt] == 0:
+                    q.append(nxt)
+        min_deg, pick = n, -1
+        for i in range(n):
+            if 1 < deg[i] < min_deg:
+                min_deg, pick = deg[i], i
+            elif deg[i] == 1:
+                deg[i] = 0
+                q.append(i)
+        if pick != -1:
+            q.append(pick)
+            deg[pick] = 0
+        elif not q:
+            break
+    return out, len(out)

@@ -314,3 +314,25 @@ def test_batch_round_trip(tmp_path):
     b2 = cxgnncomp.Batch.fromfile(str(tmp_path), 8)
     assert torch.equal(b2.x, x) and torch.equal(b2.ptr, ptr) and torch.equal(b2.idx, idx)
     assert b2.num_node_in_layer.tolist() == nn and b2.num_edge_in_layer.tolist() == ne
+
+
+def test_topo_sort_matches_restatement(capsys):
+    import cxgnncomp_backend as B
+    rng = np.random.default_rng(41)
+    for n, e, cyclic in ((1, 0, False), (50, 160, False), (300, 1500, False), (60, 200, True), (300, 900, True)):
+        if cyclic:
+            src, dst = rng.integers(0, n, e), rng.integers(0, n, e)
+        else:
+            a, b = rng.integers(0, n, e), rng.integers(0, n, e)
+            keep = a != b
+            relabel = rng.permutation(n)
+            src, dst = relabel[np.minimum(a, b)[keep]], relabel[np.maximum(a, b)[keep]]
+        ptr, idx = oracle.coo_to_csr(dst, src, n)
+        indeg = np.bincount(dst, minlength=n).astype(np.int64)
+        want, cnt = pyref.topo_sort(ptr, idx, indeg)
+        got = B.topo_sort(torch.from_numpy(ptr), torch.from_numpy(idx), torch.from_numpy(indeg))
+        assert got.dtype == torch.int64 and got[:cnt].tolist() == want
+        msg = capsys.readouterr().out
+        assert ("not a DAG" in msg) == (cnt != n)
+    with pytest.raises(ValueError):
+        B.topo_sort(torch.tensor([0, 1]), torch.tensor([5]), torch.tensor([0]))

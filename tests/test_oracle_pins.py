@@ -430,3 +430,42 @@ def test_gspmm_matches_scipy_and_reduceat(comp):
     big = np.full((1, 1), -3e9, dtype=np.float32)
     assert oracle.gspmm([0, 1], [0], big, 1)[0, 0] == np.float32(-2147483648.0)
     assert oracle.gspmm([0, 1], [0], -big, 2)[0, 0] == np.float32(2147483648.0)
+
+
+# ----------------------------------------------------------------------------- topo_sort
+def _random_dag(rng, n, e):
+    a, b = rng.integers(0, n, e), rng.integers(0, n, e)
+    keep = a != b
+    lo, hi = np.minimum(a, b)[keep], np.maximum(a, b)[keep]
+    relabel = rng.permutation(n)                       # hide the order the edges were built from
+    src, dst = relabel[lo], relabel[hi]
+    ptr, idx = oracle.coo_to_csr(dst, src, n)          # successor lists: row = src, entries = dst
+    return ptr, idx, np.bincount(dst, minlength=n)
+
+
+def test_topo_sort_restatement_on_dags_and_hand_cases():
+    rng = np.random.default_rng(31)
+    for n, e in ((1, 0), (6, 9), (200, 900)):
+        ptr, idx, indeg = _random_dag(rng, n, e)
+        order, cnt = pyref.topo_sort(ptr, idx, indeg)
+        assert cnt == n and sorted(order) == list(range(n))
+        pos = np.empty(n, dtype=np.int64)
+        pos[order] = np.arange(n)
+        src = np.repeat(np.arange(n), np.diff(ptr))
+        assert (pos[src] < pos[idx]).all()              # every edge goes forward
+        # a FIFO Kahn walk emits nodes in non-decreasing longest-path depth
+        depth = np.zeros(n, dtype=np.int64)
+        for _ in range(n):
+            nd = depth.copy()
+            np.maximum.at(nd, idx, depth[src] + 1)
+            if (nd == depth).all():
+                break
+            depth = nd
+        assert (np.diff(depth[order]) >= 0).all()
+    # 3 -> 2 -> {0, 1}, 0 <-> 1: the 2-cycle is released by the "counter == 1" rule
+    ptr, idx = [0, 1, 2, 4, 5], [1, 0, 0, 1, 2]
+    assert pyref.topo_sort(ptr, idx, [2, 2, 1, 0]) == ([3, 2, 0, 1], 4)
+    # a plain 3-cycle: all counters are 1, released in id order
+    assert pyref.topo_sort([0, 1, 2, 3], [1, 2, 0], [1, 1, 1]) == ([0, 1, 2], 3)
+    # counters the release rule cannot start from (running minimum starts at n)
+    assert pyref.topo_sort([0, 1, 2], [1, 0], [2, 3]) == ([], 0)
