@@ -173,9 +173,11 @@ def c3(iters):
     gev = torch.randn(E, H, device="cuda")
     gt = _ops.transposed(ptr, idx, N, N)
 
+    rows_t = _ops.rows32_transposed(gt)
+
     def sm_bwd():
         g_dst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, gev, N, 0.2)
-        return _ops.narrow_gather_sum(gt.ptr_t, gt.perm, t_edge, N)
+        return _ops.narrow_gather_sum(gt.ptr_t, gt.perm, t_edge, N, rows32=rows_t)
     report("c3", "edge_softmax_bwd H=4 (row pass + transposed gather)", timeit(sm_bwd, iters),
            E * H * (4 + 4 + 1 + 4) + E * (8 + 4 * H) + 8 * N * H, 6 * E * H)
     x = torch.randn(N, H, C, device="cuda") / 8

@@ -13,8 +13,11 @@
 //
 //   forward  (edge_softmax_fwd, src/cpp/src/edge_softmax.cu:3-42):
 //     t = leaky_relu(att_dst[r,h] + att_src[idx[e],h]);  out = softmax_row(t);
-//     mask = t > 0.  Online max/sum in the first sweep, write in the second
-//     (the reference makes three read-modify-write sweeps over out).
+//     mask = t > 0.  First sweep: gather, online max/sum, t parked in `out`;
+//     second sweep: the same lane normalises its own t in place.  One 16-byte
+//     gather per edge in total -- every gather is a whole cache line over the
+//     fabric, the re-read of `out` is a coalesced stream (the reference makes
+//     three read-modify-write sweeps over out).
 //   backward (edge_softmax_bwd, src/cpp/src/edge_softmax.cu:44-95):
 //     s = sum_row out*g;  t = out*(g-s)*(mask ? 1 : slope);
 //     g_dst[r,h] = sum_row t (left 0 unless the row has both signs, :91-93);
@@ -29,8 +32,18 @@ namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
-constexpr int kShortDeg = 16;
-constexpr int kWaveDeg = 512;
+#ifndef CXG_SOFTMAX_SHORT_DEG
+#define CXG_SOFTMAX_SHORT_DEG 16
+#endif
+#ifndef CXG_SOFTMAX_WAVE_DEG
+#define CXG_SOFTMAX_WAVE_DEG 512
+#endif
+#ifndef CXG_SOFTMAX_TIERS
+#define CXG_SOFTMAX_TIERS 7   // bit 0 lane tier, bit 1 wave tier, bit 2 block tier (timing experiments)
+#endif
+constexpr int kShortDeg = CXG_SOFTMAX_SHORT_DEG;
+constexpr int kWaveDeg = CXG_SOFTMAX_WAVE_DEG;
+constexpr int kTiers = CXG_SOFTMAX_TIERS;
 
 __device__ __forceinline__ float wave_max(float v) {
   for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, CXG_WAVE));
@@ -42,33 +55,109 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // Cooperative scopes: the same row code runs with 64 lanes (one wave) or with the
-// 256 threads of the block; `li`/`nl` enumerate the participants.
+// 256 threads of the block; `li`/`nl` enumerate the participants.  Reductions take
+// all N per-head values at once so that the block scope needs one LDS exchange
+// (two barriers) per reduction, not one per head.
+constexpr int kMaxRed = 8;    // most values reduced together (heads handled at once)
+
+__device__ __forceinline__ float wave_or_bits(float v) {   // small non-negative integers as floats
+  int b = (int)v;
+  for (int m = 32; m > 0; m >>= 1) b |= __shfl_xor(b, m, CXG_WAVE);
+  return (float)b;
+}
+// (m, s) pairs of an online softmax: s = sum of exp(t - m) over the values seen.
+__device__ __forceinline__ void merge_max_sum(float& m, float& s, float m2, float s2) {
+  const float mn = fmaxf(m, m2);
+  s = s * __expf(m - mn) + s2 * __expf(m2 - mn);
+  m = mn;
+}
+
 struct WaveScope {
   int li;
   static constexpr int nl = CXG_WAVE;
-  __device__ __forceinline__ float max(float v) const { return wave_max(v); }
+  template <int N> __device__ __forceinline__ void sum_n(float (&v)[N]) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = wave_sum(v[i]);
+  }
+  template <int N> __device__ __forceinline__ void or_n(float (&v)[N]) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = wave_or_bits(v[i]);
+  }
+  template <int N> __device__ __forceinline__ void combine_max_sum(float (&m)[N], float (&s)[N]) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float mw = wave_max(m[i]);
+      s[i] = wave_sum(s[i] * __expf(m[i] - mw));
+      m[i] = mw;
+    }
+  }
   __device__ __forceinline__ float sum(float v) const { return wave_sum(v); }
-  __device__ __forceinline__ bool any(bool p) const { return __ballot(p) != 0; }
   __device__ __forceinline__ bool leader() const { return li == 0; }
 };
 struct BlockScope {
   int li;
-  float* red;   // kWavesPerBlock floats of LDS
+  float* red;   // kWavesPerBlock * 2 * kMaxRed floats of LDS
   static constexpr int nl = kBlock;
-  template <bool MAX>
-  __device__ __forceinline__ float reduce(float v) const {
-    v = MAX ? wave_max(v) : wave_sum(v);
+  // every wave leaves K values, every thread reads all of them back
+  template <int K> __device__ __forceinline__ void exchange(const float (&mine)[K], float (&all)[kWavesPerBlock][K]) const {
     __syncthreads();                      // previous use of `red` is over
-    if ((li & 63) == 0) red[li >> 6] = v;
-    __syncthreads();
-    float r = red[0];
+    if ((li & 63) == 0) {
 #pragma unroll
-    for (int w = 1; w < kWavesPerBlock; ++w) r = MAX ? fmaxf(r, red[w]) : r + red[w];
-    return r;
+      for (int i = 0; i < K; ++i) red[(li >> 6) * K + i] = mine[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w)
+#pragma unroll
+      for (int i = 0; i < K; ++i) all[w][i] = red[w * K + i];
   }
-  __device__ __forceinline__ float max(float v) const { return reduce<true>(v); }
-  __device__ __forceinline__ float sum(float v) const { return reduce<false>(v); }
-  __device__ __forceinline__ bool any(bool p) const { return reduce<true>(p ? 1.f : 0.f) > 0.f; }
+  template <int N> __device__ __forceinline__ void sum_n(float (&v)[N]) const {
+    float all[kWavesPerBlock][N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = wave_sum(v[i]);
+    exchange<N>(v, all);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      v[i] = all[0][i];
+#pragma unroll
+      for (int w = 1; w < kWavesPerBlock; ++w) v[i] += all[w][i];
+    }
+  }
+  template <int N> __device__ __forceinline__ void or_n(float (&v)[N]) const {
+    float all[kWavesPerBlock][N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = wave_or_bits(v[i]);
+    exchange<N>(v, all);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int b = (int)all[0][i];
+#pragma unroll
+      for (int w = 1; w < kWavesPerBlock; ++w) b |= (int)all[w][i];
+      v[i] = (float)b;
+    }
+  }
+  template <int N> __device__ __forceinline__ void combine_max_sum(float (&m)[N], float (&s)[N]) const {
+    float mine[2 * N], all[kWavesPerBlock][2 * N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float mw = wave_max(m[i]);
+      mine[2 * i] = mw;
+      mine[2 * i + 1] = wave_sum(s[i] * __expf(m[i] - mw));
+    }
+    exchange<2 * N>(mine, all);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      m[i] = all[0][2 * i];
+      s[i] = all[0][2 * i + 1];
+#pragma unroll
+      for (int w = 1; w < kWavesPerBlock; ++w) merge_max_sum(m[i], s[i], all[w][2 * i], all[w][2 * i + 1]);
+    }
+  }
+  __device__ __forceinline__ float sum(float v) const {
+    float a[1] = {v};
+    sum_n<1>(a);
+    return a[0];
+  }
   __device__ __forceinline__ bool leader() const { return li == 0; }
 };
 
@@ -78,7 +167,7 @@ template <class ShortFn, class CoopFn>
 __device__ __forceinline__ void tiered_rows(const int64_t* __restrict__ ptr, int64_t n_rows,
                                             ShortFn short_fn, CoopFn coop_fn) {
   __shared__ unsigned long long s_very_long[kWavesPerBlock];
-  __shared__ float s_red[kWavesPerBlock];
+  __shared__ float s_red[kWavesPerBlock * 2 * kMaxRed];
   const int lane = lane_id();
   const int wave = uniform_i32(threadIdx.x >> 6);
   const int64_t row0 = (int64_t)blockIdx.x * kBlock;
@@ -87,9 +176,9 @@ __device__ __forceinline__ void tiered_rows(const int64_t* __restrict__ ptr, int
   int64_t b = 0, e = 0;
   if (valid) { b = ptr[r]; e = ptr[r + 1]; }
   const int64_t deg = e - b;
-  if (valid && deg <= kShortDeg) short_fn(r, b, e);
-  uint64_t todo = __ballot(valid && deg > kShortDeg && deg <= kWaveDeg);
-  const uint64_t very_long = __ballot(valid && deg > kWaveDeg);
+  if ((kTiers & 1) && valid && deg <= kShortDeg) short_fn(r, b, e);
+  uint64_t todo = __ballot((kTiers & 2) && valid && deg > kShortDeg && deg <= kWaveDeg);
+  const uint64_t very_long = __ballot((kTiers & 4) && valid && deg > kWaveDeg);
   WaveScope ws{lane};
   while (todo) {
     const int l = __ffsll((unsigned long long)todo) - 1;
@@ -181,6 +270,13 @@ __device__ __forceinline__ void online_add(float& m, float& s, float t) {
 
 constexpr float kMaxInit = -100000.f;  // running-max start of the reference kernel
 
+// Edges are visited kU at a time: the kU index loads, then the kU gathers, are
+// issued back to back (addresses past the row end are clamped to its last edge
+// and their results dropped), so a lane has kU independent memory round trips
+// in flight instead of one.  The row loops are latency chains; this is what
+// shortens them.
+constexpr int kU = 4;
+
 template <int H>
 __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_kernel(
     const int64_t* __restrict__ ptr, const int64_t* __restrict__ idx,
@@ -190,63 +286,75 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_kernel(
   const int nh = H > 0 ? H : heads;
   constexpr int HB = H > 0 ? H : 1;     // heads processed together
   for (int h0 = 0; h0 < nh; h0 += HB) {
-    auto short_fn = [&](int64_t r, int64_t b, int64_t e) {
-      float d[HB], m[HB], s[HB];
+    // rows of row r visited by this participant: first, first + stride, ... < e
+    auto sweep_rows = [&](int64_t r, int64_t first, int64_t stride, int64_t e, float (&m)[HB], float (&s)[HB]) {
+      float d[HB];
       load_f<HB>(att_dst + r * nh + h0, d);
 #pragma unroll
       for (int h = 0; h < HB; ++h) { m[h] = kMaxInit; s[h] = 0.f; }
-      for (int64_t k = b; k < e; ++k) {
-        float as[HB];
-        load_f<HB>(att_src + idx[k] * nh + h0, as);
+      for (int64_t k = first; k < e; k += kU * stride) {
+        int64_t kk[kU], src[kU];
+        float as[kU][HB];
 #pragma unroll
-        for (int h = 0; h < HB; ++h) online_add(m[h], s[h], leaky(d[h] + as[h], slope));
-      }
-#pragma unroll
-      for (int h = 0; h < HB; ++h) s[h] = 1.0f / s[h];
-      for (int64_t k = b; k < e; ++k) {
-        float as[HB], o[HB];
-        bool mk[HB];
-        load_f<HB>(att_src + idx[k] * nh + h0, as);
-#pragma unroll
-        for (int h = 0; h < HB; ++h) {
-          const float t = leaky(d[h] + as[h], slope);
-          o[h] = __expf(t - m[h]) * s[h];
-          mk[h] = t > 0.f;
+        for (int u = 0; u < kU; ++u) {
+          kk[u] = k + u * stride;
+          src[u] = idx[kk[u] < e ? kk[u] : e - 1];
         }
-        store_f<HB>(out + k * nh + h0, o);
-        store_b<HB>(mask + k * nh + h0, mk);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) load_f<HB>(att_src + src[u] * nh + h0, as[u]);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          if (kk[u] < e) {
+            float t[HB];
+#pragma unroll
+            for (int h = 0; h < HB; ++h) {
+              t[h] = leaky(d[h] + as[u][h], slope);
+              online_add(m[h], s[h], t[h]);
+            }
+            store_f<HB>(out + kk[u] * nh + h0, t);   // parked in `out` until the row's max / sum are known
+          }
+        }
       }
     };
-    auto coop_fn = [&](auto sc, int64_t r, int64_t b, int64_t e) {
-      float d[HB], m[HB], s[HB];
-      load_f<HB>(att_dst + r * nh + h0, d);
+    auto write_rows = [&](int64_t first, int64_t stride, int64_t e, const float (&m)[HB], const float (&s)[HB]) {
+      for (int64_t k = first; k < e; k += kU * stride) {
+        int64_t kk[kU];
+        float t[kU][HB];
 #pragma unroll
-      for (int h = 0; h < HB; ++h) { m[h] = kMaxInit; s[h] = 0.f; }
-      for (int64_t k = b + sc.li; k < e; k += sc.nl) {
-        float as[HB];
-        load_f<HB>(att_src + idx[k] * nh + h0, as);
-#pragma unroll
-        for (int h = 0; h < HB; ++h) online_add(m[h], s[h], leaky(d[h] + as[h], slope));
-      }
-#pragma unroll
-      for (int h = 0; h < HB; ++h) {
-        const float mw = sc.max(m[h]);
-        s[h] = 1.0f / sc.sum(s[h] * __expf(m[h] - mw));
-        m[h] = mw;
-      }
-      for (int64_t k = b + sc.li; k < e; k += sc.nl) {
-        float as[HB], o[HB];
-        bool mk[HB];
-        load_f<HB>(att_src + idx[k] * nh + h0, as);
-#pragma unroll
-        for (int h = 0; h < HB; ++h) {
-          const float t = leaky(d[h] + as[h], slope);
-          o[h] = __expf(t - m[h]) * s[h];
-          mk[h] = t > 0.f;
+        for (int u = 0; u < kU; ++u) {
+          kk[u] = k + u * stride;
+          load_f<HB>(out + (kk[u] < e ? kk[u] : first) * nh + h0, t[u]);   // written by this lane above
         }
-        store_f<HB>(out + k * nh + h0, o);
-        store_b<HB>(mask + k * nh + h0, mk);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          if (kk[u] < e) {
+            float o[HB];
+            bool mk[HB];
+#pragma unroll
+            for (int h = 0; h < HB; ++h) {
+              o[h] = __expf(t[u][h] - m[h]) * s[h];
+              mk[h] = t[u][h] > 0.f;
+            }
+            store_f<HB>(out + kk[u] * nh + h0, o);
+            store_b<HB>(mask + kk[u] * nh + h0, mk);
+          }
+        }
       }
+    };
+    auto short_fn = [&](int64_t r, int64_t b, int64_t e) {
+      float m[HB], s[HB];
+      sweep_rows(r, b, 1, e, m, s);
+#pragma unroll
+      for (int h = 0; h < HB; ++h) s[h] = 1.0f / s[h];
+      write_rows(b, 1, e, m, s);
+    };
+    auto coop_fn = [&](auto sc, int64_t r, int64_t b, int64_t e) {
+      float m[HB], s[HB];
+      sweep_rows(r, b + sc.li, sc.nl, e, m, s);
+      sc.template combine_max_sum<HB>(m, s);           // row-wide max and sum of exp(t - max)
+#pragma unroll
+      for (int h = 0; h < HB; ++h) s[h] = 1.0f / s[h];
+      write_rows(b + sc.li, sc.nl, e, m, s);             // the same lane revisits the same edges
     };
     tiered_rows(ptr, n_rows, short_fn, coop_fn);
   }
@@ -260,74 +368,80 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
   const int nh = H > 0 ? H : heads;
   constexpr int HB = H > 0 ? H : 1;
   for (int h0 = 0; h0 < nh; h0 += HB) {
+    auto dot_rows = [&](int64_t first, int64_t stride, int64_t e, float (&s)[HB]) {
+#pragma unroll
+      for (int h = 0; h < HB; ++h) s[h] = 0.f;
+      for (int64_t k = first; k < e; k += kU * stride) {
+        int64_t kk[kU];
+        float o[kU][HB], g[kU][HB];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          kk[u] = k + u * stride;
+          const int64_t c = kk[u] < e ? kk[u] : first;
+          load_f<HB>(out + c * nh + h0, o[u]);
+          load_f<HB>(grad + c * nh + h0, g[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u)
+          if (kk[u] < e)
+#pragma unroll
+            for (int h = 0; h < HB; ++h) s[h] += o[u][h] * g[u][h];
+      }
+    };
+    auto edge_rows = [&](int64_t first, int64_t stride, int64_t e, const float (&s)[HB], float (&dsum)[HB],
+                         int (&pos)[HB], int (&neg)[HB]) {
+#pragma unroll
+      for (int h = 0; h < HB; ++h) { dsum[h] = 0.f; pos[h] = 0; neg[h] = 0; }
+      for (int64_t k = first; k < e; k += kU * stride) {
+        int64_t kk[kU];
+        float o[kU][HB], g[kU][HB];
+        bool mk[kU][HB];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          kk[u] = k + u * stride;
+          const int64_t c = kk[u] < e ? kk[u] : first;
+          load_f<HB>(out + c * nh + h0, o[u]);
+          load_f<HB>(grad + c * nh + h0, g[u]);
+          load_b<HB>(mask + c * nh + h0, mk[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          if (kk[u] < e) {
+            float tv[HB];
+#pragma unroll
+            for (int h = 0; h < HB; ++h) {
+              float t = o[u][h] * (g[u][h] - s[h]);
+              if (!mk[u][h]) { t *= slope; neg[h] = 1; } else { pos[h] = 1; }
+              dsum[h] += t;
+              tv[h] = t;
+            }
+            store_f<HB>(t_edge + kk[u] * nh + h0, tv);
+          }
+        }
+      }
+    };
     auto short_fn = [&](int64_t r, int64_t b, int64_t e) {
       float s[HB], dsum[HB];
       int pos[HB], neg[HB];
-#pragma unroll
-      for (int h = 0; h < HB; ++h) { s[h] = 0.f; dsum[h] = 0.f; pos[h] = 0; neg[h] = 0; }
-      for (int64_t k = b; k < e; ++k)
-      {
-        float o[HB], g[HB];
-        load_f<HB>(out + k * nh + h0, o);
-        load_f<HB>(grad + k * nh + h0, g);
-#pragma unroll
-        for (int h = 0; h < HB; ++h) s[h] += o[h] * g[h];
-      }
-      for (int64_t k = b; k < e; ++k)
-      {
-        float o[HB], g[HB], tv[HB];
-        bool mk[HB];
-        load_f<HB>(out + k * nh + h0, o);
-        load_f<HB>(grad + k * nh + h0, g);
-        load_b<HB>(mask + k * nh + h0, mk);
-#pragma unroll
-        for (int h = 0; h < HB; ++h) {
-          float t = o[h] * (g[h] - s[h]);
-          if (!mk[h]) { t *= slope; neg[h] = 1; } else { pos[h] = 1; }
-          dsum[h] += t;
-          tv[h] = t;
-        }
-        store_f<HB>(t_edge + k * nh + h0, tv);
-      }
+      dot_rows(b, 1, e, s);
+      edge_rows(b, 1, e, s, dsum, pos, neg);
 #pragma unroll
       for (int h = 0; h < HB; ++h) g_dst[r * nh + h0 + h] = (pos[h] && neg[h]) ? dsum[h] : 0.f;
     };
     auto coop_fn = [&](auto sc, int64_t r, int64_t b, int64_t e) {
       float s[HB], dsum[HB];
       int pos[HB], neg[HB];
+      dot_rows(b + sc.li, sc.nl, e, s);
+      sc.template sum_n<HB>(s);
+      edge_rows(b + sc.li, sc.nl, e, s, dsum, pos, neg);
+      float flags[HB];                                   // 1: positive seen, 2: negative seen
 #pragma unroll
-      for (int h = 0; h < HB; ++h) { s[h] = 0.f; dsum[h] = 0.f; pos[h] = 0; neg[h] = 0; }
-      for (int64_t k = b + sc.li; k < e; k += sc.nl)
-      {
-        float o[HB], g[HB];
-        load_f<HB>(out + k * nh + h0, o);
-        load_f<HB>(grad + k * nh + h0, g);
+      for (int h = 0; h < HB; ++h) flags[h] = (float)(pos[h] + 2 * neg[h]);
+      sc.template sum_n<HB>(dsum);
+      sc.template or_n<HB>(flags);
+      if (sc.leader()) {
 #pragma unroll
-        for (int h = 0; h < HB; ++h) s[h] += o[h] * g[h];
-      }
-#pragma unroll
-      for (int h = 0; h < HB; ++h) s[h] = sc.sum(s[h]);
-      for (int64_t k = b + sc.li; k < e; k += sc.nl)
-      {
-        float o[HB], g[HB], tv[HB];
-        bool mk[HB];
-        load_f<HB>(out + k * nh + h0, o);
-        load_f<HB>(grad + k * nh + h0, g);
-        load_b<HB>(mask + k * nh + h0, mk);
-#pragma unroll
-        for (int h = 0; h < HB; ++h) {
-          float t = o[h] * (g[h] - s[h]);
-          if (!mk[h]) { t *= slope; neg[h] = 1; } else { pos[h] = 1; }
-          dsum[h] += t;
-          tv[h] = t;
-        }
-        store_f<HB>(t_edge + k * nh + h0, tv);
-      }
-#pragma unroll
-      for (int h = 0; h < HB; ++h) {
-        const float total = sc.sum(dsum[h]);
-        const bool both = sc.any(pos[h] != 0) && sc.any(neg[h] != 0);
-        if (sc.leader()) g_dst[r * nh + h0 + h] = both ? total : 0.f;
+        for (int h = 0; h < HB; ++h) g_dst[r * nh + h0 + h] = ((int)flags[h] == 3) ? dsum[h] : 0.f;
       }
     };
     tiered_rows(ptr, n_rows, short_fn, coop_fn);

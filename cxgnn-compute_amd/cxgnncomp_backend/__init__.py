@@ -196,7 +196,7 @@ class _EdgeSoftmaxFunction(torch.autograd.Function):
         ptr, idx, out, mask = ctx.saved_tensors
         g_dst, t_edge = _ops.edge_softmax_bwd(ptr, out, mask, grad_out.contiguous(), ctx.n_dst, ctx.slope)
         g = _ops.transposed(ptr, idx, ctx.n_dst, ctx.n_src)
-        g_src = _ops.narrow_gather_sum(g.ptr_t, g.perm, t_edge, ctx.n_src)
+        g_src = _ops.narrow_gather_sum(g.ptr_t, g.perm, t_edge, ctx.n_src, rows32=_ops.rows32_transposed(g))
         return None, None, g_dst, g_src, None, None
 
 

@@ -118,13 +118,14 @@ class TransposedGraph:
     """CSR of the reversed graph: rows = source nodes, idx_t = destination ids,
     perm = position of each transposed edge in the original idx array."""
 
-    __slots__ = ("ptr_t", "idx_t", "perm", "n_edges", "n_src", "n_dst", "_keep", "_inv_deg_t")
+    __slots__ = ("ptr_t", "idx_t", "perm", "n_edges", "n_src", "n_dst", "_keep", "_inv_deg_t", "_rows32")
 
     def __init__(self, ptr_t, idx_t, perm, n_edges, n_src, n_dst, keep):
         self.ptr_t, self.idx_t, self.perm = ptr_t, idx_t, perm
         self.n_edges, self.n_src, self.n_dst = n_edges, n_src, n_dst
         self._keep = keep  # the tensors the key was made from stay alive while cached
         self._inv_deg_t = None
+        self._rows32 = None
 
 
 _GRAPH_CACHE = collections.OrderedDict()
@@ -326,8 +327,29 @@ def edge_softmax_bwd(ptr, out, mask, grad, n_dst, slope):
     return g_dst, t_edge
 
 
-def narrow_gather_sum(ptr, sel, inp, n_rows):
-    """out[r,:] = sum_{k in row r} inp[sel[k],:] (sel None: inp[k,:]); inp [M] or [M,W]."""
+def csr_row_ids32(ptr, n_rows, n_edges):
+    """int32 row id of every edge position (the edge-parallel kernels' row lookup)."""
+    lib = _lib.load()
+    _req(ptr, "ptr", torch.int64, 1)
+    rows = torch.empty(n_edges, dtype=torch.int32, device=ptr.device)
+    with torch.cuda.device(ptr.device):
+        st = lib.cxg_csr_row_ids_i32(ptr.data_ptr(), n_rows, n_edges, _lib.ptr(rows),
+                                     _lib.current_stream(ptr.device))
+    _lib.check(st)
+    return rows
+
+
+def rows32_transposed(g):
+    """Row (source) id of every edge of a TransposedGraph, built once and kept with it."""
+    if g._rows32 is None:
+        g._rows32 = csr_row_ids32(g.ptr_t, g.n_src, g.n_edges)
+    return g._rows32
+
+
+def narrow_gather_sum(ptr, sel, inp, n_rows, rows32=None):
+    """out[r,:] = sum_{k in row r} inp[sel[k],:] (sel None: inp[k,:]); inp [M] or [M,W].
+    With ``rows32`` (int32 row id per edge of ptr[:n_rows+1], ptr[0] == 0) and W in
+    {1, 2, 4, 8} the edge-parallel segmented kernel is used."""
     lib = _lib.load()
     _req(ptr, "ptr", torch.int64, 1)
     if n_rows + 1 > ptr.shape[0]:
@@ -339,8 +361,16 @@ def narrow_gather_sum(ptr, sel, inp, n_rows):
     shape = (n_rows,) if inp.dim() == 1 else (n_rows, width)
     out = torch.empty(shape, dtype=torch.float32, device=inp.device)
     with torch.cuda.device(inp.device):
-        st = lib.cxg_narrow_gather_sum_f32(ptr.data_ptr(), _lib.ptr(sel), _lib.ptr(inp), _lib.ptr(out),
-                                           n_rows, width, _lib.current_stream(inp.device))
+        if rows32 is not None and width in (1, 2, 4, 8):
+            _req(rows32, "rows32", torch.int32, 1)
+            n_edges = rows32.shape[0]
+            ws = _workspace(lib.cxg_segment_gather_sum_workspace_bytes(n_edges, width), inp.device)
+            st = lib.cxg_segment_gather_sum_f32(_lib.ptr(rows32), ptr.data_ptr(), _lib.ptr(sel), _lib.ptr(inp),
+                                                _lib.ptr(out), n_rows, n_edges, width, ws.data_ptr(), ws.numel(),
+                                                _lib.current_stream(inp.device))
+        else:
+            st = lib.cxg_narrow_gather_sum_f32(ptr.data_ptr(), _lib.ptr(sel), _lib.ptr(inp), _lib.ptr(out),
+                                               n_rows, width, _lib.current_stream(inp.device))
     _lib.check(st)
     return out
 

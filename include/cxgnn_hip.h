@@ -185,6 +185,25 @@ int cxg_edge_softmax_bwd_f32(const int64_t* ptr, const float* out, const uint8_t
 int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const float* in,
                               float* out, int64_t n_rows, int width, void* stream);
 
+/*
+ * The same row sums, edge-parallel: rows[k] (int32) is the row of edge position
+ * ptr[0] + k for k in [0, n_edges), n_edges = ptr[n_rows] - ptr[0] (see
+ * cxg_csr_row_ids_i32); every lane owns one edge, the values of 64 edges are
+ * summed per row with a segmented scan, rows crossing a span of edges are
+ * completed by a fix-up kernel (deterministic, no atomics).  width in
+ * {1, 2, 4, 8}; `in` and `out` aligned to one item.  Rows without edges give 0.
+ * Same reference code as cxg_narrow_gather_sum_f32 (src/cpp/src/edge_softmax.cu:83-95,
+ * 216-232); this form keeps every lane busy on power-law graphs.
+ */
+size_t cxg_segment_gather_sum_workspace_bytes(int64_t n_edges, int width);
+int cxg_segment_gather_sum_f32(const int32_t* rows, const int64_t* ptr, const int64_t* sel,
+                               const float* in, float* out, int64_t n_rows, int64_t n_edges,
+                               int width, void* workspace, size_t workspace_bytes, void* stream);
+
+/* rows[k] = row containing edge position ptr[0] + k, as int32 (n_rows < 2^31). */
+int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int32_t* rows,
+                        void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Typed (relation-segmented) GEMM -- the MFMA path                            */
 /* ------------------------------------------------------------------------- */
