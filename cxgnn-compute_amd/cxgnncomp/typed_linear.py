@@ -50,14 +50,7 @@ def TypedLinearS2DPushOP(x, weights, types, src, dst, num_type, num_center, num_
 
 def _weight_grad(x_rows, g_rows, perm, seg, shape):
     """grad_W[r] = X_r^T G_r over the rows of relation r (rows given in original order)."""
-    gw = torch.zeros(shape, dtype=torch.float32, device=x_rows.device)
-    bounds = seg.tolist()
-    for r in range(shape[0]):
-        b, e = bounds[r], bounds[r + 1]
-        if e > b:
-            sel = perm[b:e].contiguous()
-            gw[r] = torch.mm(_ops.gather_rows(x_rows, sel).t(), _ops.gather_rows(g_rows, sel))
-    return gw
+    return _typed._weight_grad(x_rows, g_rows, perm, perm, seg, shape)
 
 
 class TypedLinearE2EOP(torch.autograd.Function):
@@ -151,14 +144,7 @@ class TypedLinearS2EOP(torch.autograd.Function):
             _typed.typed_gemm(grad_out, torch.transpose(weights, 1, 2).contiguous(), seg, n, src_idx=perm,
                               dst_idx=src_idx[perm], out=grad_x, atomic=True)
         if ctx.needs_input_grad[1]:
-            grad_w = torch.zeros_like(weights)
-            bounds = seg.tolist()
-            for r in range(weights.shape[0]):
-                b, e = bounds[r], bounds[r + 1]
-                if e > b:
-                    sel = perm[b:e].contiguous()
-                    xs = _ops.gather_rows(x, src_idx[sel].contiguous())
-                    grad_w[r] = torch.mm(xs.t(), _ops.gather_rows(grad_out, sel))
+            grad_w = _typed._weight_grad(x, grad_out, src_idx[perm].contiguous(), perm, seg, weights.shape)
         return grad_x, grad_w, None, None, None, None, None
 
 

@@ -50,6 +50,9 @@ SIGNATURES = {
     "cxg_csr_row_ids_i64": (_I32, [_P, _I64, _I64, _P, _P]),
     "cxg_edge_value_degree_f32": (_I32, [_P, _I64, _P, _P]),
     "cxg_pad_rel_i64": (_I32, [_P, _P, _P, _I32, _I32, _I64, _P]),
+    "cxg_typed_gemm_wgrad_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32]),
+    "cxg_typed_gemm_wgrad_f32": (_I32, [_P, _I64, _P, _I64, _P, _P, _P, _I64, _I32, _I32, _I32, _P, _U32, _P, _SZ,
+                                        _P]),
     "cxg_csr_row_ids_i32": (_I32, [_P, _I64, _I64, _P, _P]),
     "cxg_segment_gather_sum_workspace_bytes": (_SZ, [_I64, _I32]),
     "cxg_segment_gather_sum_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _P, _SZ, _P]),

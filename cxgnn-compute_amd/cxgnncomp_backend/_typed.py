@@ -175,9 +175,36 @@ def _edge_segments(ptr, idx, rel, n, num_rel):
     return n_edges, idx[:n_edges][perm], rows[perm], seg
 
 
+def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=None, precision=None):
+    """gw[r] = sum over the rows i of segment r of a[src(i)]^T (x) g[dst(i)] -> [num_rel, K, N]
+    (see cxg_typed_gemm_wgrad_f32).  Returns None for shapes the kernel does not take
+    (K > 128, or K / N not multiples of 4)."""
+    lib = _lib.load()
+    _req(a, "a", torch.float32, 2)
+    _req(g, "g", torch.float32, 2)
+    K, N = a.shape[1], g.shape[1]
+    if K > 128 or K % 4 or N % 4:
+        return None
+    precision = precision or GEMM_PRECISION
+    flags = GEMM_SPLIT_BF16X3 if precision == "split3" else GEMM_SPLIT_BF16X6
+    gw = torch.empty((num_rel, K, N), dtype=torch.float32, device=a.device)
+    ws = _workspace(lib.cxg_typed_gemm_wgrad_workspace_bytes(m_rows, K, N, num_rel), a.device)
+    with torch.cuda.device(a.device):
+        st = lib.cxg_typed_gemm_wgrad_f32(a.data_ptr(), K, g.data_ptr(), N, _lib.ptr(src_idx), _lib.ptr(dst_idx),
+                                          seg_ptr.data_ptr(), m_rows, K, N, num_rel, gw.data_ptr(), flags,
+                                          ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
+    _lib.check(st)
+    return gw
+
+
 def _weight_grad(x, g, src, dst, seg, shape):
-    """grad_W[r] = sum over the rows of segment r of x[src]^T g[dst]; the row
-    gather is ours, the K x cnt x N product per relation is a plain library GEMM."""
+    """grad_W[r] = sum over the rows of segment r of x[src]^T g[dst]: one launch of the
+    typed weight-gradient kernel; shapes it does not take use a row gather plus one
+    library GEMM per relation."""
+    x, g = x.contiguous(), g.contiguous()
+    gw = typed_gemm_wgrad(x, g, seg, src.shape[0], shape[0], src_idx=src, dst_idx=dst)
+    if gw is not None:
+        return gw
     gw = torch.zeros(shape, dtype=torch.float32, device=x.device)
     bounds = seg.tolist()
     for r in range(shape[0]):
@@ -299,7 +326,10 @@ class _RgcnFusedFunction(torch.autograd.Function):
             if ctx.needs_input_grad[3]:
                 # gY[s, r] = sum of g over the edges (s -> d) of relation r; gW[r] = x^T gY[:, r]
                 gy = _ops.spmm(rg.ptr_key, rg.idx_key, grad_out, n_src * R)      # [n_src*R, N]
-                gw = torch.mm(x.t(), gy.view(n_src, R * N)).view(K, R, N).permute(1, 0, 2).contiguous()
+                gw = typed_gemm_wgrad(x, gy.view(n_src, R * N), _dense_seg(n_src, x.device), n_src, 1)
+                if gw is None:
+                    gw = torch.mm(x.t(), gy.view(n_src, R * N))
+                gw = gw.view(K, R, N).permute(1, 0, 2).contiguous()
             return gx, None, None, gw, None, None, None
         src, dst, seg = ctx.saved_tensors[3:]
         if ctx.needs_input_grad[0]:

@@ -247,6 +247,25 @@ int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, flo
                         unsigned flags, void* stream);
 
 /*
+ * Weight gradient of the typed GEMM: gw[r] (K x N, fp32, overwritten) = sum over
+ * the rows i of segment r of A[src(i), :]^T (x) G[dst(i), :]; relations without
+ * rows give zeros.  A is [*, K] (row stride lda), G is [*, N] (row stride ldg);
+ * src / dst / seg_ptr as in cxg_typed_gemm_f32.  fp32 operands multiplied as six
+ * (CXG_GEMM_SPLIT_BF16X6 or no flag) or three (CXG_GEMM_SPLIT_BF16X3) bf16 partial
+ * products on v_mfma_f32_32x32x16_bf16; partial sums over row chunks are added in
+ * chunk order by a second kernel (deterministic).  Needs K <= 128, K, N, lda, ldg
+ * multiples of 4 and 16-byte aligned operands (otherwise CXG_ERR_UNSUPPORTED).
+ * Replaces the per-relation torch.mm of TypedLinearE2EOP.backward and
+ * TypedLinearS2DMMAggrOP.backward (cxgnncomp/typed_linear.py:114-137,205-221).
+ */
+size_t cxg_typed_gemm_wgrad_workspace_bytes(int64_t M, int K, int N, int R);
+int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_t ldg,
+                             const int64_t* src_idx, const int64_t* dst_idx,
+                             const int64_t* seg_ptr, int64_t M, int K, int N, int R, float* gw,
+                             unsigned flags, void* workspace, size_t workspace_bytes,
+                             void* stream);
+
+/*
  * Relation segmentation: perm[k] = original row of the k-th row in relation
  * order (stable), seg_ptr[r] = number of rows with relation id < r for r in
  * [0, num_rel].  Ids equal to num_rel (the padding sentinel of pad_rel) sort
