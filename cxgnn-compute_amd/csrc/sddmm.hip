@@ -192,6 +192,107 @@ __global__ __launch_bounds__(kBlock) void sddmm_coo_packed_kernel(SddmmArgs a) {
   }
 }
 
+// Tiled-output variants of the packed kernels for GROUP = channels / V in
+// {8, 16, 32, 64} lanes per head.  After the lane-group reduction every lane of
+// a group holds the (edge, head) product; instead of one 4-byte store per edge
+// by the group leader (61.9M single-lane store instructions at the GAT shape),
+// lane q of the group keeps the products of the edges q, GROUP + q, ... of the
+// 64-edge step in registers, and the step ends with 64 / GROUP wave-wide stores
+// that each cover 64 consecutive floats of `out`.
+template <int V, int GROUP, bool COO>
+__global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(SddmmArgs a) {
+  using vec_t = typename Vec<V>::type;
+  constexpr int S = CXG_WAVE / GROUP;                 // products kept per lane and step
+  constexpr int U = COO ? 4 : (V == 4 ? 8 : 4);       // gathers in flight (measured optimum)
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t n_rows = a.n_rows;
+  const int64_t e_begin = COO ? 0 : a.ptr[0];
+  const int64_t e_end = COO ? a.n_edges : a.ptr[n_rows];
+  const int64_t e0 = e_begin + s * kSpan;
+  if (e0 >= e_end) return;
+  const int n = (int)((e_end - e0) < (int64_t)kSpan ? (e_end - e0) : (int64_t)kSpan);
+  const int F = a.heads * a.channels;
+  const bool active = lane * V < F;
+  const int head = lane / GROUP;
+  const int q = lane % GROUP;
+  const int bcol = a.b_heads ? lane * V : q * V;
+  const int64_t ldb = a.b_heads ? F : a.channels;
+
+  // CSR form: row containing e0 and the ends of the next 64 rows, relative to e0
+  int64_t r = 0, rbase = 0;
+  int row_ends = 0, cur_end = 0;
+  vec_t brow = vzero<V>();
+  auto load_row_ends = [&](int64_t rb) -> int {
+    int64_t k = rb + 1 + lane;
+    if (k > n_rows) k = n_rows;
+    const int64_t d = (int64_t)a.ptr[k] - e0;
+    return (int)(d < (int64_t)n + 1 ? d : (int64_t)n + 1);
+  };
+  if (!COO) {
+    r = wave_lower_bound(a.ptr, n_rows + 1, e0 + 1) - 1;
+    rbase = r;
+    row_ends = load_row_ends(rbase);
+    cur_end = bcast_i32(row_ends, 0);
+    if (active) brow = *reinterpret_cast<const vec_t*>(a.b + r * ldb + bcol);
+  }
+
+  for (int c0 = 0; c0 < n; c0 += CXG_WAVE) {
+    const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
+    int64_t my_src = 0, my_dst = 0;
+    if (lane < cn) {
+      my_src = COO ? a.src[e0 + c0 + lane] : a.idx[e0 + c0 + lane];
+      if (COO) my_dst = a.dst[e0 + c0 + lane];
+    }
+    float res[S];
+#pragma unroll
+    for (int t = 0; t < S; ++t) res[t] = 0.f;
+#pragma unroll
+    for (int t = 0; t < S; ++t) {
+      if (t * GROUP >= cn) break;
+      for (int b0 = 0; b0 < GROUP; b0 += U) {
+        vec_t va[U], vb[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int jj = t * GROUP + b0 + u;
+          if (jj < cn) {
+            const int64_t src = bcast_i64(my_src, jj);
+            va[u] = active ? *reinterpret_cast<const vec_t*>(a.a + src * F + lane * V) : vzero<V>();
+            if (COO) {
+              const int64_t dst = bcast_i64(my_dst, jj);
+              vb[u] = active ? *reinterpret_cast<const vec_t*>(a.b + dst * ldb + bcol) : vzero<V>();
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int jj = t * GROUP + b0 + u;
+          if (jj < cn) {
+            if (!COO) {
+              const int j = c0 + jj;
+              while (j >= cur_end) {
+                ++r;
+                if (r - rbase == CXG_WAVE) { rbase = r; row_ends = load_row_ends(rbase); }
+                cur_end = bcast_i32(row_ends, (int)(r - rbase));
+                if (j < cur_end)
+                  brow = active ? *reinterpret_cast<const vec_t*>(a.b + r * ldb + bcol) : vzero<V>();
+              }
+            }
+            const float p = group_sum(vdot(va[u], COO ? vb[u] : brow), GROUP);
+            if (q == b0 + u) res[t] = p;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < S; ++t) {
+      const int jj = t * GROUP + q;
+      if (active && jj < cn) a.out[(e0 + c0 + jj) * a.heads + head] = res[t];
+    }
+  }
+}
+
 // General layout (any heads / channels): one wave-wide reduction per (edge, head).
 // COO == false walks CSR rows (dst = row), COO == true reads src/dst arrays.
 template <bool COO>
@@ -244,6 +345,21 @@ int packed_vec(const SddmmArgs& a) {
   return 0;
 }
 
+// Launches the tiled-output kernel when the group width has an instantiation.
+template <bool COO>
+bool launch_tiled(const SddmmArgs& a, int v, dim3 grid, dim3 block, hipStream_t st) {
+#define CXG_TILED(VV, GG)                                                                   \
+  if (v == VV && a.group == GG) {                                                           \
+    hipLaunchKernelGGL((sddmm_tiled_kernel<VV, GG, COO>), grid, block, 0, st, a);           \
+    return true;                                                                            \
+  }
+  CXG_TILED(4, 8) CXG_TILED(4, 16) CXG_TILED(4, 32) CXG_TILED(4, 64)
+  CXG_TILED(2, 8) CXG_TILED(2, 16) CXG_TILED(2, 32) CXG_TILED(2, 64)
+  CXG_TILED(1, 8) CXG_TILED(1, 16) CXG_TILED(1, 32) CXG_TILED(1, 64)
+#undef CXG_TILED
+  return false;
+}
+
 int check_common(const float* a, const float* b, float* out, int heads, int channels) {
   CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
   CXG_REQUIRE(a && b && out, CXG_ERR_ARG, "null feature/output pointer");
@@ -272,7 +388,8 @@ int cxg_sddmm_csr_f32(const int64_t* ptr, const int64_t* idx, const float* src_f
   dim3 block(cxg::kBlock);
   const int v = cxg::packed_vec(a);
   if (v) a.group = channels / v;
-  if (v == 4) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<4>, grid, block, 0, st, a);
+  if (v && cxg::launch_tiled<false>(a, v, grid, block, st)) { /* coalesced-output form */ }
+  else if (v == 4) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<4>, grid, block, 0, st, a);
   else if (v == 2) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<2>, grid, block, 0, st, a);
   else if (v == 1) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<1>, grid, block, 0, st, a);
   else hipLaunchKernelGGL(cxg::sddmm_general_kernel<false>, grid, block, 0, st, a);
@@ -297,7 +414,8 @@ int cxg_sddmm_coo_f32(const int64_t* src, const int64_t* dst, const float* src_f
   dim3 block(cxg::kBlock);
   const int v = cxg::packed_vec(a);
   if (v) a.group = channels / v;
-  if (v == 4) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<4>, grid, block, 0, st, a);
+  if (v && cxg::launch_tiled<true>(a, v, grid, block, st)) { /* coalesced-output form */ }
+  else if (v == 4) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<4>, grid, block, 0, st, a);
   else if (v == 2) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<2>, grid, block, 0, st, a);
   else if (v == 1) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<1>, grid, block, 0, st, a);
   else hipLaunchKernelGGL(cxg::sddmm_general_kernel<true>, grid, block, 0, st, a);
