@@ -30,6 +30,7 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 constexpr int kBM = 64;
 constexpr int kThreads = 256;
+constexpr int kXcds = 8;                 // accelerator dies of an MI355X, one L2 each
 
 struct GemmArgs {
   const void* a;
@@ -302,11 +303,15 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
   const int64_t span = (int64_t)kBM * G;
   int rel = -1;
   int64_t row0 = 0, row_end = 0;
-  // Column tiles vary fastest over the block index, so the blocks that read the
-  // same A rows run at the same time and share them through the caches.
+  // Blocks are handed to the 8 XCDs round-robin by block index and every XCD has
+  // its own L2: the column tiles of one row chunk are given consecutive slots of
+  // ONE XCD (chunk = 8 * (slot / n_ct) + xcd), so the chunk's A rows are fetched
+  // into a single L2 once and shared by the blocks that run there together.
   const int n_ct = (g.N + 127) / 128;
+  const int64_t slot = blockIdx.x / kXcds;
+  const int64_t chunk = (slot / n_ct) * kXcds + (blockIdx.x % kXcds);
   {
-    int64_t t = blockIdx.x / n_ct;
+    int64_t t = chunk;
     for (int r = 0; r < g.R; ++r) {
       const int64_t b = g.seg[r], e = g.seg[r + 1];
       const int64_t nt = (e - b + span - 1) / span;
@@ -316,7 +321,7 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
   }
   if (rel < 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = (int)(blockIdx.x % n_ct) * 128;
+  const int n0 = (int)(slot % n_ct) * 128;
   const int K = g.K, N = g.N;
   const int64_t rows_here = (row_end - row0) < span ? (row_end - row0) : span;
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
@@ -451,7 +456,8 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
     // 64*G rows per block: up to 32 tiles while the launch keeps a few thousand blocks
     int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));
     G = G < 1 ? 1 : (G > 32 ? 32 : G);
-    const int64_t n_blocks = (cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R) * cxg::ceil_div(N, 128);
+    const int64_t n_chunks = cxg::ceil_div(cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R, cxg::kXcds) * cxg::kXcds;
+    const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
     CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
     const dim3 grid((unsigned)n_blocks);
 #define CXG_SPLIT(KS)                                                                          \

@@ -31,6 +31,7 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
+constexpr int kXcds = 8;                 // accelerator dies of an MI355X, one L2 each
 constexpr int kMT = 32;                  // rows per step
 constexpr int kMP = kMT + 8;             // padded row extent in LDS (bf16 elements): 80-byte pitch
 
@@ -75,9 +76,12 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
   __shared__ __attribute__((aligned(16))) uint16_t At[NS][128][kMP];   // [part][k][row]
   __shared__ __attribute__((aligned(16))) uint16_t Gt[NS][128][kMP];   // [part][n][row]
   __shared__ int64_t s_src[3][kMT], s_dst[3][kMT];
+  // The column tiles of one row chunk get consecutive slots of one XCD (blocks go to
+  // the 8 XCDs round-robin by index), so the chunk's A rows are fetched into one L2.
   const int n_ct = (g.N + 127) / 128;
-  const int64_t chunk = blockIdx.x / n_ct;
-  const int n0 = (int)(blockIdx.x % n_ct) * 128;
+  const int64_t slot = blockIdx.x / kXcds;
+  const int64_t chunk = (slot / n_ct) * kXcds + (blockIdx.x % kXcds);
+  const int n0 = (int)(slot % n_ct) * 128;
   int rel = 0;
   int64_t row0 = 0, row_end = 0;
   const bool have = locate_chunk(g.seg, g.R, g.rows_per_chunk, chunk, rel, row0, row_end);
@@ -221,7 +225,7 @@ extern "C" {
 
 size_t cxg_typed_gemm_wgrad_workspace_bytes(int64_t M, int K, int N, int R) {
   if (M < 0 || K < 1 || N < 1 || R < 1) return 0;
-  const int64_t chunks = cxg::ceil_div(M, cxg::chunk_rows(M, N)) + R;
+  const int64_t chunks = cxg::ceil_div(cxg::ceil_div(M, cxg::chunk_rows(M, N)) + R, cxg::kXcds) * cxg::kXcds;
   return (size_t)chunks * (size_t)K * (size_t)N * sizeof(float) + 256;
 }
 
@@ -243,7 +247,7 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
   CXG_REQUIRE(((uintptr_t)workspace & 255) == 0, CXG_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int64_t rows = cxg::chunk_rows(M, N);
-  const int64_t chunks = cxg::ceil_div(M, rows) + R;
+  const int64_t chunks = cxg::ceil_div(cxg::ceil_div(M, rows) + R, cxg::kXcds) * cxg::kXcds;
   const int n_ct = (int)cxg::ceil_div(N, 128);
   CXG_REQUIRE(chunks * n_ct < ((int64_t)1 << 31), CXG_ERR_UNSUPPORTED, "too many chunks for one launch");
   cxg::WgradArgs wa{a, lda, g, ldg, src_idx, dst_idx, seg_ptr, reinterpret_cast<float*>(workspace),
