@@ -153,6 +153,27 @@ def c2(iters):
         bench_aggregation("c2", ptr, idx, 169343, 169343, f, iters)
         if CPU_BASELINE:
             cpu_spmm("c2", ptr, idx, 169343, f, 169343)
+    # the configuration's model: 3 GCN layers 128 -> 256 -> 256 -> 40, BatchNorm + ReLU between
+    import cxgnncomp
+    cxgnncomp.set_timers()                       # MyGCNConv brackets its phases with TimerOP, as upstream
+    n = 169343
+    x = torch.randn(n, 128, device="cuda")
+    for normalize in (False, True):
+        convs = [cxgnncomp.MyGCNConv(128, 256, normalize).cuda(), cxgnncomp.MyGCNConv(256, 256, normalize).cuda(),
+                 cxgnncomp.MyGCNConv(256, 40, normalize).cuda()]
+        bns = [torch.nn.BatchNorm1d(256).cuda(), torch.nn.BatchNorm1d(256).cuda()]
+        xg = x.clone().requires_grad_(True)
+
+        def step():
+            xg.grad = None
+            h = xg
+            for li, conv in enumerate(convs):
+                h = conv(h, ptr, idx, n)
+                if li < 2:
+                    h = torch.relu(bns[li](h))
+            h.sum().backward()
+        report("c2", "3-layer GCN fwd+bwd, %s aggregation" % ("1/deg-weighted" if normalize else "sum"),
+               timeit(step, iters))
 
 
 def c3(iters):
@@ -194,8 +215,20 @@ def c3(iters):
     report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),
            E * (8 * H * C + 16) + 4 * E * H, 2 * E * H * C)
     del x, g
-    # scheduling helpers (index work): bytes = arrays read + written once
+    # the configuration's layer: GAT 128 -> 4 heads x 64, forward + backward through the
+    # softmax and the edge-weighted aggregation including the edge-value gradient
     import cxgnncomp
+    cxgnncomp.set_timers()
+    layer = cxgnncomp.MyGATConv(128, 64, heads=4, concat=True).cuda()
+    xin = torch.randn(N, 128, device="cuda").requires_grad_(True)
+
+    def gat_step():
+        xin.grad = None
+        layer(xin, ptr, idx, N, N, E).sum().backward()
+    report("c3", "MyGATConv 128 -> 4x64 fwd+bwd (linear, softmax, SpMM, SDDMM)", timeit(gat_step, max(2, iters // 3)))
+    del layer, xin
+    torch.cuda.empty_cache()
+    # scheduling helpers (index work): bytes = arrays read + written once
     new_ptr, _ = cxgnncomp.neighbor_grouping(ptr, 32)
     n_groups = new_ptr.shape[0] - 1
     report("c3", "neighbor_grouping thres=32 (%d groups)" % n_groups,

@@ -428,6 +428,116 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
   }
 }
 
+// ----------------------------------------------------------------------------
+// bf16 operands, K <= 128: the same block structure as the split kernel
+// ----------------------------------------------------------------------------
+// A block owns up to G consecutive 64-row tiles of one relation and keeps the
+// relation's W^T slab (its 32 columns per wave) in registers in B-operand layout
+// -- one 16-byte load per k-step straight from W^T [R, N, K]; A rows are fetched
+// as 16-byte-per-lane segments (8 bf16) and go to LDS unchanged; the loads of the
+// next two tiles are in flight while the current one is multiplied.
+template <int KS>
+__global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(GemmArgs g, int G) {
+  constexpr int KP = KS * 16 + 8;          // padded LDS row (bf16 elements)
+  constexpr int LPR = KS * 2;              // lanes per A row, 8 bf16 each
+  constexpr int RPI = kThreads / LPR;      // rows per load instruction
+  constexpr int NLD = kBM / RPI;           // load instructions per tile
+  __shared__ __attribute__((aligned(16))) uint16_t Ap[kBM][KP];
+  __shared__ int64_t s_src[3][kBM], s_dst[3][kBM];
+  const int64_t span = (int64_t)kBM * G;
+  int rel = -1;
+  int64_t row0 = 0, row_end = 0;
+  const int n_ct = (g.N + 127) / 128;
+  const int64_t slot = blockIdx.x / kXcds;
+  const int64_t chunk = (slot / n_ct) * kXcds + (blockIdx.x % kXcds);   // see typed_gemm_split_kernel
+  {
+    int64_t t = chunk;
+    for (int r = 0; r < g.R; ++r) {
+      const int64_t b = g.seg[r], e = g.seg[r + 1];
+      const int64_t nt = (e - b + span - 1) / span;
+      if (t < nt) { rel = r; row0 = b + t * span; row_end = e; break; }
+      t -= nt;
+    }
+  }
+  if (rel < 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = (int)(slot % n_ct) * 128;
+  const int K = g.K, N = g.N;
+  const int64_t rows_here = (row_end - row0) < span ? (row_end - row0) : span;
+  const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
+
+  v8bf bw[KS];
+  {
+    const uint16_t* Wt = reinterpret_cast<const uint16_t*>(g.w) + (int64_t)rel * N * K;
+    const int col = n0 + wave * 32 + (lane & 31);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int k = s * 16 + (lane >> 5) * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (col < N && k < K) v = *reinterpret_cast<const uint4*>(Wt + (int64_t)col * K + k);
+      bw[s] = *reinterpret_cast<const v8bf*>(&v);
+    }
+  }
+
+  const int c8 = tid % LPR, rsub = tid / LPR;
+  const bool k_ok = 8 * c8 < K;
+  const uint16_t* A = reinterpret_cast<const uint16_t*>(g.a);
+  auto load_maps = [&](int t) {
+    if (tid < kBM && t < n_tiles) {
+      const int64_t gr = row0 + (int64_t)t * kBM + tid;
+      int64_t sidx = -1, didx = -1;
+      if (gr < row_end) {
+        sidx = g.src ? g.src[gr] : gr;
+        didx = g.dst ? g.dst[gr] : gr;
+        if (sidx < 0 || didx < 0) { sidx = -1; didx = -1; }
+      }
+      s_src[t % 3][tid] = sidx;
+      s_dst[t % 3][tid] = didx;
+    }
+  };
+  auto gload = [&](uint4 (&areg)[NLD], int t) {
+    if (t >= n_tiles) return;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int64_t sidx = s_src[t % 3][i * RPI + rsub];
+      areg[i] = (sidx >= 0 && k_ok) ? *reinterpret_cast<const uint4*>(A + sidx * g.lda + 8 * c8)
+                                    : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  auto tile_step = [&](uint4 (&areg)[NLD], int t) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) *reinterpret_cast<uint4*>(&Ap[i * RPI + rsub][8 * c8]) = areg[i];
+    load_maps(t + 2);
+    __syncthreads();
+    gload(areg, t + 2);
+    v16f acc[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const v8bf a = *reinterpret_cast<const v8bf*>(&Ap[mt * 32 + (lane & 31)][s * 16 + (lane >> 5) * 8]);
+        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bw[s], acc[mt], 0, 0, 0);
+      }
+    }
+    store_tile<128, 2>(g, acc, s_dst[t % 3], 0, wave, lane, n0);
+    __syncthreads();
+  };
+  uint4 areg0[NLD], areg1[NLD];
+  load_maps(0);
+  load_maps(1);
+  __syncthreads();
+  gload(areg0, 0);
+  gload(areg1, 1);
+  for (int t = 0; t < n_tiles; t += 2) {
+    tile_step(areg0, t);
+    if (t + 1 < n_tiles) tile_step(areg1, t + 1);
+  }
+}
+
 int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64_t M, int K, int N,
                int R, unsigned flags) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
@@ -497,6 +607,19 @@ int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, flo
   cxg::GemmArgs g{a, lda, w_t, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
                   (int)(flags & 1u), (int)((flags >> 1) & 1u)};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (K <= 128) {
+    int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));
+    G = G < 1 ? 1 : (G > 32 ? 32 : G);
+    const int64_t n_chunks = cxg::ceil_div(cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R, cxg::kXcds) * cxg::kXcds;
+    const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
+    CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
+    const dim3 grid((unsigned)n_blocks), block(cxg::kThreads);
+    if (K <= 32) hipLaunchKernelGGL(cxg::typed_gemm_bf16_resident_kernel<2>, grid, block, 0, st, g, G);
+    else if (K <= 64) hipLaunchKernelGGL(cxg::typed_gemm_bf16_resident_kernel<4>, grid, block, 0, st, g, G);
+    else hipLaunchKernelGGL(cxg::typed_gemm_bf16_resident_kernel<8>, grid, block, 0, st, g, G);
+    CXG_LAUNCH_CHECK("typed_gemm_bf16_resident_kernel");
+    return CXG_OK;
+  }
   const unsigned tiles = (unsigned)(cxg::ceil_div(M, cxg::kBM) + R);
   if (N > 64) {
     hipLaunchKernelGGL(cxg::typed_gemm_bf16_kernel<128>, dim3(tiles, (unsigned)cxg::ceil_div(N, 128)),

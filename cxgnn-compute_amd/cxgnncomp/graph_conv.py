@@ -369,6 +369,8 @@ class MyGCNConv(torch.nn.Module):
 
     def gcn_norm(self, ptr, idx):
         """1 / in-degree per edge, 0 where the degree is 0 (upstream :587-596)."""
+        if ptr.is_cuda:
+            return cxgnncomp_backend.edge_value_degree(ptr, ptr.shape[0] - 1, idx.shape[0])
         deg = ptr[1:] - ptr[:-1]
         edge_value = deg.repeat_interleave(deg).float().pow(-1)
         edge_value.masked_fill_(edge_value == float("inf"), 0.0)
