@@ -342,6 +342,13 @@ def c5(iters):
     for li, (rows, edges) in enumerate(zip(nn[2::-1], ne[::-1])):
         report("c5", "sage_mean_forward rows=%d edges=%d F=128" % (rows, edges),
                timeit(lambda: B.sage_mean_forward(x, ptr, idx, rows), iters), spmm_bytes(rows, edges, 128), edges * 128)
+    from cxgnncomp_backend import _ops
+
+    def prepare():
+        # what a NEW batch pays once before its first backward: the reversed graph of each layer
+        for rows in nn[2::-1]:
+            _ops.csr_transpose(ptr, idx, rows, n_src)
+    report("c5", "per-batch preparation: reversed CSR of the 3 layers (stable sort + fills)", timeit(prepare, iters))
     xg = x.clone().requires_grad_(True)
 
     def batch_step():
