@@ -261,9 +261,27 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   const int64_t row_begin = (int64_t)a.ptr[t];
   const int64_t row_end = (int64_t)a.ptr[t + 1];
   const int64_t s_last = (row_end - 1 - e_begin) / T;
+  // Head partials of the following spans, 16 independent loads at a time (a row that
+  // covers thousands of spans would otherwise be one long chain of dependent loads);
+  // the 16 running sums are combined in a fixed order, so the result is deterministic.
+  constexpr int kChain = 16;
+  vec_t part[kChain];
+#pragma unroll
+  for (int u = 0; u < kChain; ++u) part[u] = vzero<V>();
+  int64_t q = s + 1;
+  for (; q + kChain - 1 <= s_last; q += kChain) {      // whole groups: no guards, loads cluster
+    vec_t got[kChain];
+#pragma unroll
+    for (int u = 0; u < kChain; ++u)
+      got[u] = *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * (q + u)) * F + col);
+#pragma unroll
+    for (int u = 0; u < kChain; ++u) vadd(part[u], got[u]);
+  }
+  for (; q <= s_last; ++q)
+    vadd(part[0], *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * q) * F + col));
   vec_t acc = *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * s + 1) * F + col);
-  for (int64_t q = s + 1; q <= s_last; ++q)
-    vadd(acc, *reinterpret_cast<const vec_t*>(a.carry + (size_t)(2 * q) * F + col));
+#pragma unroll
+  for (int u = 0; u < kChain; ++u) vadd(acc, part[u]);
   if (a.targets) {
     atomic_add_vec(a.out + a.targets[t] * a.ldo + col, acc);
     return;

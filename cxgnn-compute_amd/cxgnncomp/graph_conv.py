@@ -13,6 +13,7 @@ import torch.nn.functional as F
 from torch.nn import Parameter
 
 import cxgnncomp_backend
+from cxgnncomp_backend import _typed
 from cxgnncomp_backend import (aggr_rel, aggr_rgcn_direct_func, edge_attention, gather,
                                sage_mean_forward, sage_sum_forward, sage_sum_forward_edge_value,
                                selective_aggr, selective_aggr_bwd)
@@ -237,6 +238,59 @@ class MyRGCNConv(torch.nn.Module):
         return cxgnncomp_backend.aggr_rgcn_mean(x, ptr, idx, self.linear, edge_types, num_node)
 
 
+_ARANGE = {}
+
+
+def _arange_ptr(n, device):
+    key = (int(n), str(device))
+    if key not in _ARANGE:
+        if len(_ARANGE) > 8:
+            _ARANGE.clear()
+        _ARANGE[key] = (torch.tensor([0, int(n)], dtype=torch.int64, device=device),
+                        torch.arange(int(n), dtype=torch.int64, device=device))
+    return _ARANGE[key]
+
+
+class HeadDotOP(torch.autograd.Function):
+    """alpha[n, h] = sum_c x[n, h, c] * att[h, c]: upstream's ``(x * att).sum(dim=-1)``
+    (cxgnncomp/graph_conv.py:460-461) without the [N, H, C] temporaries.  On the GPU it is
+    the SDDMM of every node row against the single row ``att`` (a one-row CSR over all
+    nodes); its weight gradient is a [H, N] x [N, H*C] product on the typed weight-gradient
+    kernel.  Host tensors use the upstream expression."""
+
+    @staticmethod
+    def forward(ctx, x, att):
+        ctx.save_for_backward(x, att)
+        if not x.is_cuda:
+            return (x * att).sum(dim=-1)
+        n, heads, channels = x.shape
+        ptr, ar = _arange_ptr(n, x.device)
+        return cxgnncomp_backend._ops.sddmm_csr(ptr, ar, x.contiguous(),
+                                                att.reshape(1, heads, channels).contiguous(), 1)
+
+    @staticmethod
+    def backward(ctx, grad):
+        x, att = ctx.saved_tensors
+        grad = grad.contiguous()
+        gx = gatt = None
+        if ctx.needs_input_grad[0]:
+            gx = grad.unsqueeze(-1) * att
+        if ctx.needs_input_grad[1]:
+            gatt = None
+            if x.is_cuda:
+                # grad^T x on the matrix cores: [H, N] x [N, H*C]; head h's gradient is the
+                # h-th diagonal block of the [H, H*C] product
+                n, heads, channels = x.shape
+                seg = torch.tensor([0, n], dtype=torch.int64, device=x.device)
+                full = _typed.typed_gemm_wgrad(grad, x.contiguous().view(n, heads * channels), seg, n, 1)
+                if full is not None:
+                    full = full.view(heads, heads, channels)
+                    gatt = torch.stack([full[h, h] for h in range(heads)]).view_as(att)
+            if gatt is None:
+                gatt = (grad.unsqueeze(-1) * x).sum(dim=0).view_as(att)
+        return gx, gatt
+
+
 class MyGATConv(torch.nn.Module):
 
     def __init__(self, in_channels, out_channels, heads=1, concat=False, negative_slope=0.2,
@@ -298,8 +352,8 @@ class MyGATConv(torch.nn.Module):
         x_src = x_dst = F.linear(x[:num_src], self.lin_src).view(-1, H, C)
         x_src = TimerOP.apply(x_src, "linear1", False)
         x_src = TimerOP.apply(x_src, "sum1", True)
-        alpha_src = (x_src * self.att_src).sum(dim=-1).view(-1, H)
-        alpha_dst = (x_dst[:num_dst] * self.att_dst).sum(dim=-1).view(-1, H)
+        alpha_src = HeadDotOP.apply(x_src, self.att_src).view(-1, H)
+        alpha_dst = HeadDotOP.apply(x_dst[:num_dst], self.att_dst).view(-1, H)
         alpha_dst = TimerOP.apply(alpha_dst, "sum1", False)
         alpha_dst = TimerOP.apply(alpha_dst, "softmax1", True)
         edge_value = self.edge_softmax(ptr=ptr, idx=idx, att_src=alpha_src, att_dst=alpha_dst,
