@@ -361,7 +361,9 @@ def c5(iters):
             if li < 2:
                 h = torch.relu(h)
         h.sum().backward()
-    report("c5", "3-layer SAGE fwd+bwd per batch (%s nodes per layer)" % nn, timeit(batch_step, iters))
+    report("c5", "3-layer SAGE fwd+bwd per batch (%s nodes per layer)" % nn, timeit(batch_step, iters),
+           note="60 kernel launches per batch, 12 of them this library's (6 aggregations x span + fix-up); "
+                "counted with a rocprofv3 kernel trace of 10 vs 20 steps")
     if CPU_BASELINE:
         cpu_spmm("c5", ptr, idx, n_src, 128, nn[2])
 
