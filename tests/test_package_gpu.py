@@ -343,3 +343,25 @@ def test_schedule_helpers_on_gpu_tensors():
     a = cxgnncomp.remove_from_graph(ptr.cuda(), idx.cuda(), flag.cuda())
     b = cxgnncomp.remove_from_graph(ptr, idx, flag)
     assert torch.equal(a[0].cpu(), b[0]) and torch.equal(a[1].cpu(), b[1])
+
+
+@pytest.mark.parametrize("heads,channels", [(4, 64), (1, 128), (2, 16), (3, 10)])
+def test_head_dot_op(heads, channels):
+    """HeadDotOP == (x * att).sum(-1) with the gradients autograd gives that expression."""
+    from cxgnncomp.graph_conv import HeadDotOP
+    torch.manual_seed(heads * 100 + channels)
+    n = 5000
+    x = torch.randn(n, heads, channels) / channels ** 0.5
+    att = torch.randn(1, heads, channels)
+    g = torch.randn(n, heads) / n ** 0.5
+    xr, ar = x.double().requires_grad_(True), att.double().requires_grad_(True)
+    ((xr * ar).sum(-1) * g.double()).sum().backward()
+    xc, ac = x.cuda().requires_grad_(True), att.cuda().requires_grad_(True)
+    announce("HeadDotOP H=%d C=%d" % (heads, channels))
+    out = HeadDotOP.apply(xc, ac)
+    out.backward(g.cuda())
+    assert_close(_np(out), (x.double() * att.double()).sum(-1).numpy(), RTOL, ATOL, "head dot")
+    assert_close(_np(xc.grad), xr.grad.numpy(), RTOL, ATOL, "head dot grad x")
+    assert_close(_np(ac.grad), ar.grad.numpy(), RTOL, 2 * ATOL, "head dot grad att")
+    # host tensors take the upstream expression
+    assert torch.allclose(HeadDotOP.apply(x, att), (x * att).sum(-1))

@@ -205,3 +205,33 @@ def test_rgcn_fused_forward_backward(K, N, R, strategy, monkeypatch):
     assert_close(_np(so), ref, RTOL, 2 * ATOL, "seastar fwd")
     sgx, sgw = B.seastar_backward(x.cuda(), ptr.cuda(), idx.cuda(), w.cuda(), etype.cuda(), g.cuda())
     assert_close(_np(sgx) / scx, x64.grad.numpy() / scx, RTOL, 2 * ATOL, "seastar grad x")
+
+
+@pytest.mark.parametrize("K,N,R,M", [(128, 128, 16, 5000), (64, 48, 3, 1000), (4, 256, 1, 3000), (128, 2048, 1, 700),
+                                     (32, 40, 4, 70000), (12, 20, 5, 1)])
+def test_typed_gemm_wgrad(K, N, R, M):
+    """gw[r] = sum over the rows of relation r of a[src]^T (x) g[dst], against per-relation
+    float64 products; covers several column tiles (N = 2048), K far below one tile (K = 4),
+    many row chunks (M = 70000) and relations without rows."""
+    from cxgnncomp_backend import _typed
+    gen = torch.Generator().manual_seed(K + N + M)
+    n_a, n_g = max(1, M // 2), max(1, M // 3)
+    a = torch.randn(n_a, K, generator=gen)
+    g = torch.randn(n_g, N, generator=gen) / max(1.0, (M / R) ** 0.5)
+    src = torch.randint(0, n_a, (M,), generator=gen)
+    dst = torch.randint(0, n_g, (M,), generator=gen)
+    types = torch.randint(0, R, (M,), generator=gen).int()
+    if R > 2:
+        types[types == 1] = 0
+    perm, seg = _typed.rel_segment(types.cuda(), R)
+    announce("typed_gemm_wgrad K=%d N=%d R=%d M=%d" % (K, N, R, M))
+    gw = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg, M, R, src_idx=src.cuda()[perm], dst_idx=dst.cuda()[perm])
+    assert gw is not None and gw.shape == (R, K, N)
+    want = torch.zeros(R, K, N, dtype=torch.float64)
+    for r in range(R):
+        m = types == r
+        want[r] = a[src[m]].double().t() @ g[dst[m]].double()
+    assert_close(_np(gw), want.numpy(), RTOL, 2 * ATOL, "wgrad")
+    again = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg, M, R, src_idx=src.cuda()[perm], dst_idx=dst.cuda()[perm])
+    assert torch.equal(gw, again)                                   # deterministic
+    assert _typed.typed_gemm_wgrad(torch.zeros(4, 130).cuda(), g.cuda(), seg, 0, R) is None   # K > 128: not taken
