@@ -21,6 +21,9 @@
 namespace cxg {
 namespace {
 
+#ifndef CXG_SPMM_SPAN_DIV
+#define CXG_SPMM_SPAN_DIV 16384   // target number of spans for graphs too small for 512-edge spans
+#endif
 #ifndef CXG_SPMM_U
 #define CXG_SPMM_U 1
 #endif
@@ -295,7 +298,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
 // Span length: 512 edges for large graphs, shorter for small ones so that the
 // launch still has a few thousand waves.
 int choose_span(int64_t n_edges_cap) {
-  int64_t t = n_edges_cap / 16384;
+  int64_t t = n_edges_cap / CXG_SPMM_SPAN_DIV;
   t = (t + 63) / 64 * 64;
   if (t < 64) t = 64;
   if (t > 512) t = 512;
