@@ -2,8 +2,9 @@
 
 The hot-path names of the reference package (cxgnncomp/__init__.py:1-18) are
 importable from here and run on libcxgnn_hip.so through ``cxgnncomp_backend``.
-Model zoo, trainer and dataset loading of the reference need dgl / PyG / cxgnndl
-and are not part of this package.
+The model stacks (``SAGE``, ``GCN``, ``GIN``, ``GAT``, ``RGCN``) run the CSR graph types;
+trainer and dataset loading of the reference need dgl / PyG / cxgnndl and are not part of
+this package.
 """
 from .graph_conv import (MyGATConv, MyGCNConv, MySageConv, MyGINConv, MyRGCNConv, RGCNOP, RGCNOP2,
                          RGCNOP3, RGCNOP_sorted, AggrOP, AggrDirectedOP, SeastarRGCNOP, run_rgcn4)
@@ -19,4 +20,5 @@ from .schedule import (neighbor_grouping, neighbor_grouping_gpu, partition_2d, r
 from .batch import Batch, PyGBatch
 from .util import global_tuner
 from .graph_kernel import SpMMValOP
+from .model import GNN, SAGE, GCN, GIN, GAT, RGCN
 from . import synthetic  # noqa: F401
