@@ -13,6 +13,7 @@ from . import _lib
 
 SPMM_MEAN = 1
 SPMM_ACCUMULATE = 2
+SPMM_HINT_EXACT_EDGES = 4
 
 
 def as_int(v):
@@ -94,6 +95,8 @@ def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, 
     ws_bytes = lib.cxg_spmm_workspace_bytes(n_cap, row)
     ws = _workspace(ws_bytes, x.device)
     flags = (SPMM_MEAN if mean else 0) | (SPMM_ACCUMULATE if accumulate else 0)
+    if n_rows == ptr.shape[0] - 1:
+        flags |= SPMM_HINT_EXACT_EDGES       # all rows of ptr: idx holds exactly their edges
     stream = _lib.current_stream(x.device)
     with torch.cuda.device(x.device):
         if val is None:

@@ -50,6 +50,7 @@ const char* cxg_last_error(void);
 /* flags for cxg_spmm_* */
 #define CXG_SPMM_MEAN 1u       /* divide each row by its degree; empty rows stay 0 */
 #define CXG_SPMM_ACCUMULATE 2u /* out += result instead of out = result           */
+#define CXG_SPMM_HINT_EXACT_EDGES 4u /* n_edges_cap is the real edge count of the rows (tuning hint only) */
 
 /* Bytes of workspace needed by cxg_spmm_* for a graph whose idx array has
  * n_edges_cap entries and rows of `row_floats` floats (heads*channels). */
