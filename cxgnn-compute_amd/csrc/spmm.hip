@@ -242,6 +242,186 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   if (lane == 0 && blockIdx.y == 0) a.tail_row[s] = tail;
 }
 
+// ----------------------------------------------------------------------------
+// Narrow rows: several edges per gather instruction
+// ----------------------------------------------------------------------------
+// For rows of at most 32 * V floats a whole wave per edge leaves most lanes idle
+// and the kernel is bound by one gather instruction per edge (F <= 64 took the
+// same ~3.5 ms as F = 128 on the 61.9M-edge graph).  Here the wave is cut into
+// G = 64 / L groups of L lanes (L * V >= F): one step gathers G consecutive edges
+// of the current row, one per group, each group keeping its own partial sum; when
+// the row ends the partials are added across groups with xor-shuffles and group 0
+// writes the row.  Same spans, row walk, carry buffer and fix-up kernel as
+// spmm_span_kernel.  WMODE 0 (sum / mean) and 1 (one weight per edge, optionally
+// read through `perm`).
+__device__ __forceinline__ int64_t shfl_i64(int64_t v, int src_lane) {
+  const int lo = __shfl((int)(v & 0xffffffffll), src_lane, CXG_WAVE);
+  const int hi = __shfl((int)(v >> 32), src_lane, CXG_WAVE);
+  return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+__device__ __forceinline__ void vxor_add(float& a, int m) { a += __shfl_xor(a, m, CXG_WAVE); }
+__device__ __forceinline__ void vxor_add(float2& a, int m) {
+  a.x += __shfl_xor(a.x, m, CXG_WAVE); a.y += __shfl_xor(a.y, m, CXG_WAVE);
+}
+__device__ __forceinline__ void vxor_add(float4& a, int m) {
+  a.x += __shfl_xor(a.x, m, CXG_WAVE); a.y += __shfl_xor(a.y, m, CXG_WAVE);
+  a.z += __shfl_xor(a.z, m, CXG_WAVE); a.w += __shfl_xor(a.w, m, CXG_WAVE);
+}
+
+template <typename IdxT, int V, int L, int WMODE, bool PERM>
+__global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
+  using vec_t = typename Vec<V>::type;
+  constexpr int G = CXG_WAVE / L;
+  constexpr int UF = 4;                       // steps issued together inside long rows
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t n_rows = a.n_rows;
+  const int64_t e_begin = (int64_t)a.ptr[0];
+  const int64_t e_end = (int64_t)a.ptr[n_rows];
+  const int64_t total = e_end - e_begin;
+  const int T = a.T;
+  const int64_t n_spans = total > 0 ? (total + T - 1) / T : 1;
+  if (s >= n_spans) return;
+  const bool last = (s == n_spans - 1);
+  const int64_t e0 = e_begin + s * T;
+  const int n = (int)((e_end - e0) < (int64_t)T ? (e_end - e0) : (int64_t)T);
+  const int F = a.F;
+  const int g = lane / L;
+  const int col = (lane % L) * V;
+  const bool col_ok = col < F;
+  const bool writer = (g == 0) && col_ok;
+
+  const int64_t r_lo = wave_lower_bound(a.ptr, n_rows, e0);
+  bool is_head = (r_lo == n_rows) || ((int64_t)a.ptr[r_lo] > e0);
+  int64_t r = is_head ? r_lo - 1 : r_lo;
+  int64_t rbase = r;
+  auto load_row_ends = [&](int64_t rb) -> int {
+    int64_t q = rb + 1 + lane;
+    if (q > n_rows) q = n_rows;
+    const int64_t d = (int64_t)a.ptr[q] - e0;
+    return (int)(d < (int64_t)n + 1 ? d : (int64_t)n + 1);
+  };
+  int row_ends = load_row_ends(rbase);
+  int cur_start = is_head ? -1 : 0;
+  int cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
+
+  vec_t acc = vzero<V>();
+  int row_take = 0;                          // most groups used by a step of the current row
+  float* const carry_head = a.carry + (size_t)(2 * s) * F;
+  float* const carry_tail = carry_head + F;
+
+  auto next_row = [&]() {
+    ++r;
+    if (r - rbase == CXG_WAVE) {
+      rbase = r;
+      row_ends = load_row_ends(rbase);
+    }
+    cur_start = cur_end;
+    cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
+    is_head = false;
+  };
+  // sum of the groups' partials, valid in group 0 afterwards
+  auto reduce_groups = [&]() {
+#pragma unroll
+    for (int m = L; m < CXG_WAVE; m <<= 1)
+      if (row_take > m / L) vxor_add(acc, m);
+  };
+  auto store_vec = [&](float* dst, vec_t v) {
+    if (writer) *reinterpret_cast<vec_t*>(dst + col) = v;
+  };
+  auto finish_row = [&]() {
+    reduce_groups();
+    if (is_head) {
+      store_vec(carry_head, acc);
+    } else {
+      float* dst = a.out + r * a.ldo;
+      if (a.mean) {
+        const int deg = cur_end - cur_start;
+        if (deg > 0) vscale(acc, 1.0f / (float)deg);
+      }
+      if (a.accumulate) {
+        if (writer) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
+      }
+      store_vec(dst, acc);
+    }
+    acc = vzero<V>();
+    row_take = 0;
+  };
+
+  for (int c0 = 0; c0 < n; c0 += CXG_WAVE) {
+    const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
+    int64_t my_src = 0, my_vrow = 0;
+    float my_w = 0.f;
+    if (lane < cn) {
+      const int64_t pos = e0 + c0 + lane;
+      my_src = (int64_t)a.idx[pos];
+      if (PERM) my_vrow = a.perm[pos];
+      if (WMODE == 1 && !PERM) my_w = a.val[pos];
+    }
+    auto gather = [&](int e_idx, bool act, vec_t& v, float& w) {
+      const int64_t src = shfl_i64(my_src, e_idx & 63);
+      v = (act && col_ok) ? *reinterpret_cast<const vec_t*>(a.x + src * a.ldx + col) : vzero<V>();
+      if (WMODE == 1) {
+        if (PERM) {
+          const int64_t vrow = shfl_i64(my_vrow, e_idx & 63);
+          w = act ? a.val[vrow] : 0.f;
+        } else {
+          w = __shfl(my_w, e_idx & 63, CXG_WAVE);
+        }
+      }
+    };
+    int j = 0;
+    while (j < cn) {
+      while (c0 + j >= cur_end) {
+        finish_row();
+        next_row();
+      }
+      const int left = (cur_end - (c0 + j)) < (cn - j) ? (cur_end - (c0 + j)) : (cn - j);
+      if (left >= UF * G) {                   // long row: UF steps of G edges, loads first
+        vec_t v[UF];
+        float w[UF];
+#pragma unroll
+        for (int u = 0; u < UF; ++u) gather(j + u * G + g, true, v[u], w[u]);
+#pragma unroll
+        for (int u = 0; u < UF; ++u) {
+          if (WMODE == 0) vadd(acc, v[u]);
+          else vfma(acc, v[u], w[u]);
+        }
+        row_take = G;
+        j += UF * G;
+      } else {
+        const int take = left < G ? left : G;
+        vec_t v;
+        float w = 0.f;
+        gather(j + g, g < take, v, w);
+        if (WMODE == 0) vadd(acc, v);
+        else vfma(acc, v, w);
+        if (take > row_take) row_take = take;
+        j += take;
+      }
+    }
+  }
+
+  int64_t tail = -1;
+  while (r < n_rows) {
+    if (cur_end > n) {
+      reduce_groups();
+      if (is_head) {
+        store_vec(carry_head, acc);
+      } else if (cur_start < n) {
+        store_vec(carry_tail, acc);
+        tail = r;
+      }
+      break;
+    }
+    if (!(is_head || cur_start < n || last)) break;
+    finish_row();
+    next_row();
+  }
+  if (lane == 0) a.tail_row[s] = tail;
+}
+
 // One wave per span: if the span holds the tail partial of row t, add the head
 // partials of the following spans that row t runs through, in span order.
 template <typename IdxT, int V, bool GUARD>
@@ -366,8 +546,46 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   return CXG_OK;
 }
 
+// Narrow rows (at most 32 lanes of the widest aligned vector): grouped-lane kernel.
+// Returns 1 if it launched, 0 if the shape is not narrow, < 0 on a launch error.
+template <typename IdxT, int WMODE, bool PERM>
+int launch_group(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
+  const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry |
+                               (uintptr_t)(a.ldx * 4) | (uintptr_t)(a.ldo * 4) | (uintptr_t)(a.F * 4);
+  int v = 1;
+  for (int t = 2; t <= 4; t *= 2) {
+    if (a.F % t != 0 || (align_bits & (uintptr_t)(4 * t - 1)) != 0) break;
+    v = t;
+  }
+  const int lanes = (int)ceil_div(a.F, v);
+  if (lanes > 32) return 0;
+  int L = 4;
+  while (L < lanes) L <<= 1;
+  const dim3 grid((unsigned)ceil_div(n_spans_cap, kWavesPerBlock), 1, 1), block(kBlock, 1, 1);
+  bool done = false;
+#define CXG_GROUP(VV, LL)                                                                        \
+  if (!done && v == VV && L == LL) {                                                             \
+    hipLaunchKernelGGL((spmm_group_kernel<IdxT, VV, LL, WMODE, PERM>), grid, block, 0, stream, a); \
+    done = true;                                                                                 \
+  }
+  CXG_GROUP(4, 4) CXG_GROUP(4, 8) CXG_GROUP(4, 16) CXG_GROUP(4, 32)
+  CXG_GROUP(2, 4) CXG_GROUP(2, 8) CXG_GROUP(2, 16) CXG_GROUP(2, 32)
+  CXG_GROUP(1, 4) CXG_GROUP(1, 8) CXG_GROUP(1, 16) CXG_GROUP(1, 32)
+#undef CXG_GROUP
+  if (!done) return 0;
+  CXG_LAUNCH_CHECK("spmm_group_kernel");
+  const dim3 fgrid(grid.x, (unsigned)ceil_div(a.F, CXG_WAVE), 1);
+  hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 1, true>), fgrid, block, 0, stream, a);
+  CXG_LAUNCH_CHECK("spmm_fixup_kernel");
+  return 1;
+}
+
 template <typename IdxT, int WMODE, bool PERM, bool EXT = false>
 int dispatch_shape(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
+  if constexpr (!EXT && WMODE != 2) {
+    const int rc = launch_group<IdxT, WMODE, PERM>(a, n_spans_cap, stream);
+    if (rc != 0) return rc < 0 ? rc : CXG_OK;
+  }
   // widest vector that divides the row (and the head, for per-head weights) and
   // keeps every access aligned; among those the one needing the fewest column
   // tiles, ties to the narrower vector (more lanes busy).
