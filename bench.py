@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy kernel;
 # the summaries are kept under profiles/.  None until measured for a workload.
 MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE x 2.0000 + WRITE_SIZE x 1.0000 of one spmm_span_kernel launch
-    "c3_powerlaw_2.45M_nodes_61.9M_edges_F128": 25931503308,
+    # FETCH_SIZE x 2.0000 + WRITE_SIZE x 1.0000 of one spmm_group_kernel launch
+    "c3_powerlaw_2.45M_nodes_61.9M_edges_F128": 25959537868,
 }
 
 WORKLOADS = {
@@ -187,7 +187,7 @@ def main():
         "algorithmic_bytes_per_step": bytes_step,
         "roofline": {
             "bound": "hbm",
-            "kernel": "spmm_span_kernel (+ spmm_fixup_kernel), one cxg_spmm_sum_f32 call",
+            "kernel": "spmm_group_kernel (+ spmm_fixup_kernel), one cxg_spmm_sum_f32 call",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -24,6 +24,9 @@ namespace {
 #ifndef CXG_SPMM_SPAN_DIV
 #define CXG_SPMM_SPAN_DIV 16384   // target number of spans for graphs too small for 512-edge spans
 #endif
+#ifndef CXG_SPMM_GROUP_UF
+#define CXG_SPMM_GROUP_UF 4
+#endif
 #ifndef CXG_SPMM_U
 #define CXG_SPMM_U 1
 #endif
@@ -272,7 +275,7 @@ template <typename IdxT, int V, int L, int WMODE, bool PERM>
 __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   using vec_t = typename Vec<V>::type;
   constexpr int G = CXG_WAVE / L;
-  constexpr int UF = 4;                       // steps issued together inside long rows
+  constexpr int UF = CXG_SPMM_GROUP_UF;       // steps issued together inside long rows
   const int lane = lane_id();
   const int wave = uniform_i32(threadIdx.x >> 6);
   const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
