@@ -255,8 +255,9 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
 // of the current row, one per group, each group keeping its own partial sum; when
 // the row ends the partials are added across groups with xor-shuffles and group 0
 // writes the row.  Same spans, row walk, carry buffer and fix-up kernel as
-// spmm_span_kernel.  WMODE 0 (sum / mean) and 1 (one weight per edge, optionally
-// read through `perm`).
+// spmm_span_kernel.  WMODE 0 (sum / mean), 1 (one weight per edge) and 2 (one weight
+// per edge and head; a lane's V columns lie in one head), weights optionally read
+// through `perm`.
 __device__ __forceinline__ int64_t shfl_i64(int64_t v, int src_lane) {
   const int lo = __shfl((int)(v & 0xffffffffll), src_lane, CXG_WAVE);
   const int hi = __shfl((int)(v >> 32), src_lane, CXG_WAVE);
@@ -309,6 +310,8 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   int cur_start = is_head ? -1 : 0;
   int cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
 
+  int head_of_lane = 0;
+  if (WMODE == 2) head_of_lane = col_ok ? col / a.channels : 0;
   vec_t acc = vzero<V>();
   int row_take = 0;                          // most groups used by a step of the current row
   float* const carry_head = a.carry + (size_t)(2 * s) * F;
@@ -372,6 +375,9 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
         } else {
           w = __shfl(my_w, e_idx & 63, CXG_WAVE);
         }
+      } else if (WMODE == 2) {
+        const int64_t vrow = PERM ? shfl_i64(my_vrow, e_idx & 63) : (e0 + c0 + e_idx);
+        w = (act && col_ok) ? a.val[vrow * a.heads + head_of_lane] : 0.f;
       }
     };
     int j = 0;
@@ -555,9 +561,10 @@ template <typename IdxT, int WMODE, bool PERM>
 int launch_group(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
   const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry |
                                (uintptr_t)(a.ldx * 4) | (uintptr_t)(a.ldo * 4) | (uintptr_t)(a.F * 4);
+  const int unit = (WMODE == 2) ? a.channels : a.F;
   int v = 1;
   for (int t = 2; t <= 4; t *= 2) {
-    if (a.F % t != 0 || (align_bits & (uintptr_t)(4 * t - 1)) != 0) break;
+    if (unit % t != 0 || a.F % t != 0 || (align_bits & (uintptr_t)(4 * t - 1)) != 0) break;
     v = t;
   }
   const int lanes = (int)ceil_div(a.F, v);
@@ -577,15 +584,19 @@ int launch_group(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t strea
 #undef CXG_GROUP
   if (!done) return 0;
   CXG_LAUNCH_CHECK("spmm_group_kernel");
-  const dim3 fgrid(grid.x, (unsigned)ceil_div(a.F, CXG_WAVE), 1);
-  hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 1, true>), fgrid, block, 0, stream, a);
+  if (a.F % 128 == 0 && v >= 2) {
+    hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 2, false>), dim3(grid.x, (unsigned)(a.F / 128), 1), block, 0, stream, a);
+  } else {
+    const dim3 fgrid(grid.x, (unsigned)ceil_div(a.F, CXG_WAVE), 1);
+    hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 1, true>), fgrid, block, 0, stream, a);
+  }
   CXG_LAUNCH_CHECK("spmm_fixup_kernel");
   return 1;
 }
 
 template <typename IdxT, int WMODE, bool PERM, bool EXT = false>
 int dispatch_shape(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
-  if constexpr (!EXT && WMODE != 2) {
+  if constexpr (!EXT) {
     const int rc = launch_group<IdxT, WMODE, PERM>(a, n_spans_cap, stream);
     if (rc != 0) return rc < 0 ? rc : CXG_OK;
   }
