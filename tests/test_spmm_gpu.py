@@ -76,3 +76,46 @@ def test_spmm_mean_and_prefix_rows(kind):
         ref = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), rows, mean=True)
         assert out.shape == (rows, 128)
         assert_close(out.cpu().numpy(), ref, RTOL, ATOL, "mean %s rows=%d" % (kind, rows))
+
+
+# Row widths that reach every (vector width, lanes per edge) form of the grouped-lane
+# kernel (F <= 32 vector lanes) plus the first widths past it.
+WIDTHS = [2, 3, 4, 6, 7, 8, 12, 16, 20, 24, 30, 31, 33, 48, 52, 62, 64, 66, 96, 124, 126, 128, 130, 132]
+
+
+@pytest.mark.parametrize("feat", WIDTHS)
+def test_spmm_width_sweep(feat):
+    """Sum, mean, accumulate and a row prefix at every width, on a graph whose 2.33M edges
+    give spans of several 64-edge steps, hub rows that cross spans, and empty rows."""
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    ptr, idx = S.powerlaw_directed_symmetrised(169343, 1166243, seed=3)
+    n = ptr.shape[0] - 1
+    torch.manual_seed(feat)
+    x = torch.randn(n, feat) * _scale(ptr)
+    pc, ic, xc = ptr.cuda(), idx.cuda(), x.cuda()
+    announce("spmm width sweep F=%d" % feat)
+    got = _ops.spmm(pc, ic, xc, n)
+    want = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n)
+    assert_close(got.cpu().numpy(), want, RTOL, ATOL, "sum F=%d" % feat)
+    assert torch.equal(got, _ops.spmm(pc, ic, xc, n))                       # deterministic
+    rows = n // 7
+    got = _ops.spmm(pc, ic, xc, rows, mean=True)
+    want = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), rows, mean=True)
+    assert_close(got.cpu().numpy(), want, RTOL, ATOL, "mean prefix F=%d" % feat)
+    base = torch.randn(n, feat) / 4
+    out = base.clone().cuda()
+    _ops.spmm(pc, ic, xc, n, out=out, accumulate=True)
+    want = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n) + base.numpy()
+    assert_close(out.cpu().numpy(), want, RTOL, ATOL, "accumulate F=%d" % feat)
+    # one weight per edge, also read through a permutation
+    val = torch.rand(idx.shape[0]) + 0.5
+    got = _ops.spmm(pc, ic, xc, n, val=val.cuda())
+    want = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n, val=val.numpy())
+    sc = max(1.0, float(np.abs(want).max()))
+    assert_close(got.cpu().numpy() / sc, want / sc, RTOL, ATOL, "weighted F=%d" % feat)
+    perm = torch.randperm(idx.shape[0])
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(idx.shape[0])
+    got2 = _ops.spmm(pc, ic, xc, n, val=val[perm].cuda(), val_perm=inv.cuda())
+    assert torch.equal(got, got2)
