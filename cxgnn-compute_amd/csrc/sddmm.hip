@@ -293,6 +293,117 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(SddmmArgs a) {
   }
 }
 
+// Narrow rows (heads * channels <= 128 floats): several edges per gather
+// instruction.  An edge occupies LE = heads * GROUP lanes (16 bytes each), the
+// wave holds 64 / LE edge slots; one step gathers one source row per slot (CSR
+// form: consecutive edges of the current destination row, whose row all slots
+// share; COO form: every slot also fetches its own destination row).  The group
+// leaders leave the products in a per-wave LDS tile of 64 x heads floats and each
+// 64-edge step ends with coalesced stores from that tile.  One whole wave per edge
+// left these shapes bound by one gather instruction per edge.
+constexpr int kMultiMaxHeads = 8;
+
+__device__ __forceinline__ int64_t sd_shfl_i64(int64_t v, int src_lane) {
+  const int lo = __shfl((int)(v & 0xffffffffll), src_lane, CXG_WAVE);
+  const int hi = __shfl((int)(v >> 32), src_lane, CXG_WAVE);
+  return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+template <int GROUP, bool COO>
+__global__ __launch_bounds__(kBlock) void sddmm_multi_kernel(SddmmArgs a) {
+  constexpr int V = 4;
+  constexpr int UF = 4;                              // steps issued together
+  using vec_t = typename Vec<V>::type;
+  __shared__ float s_res[kWavesPerBlock][CXG_WAVE * kMultiMaxHeads];
+  const int lane = lane_id();
+  const int wave = uniform_i32(threadIdx.x >> 6);
+  const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t n_rows = a.n_rows;
+  const int64_t e_begin = COO ? 0 : a.ptr[0];
+  const int64_t e_end = COO ? a.n_edges : a.ptr[n_rows];
+  const int64_t e0 = e_begin + s * kSpan;
+  if (e0 >= e_end) return;
+  const int n = (int)((e_end - e0) < (int64_t)kSpan ? (e_end - e0) : (int64_t)kSpan);
+  const int H = a.heads;
+  const int F = H * a.channels;                      // = LE * V
+  const int LE = H * GROUP;                          // lanes per edge (power of two <= 32)
+  const int EPI = CXG_WAVE / LE;                     // edges per step
+  const int es = lane / LE, le = lane % LE;
+  const int head = le / GROUP, q = lane % GROUP;
+  const int bcol = a.b_heads ? le * V : q * V;
+  const int64_t ldb = a.b_heads ? F : a.channels;
+  float* const res = s_res[wave];
+
+  int64_t r = 0, rbase = 0;
+  int row_ends = 0, cur_end = 0;
+  vec_t brow = vzero<V>();
+  auto load_row_ends = [&](int64_t rb) -> int {
+    int64_t k = rb + 1 + lane;
+    if (k > n_rows) k = n_rows;
+    const int64_t d = (int64_t)a.ptr[k] - e0;
+    return (int)(d < (int64_t)n + 1 ? d : (int64_t)n + 1);
+  };
+  if (!COO) {
+    r = wave_lower_bound(a.ptr, n_rows + 1, e0 + 1) - 1;
+    rbase = r;
+    row_ends = load_row_ends(rbase);
+    cur_end = bcast_i32(row_ends, 0);
+    brow = *reinterpret_cast<const vec_t*>(a.b + r * ldb + bcol);
+  }
+
+  for (int c0 = 0; c0 < n; c0 += CXG_WAVE) {
+    const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
+    int64_t my_src = 0, my_dst = 0;
+    if (lane < cn) {
+      my_src = COO ? a.src[e0 + c0 + lane] : a.idx[e0 + c0 + lane];
+      if (COO) my_dst = a.dst[e0 + c0 + lane];
+    }
+    auto fetch = [&](int jj, bool act, vec_t& va, vec_t& vb) {
+      const int64_t src = sd_shfl_i64(my_src, jj & 63);
+      va = act ? *reinterpret_cast<const vec_t*>(a.a + src * F + le * V) : vzero<V>();
+      if (COO) {
+        const int64_t dst = sd_shfl_i64(my_dst, jj & 63);
+        vb = act ? *reinterpret_cast<const vec_t*>(a.b + dst * ldb + bcol) : vzero<V>();
+      }
+    };
+    int j = 0;
+    while (j < cn) {
+      if (!COO) {
+        while (c0 + j >= cur_end) {
+          ++r;
+          if (r - rbase == CXG_WAVE) { rbase = r; row_ends = load_row_ends(rbase); }
+          cur_end = bcast_i32(row_ends, (int)(r - rbase));
+          if (c0 + j < cur_end) brow = *reinterpret_cast<const vec_t*>(a.b + r * ldb + bcol);
+        }
+      }
+      int left = cn - j;
+      if (!COO && cur_end - (c0 + j) < left) left = cur_end - (c0 + j);
+      if (left >= UF * EPI) {
+        vec_t va[UF], vb[UF];
+#pragma unroll
+        for (int u = 0; u < UF; ++u) fetch(j + u * EPI + es, true, va[u], vb[u]);
+#pragma unroll
+        for (int u = 0; u < UF; ++u) {
+          const float p = group_sum(vdot(va[u], COO ? vb[u] : brow), GROUP);
+          if (q == 0) res[(j + u * EPI + es) * H + head] = p;
+        }
+        j += UF * EPI;
+      } else {
+        const int take = left < EPI ? left : EPI;
+        const bool act = es < take;
+        vec_t va, vb;
+        fetch(j + es, act, va, vb);
+        const float p = group_sum(vdot(va, COO ? vb : brow), GROUP);
+        if (q == 0 && act) res[(j + es) * H + head] = p;
+        j += take;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();                 // the tile is complete (one wave, in-order LDS)
+    for (int i = lane; i < cn * H; i += CXG_WAVE) a.out[(e0 + c0) * H + i] = res[i];
+    __builtin_amdgcn_wave_barrier();                 // read before the next step overwrites it
+  }
+}
+
 // General layout (any heads / channels): one wave-wide reduction per (edge, head).
 // COO == false walks CSR rows (dst = row), COO == true reads src/dst arrays.
 template <bool COO>
@@ -345,6 +456,24 @@ int packed_vec(const SddmmArgs& a) {
   return 0;
 }
 
+// Launches the several-edges-per-step kernel when an edge fits 32 lanes of 16 bytes.
+template <bool COO>
+bool launch_multi(SddmmArgs a, dim3 grid, dim3 block, hipStream_t st) {
+  const uintptr_t bits = (uintptr_t)a.a | (uintptr_t)a.b;
+  if (a.channels % 4 != 0 || (bits & 15) != 0 || a.heads > kMultiMaxHeads) return false;
+  a.group = a.channels / 4;
+  const int le = a.heads * a.group;
+  if (!is_pow2(a.group) || !is_pow2(le) || le > 32) return false;
+#define CXG_MULTI(GG)                                                               \
+  if (a.group == GG) {                                                              \
+    hipLaunchKernelGGL((sddmm_multi_kernel<GG, COO>), grid, block, 0, st, a);       \
+    return true;                                                                    \
+  }
+  CXG_MULTI(1) CXG_MULTI(2) CXG_MULTI(4) CXG_MULTI(8) CXG_MULTI(16) CXG_MULTI(32)
+#undef CXG_MULTI
+  return false;
+}
+
 // Launches the tiled-output kernel when the group width has an instantiation.
 template <bool COO>
 bool launch_tiled(const SddmmArgs& a, int v, dim3 grid, dim3 block, hipStream_t st) {
@@ -388,7 +517,8 @@ int cxg_sddmm_csr_f32(const int64_t* ptr, const int64_t* idx, const float* src_f
   dim3 block(cxg::kBlock);
   const int v = cxg::packed_vec(a);
   if (v) a.group = channels / v;
-  if (v && cxg::launch_tiled<false>(a, v, grid, block, st)) { /* coalesced-output form */ }
+  if (cxg::launch_multi<false>(a, grid, block, st)) { /* several edges per step */ }
+  else if (v && cxg::launch_tiled<false>(a, v, grid, block, st)) { /* coalesced-output form */ }
   else if (v == 4) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<4>, grid, block, 0, st, a);
   else if (v == 2) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<2>, grid, block, 0, st, a);
   else if (v == 1) hipLaunchKernelGGL(cxg::sddmm_csr_packed_kernel<1>, grid, block, 0, st, a);
@@ -414,7 +544,8 @@ int cxg_sddmm_coo_f32(const int64_t* src, const int64_t* dst, const float* src_f
   dim3 block(cxg::kBlock);
   const int v = cxg::packed_vec(a);
   if (v) a.group = channels / v;
-  if (v && cxg::launch_tiled<true>(a, v, grid, block, st)) { /* coalesced-output form */ }
+  if (cxg::launch_multi<true>(a, grid, block, st)) { /* several edges per step */ }
+  else if (v && cxg::launch_tiled<true>(a, v, grid, block, st)) { /* coalesced-output form */ }
   else if (v == 4) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<4>, grid, block, 0, st, a);
   else if (v == 2) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<2>, grid, block, 0, st, a);
   else if (v == 1) hipLaunchKernelGGL(cxg::sddmm_coo_packed_kernel<1>, grid, block, 0, st, a);

@@ -25,8 +25,9 @@ def _coo(ptr, idx):
     return idx.clone(), dst
 
 
-@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows"])
-@pytest.mark.parametrize("shape", [(4, 64), (1, 128), (1, 64), (2, 32), (3, 40), (1, 300), (8, 8)])
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
+@pytest.mark.parametrize("shape", [(4, 64), (1, 128), (1, 64), (2, 32), (3, 40), (1, 300), (8, 8), (1, 4), (1, 8),
+                                   (2, 4), (1, 16), (1, 32), (4, 8), (4, 16), (4, 32), (8, 16), (2, 64), (1, 12)])
 @pytest.mark.parametrize("dst_heads", [True, False])
 def test_sddmm_coo_and_csr(kind, shape, dst_heads):
     import cxgnncomp_backend as B
