@@ -90,6 +90,51 @@ __device__ __forceinline__ int64_t wave_lower_bound(const T* __restrict__ a,
   }
   return uniform_i64(lo);
 }
+
+// Rows of consecutive edge positions, one position per lane, for a wave that walks
+// forward through the edge array: row(p) = the r with ptr[r] <= p < ptr[r+1].  The wave
+// keeps the ends of 64 rows (relative to its first position) in one register per lane;
+// a position is located by a six-step search through lane shuffles, and only when a
+// position lies past the window is the window moved, by one cooperative search of ptr.
+struct RowWalker {
+  const int64_t* ptr;
+  int64_t n_rows, p0, rbase;
+  int ends;                                  // ptr[rbase + 1 + lane] - p0, clamped
+
+  __device__ __forceinline__ void load_window() {
+    const int64_t k = rbase + 1 + lane_id();
+    const int64_t d = k <= n_rows ? ptr[k] - p0 : (int64_t)(1 << 30);   // past the last row: never reached
+    ends = d > (int64_t)(1 << 30) ? (1 << 30) : (int)d;
+  }
+  __device__ __forceinline__ void init(const int64_t* ptr_, int64_t n_rows_, int64_t p0_) {
+    ptr = ptr_; n_rows = n_rows_; p0 = p0_;
+    rbase = wave_lower_bound(ptr, n_rows + 1, p0 + 1) - 1;
+    load_window();
+  }
+  // `rel` = position - p0 (non-decreasing over lanes and over calls, < 2^30);
+  // lanes with !valid get -1; positions at or past ptr[n_rows] get n_rows.  Every pass
+  // settles at least the first pending lane, so 64 passes always suffice; the bound
+  // makes the loop end on a ptr that is not sorted, too.
+  __device__ __forceinline__ int64_t row_of(int rel, bool valid) {
+    int64_t row = -1;
+    for (int pass = 0; pass < CXG_WAVE + 1; ++pass) {
+      // the shuffles run with every lane active; only the use of their result is per lane
+      const int window_end = __shfl(ends, CXG_WAVE - 1, CXG_WAVE);
+      int cnt = 0;                           // window rows whose end is <= rel
+#pragma unroll
+      for (int step = 32; step >= 1; step >>= 1)
+        if (__shfl(ends, cnt + step - 1, CXG_WAVE) <= rel) cnt += step;
+      if (row < 0 && valid && window_end > rel) row = rbase + cnt;
+      const unsigned long long pending = __ballot(valid && row < 0);
+      if (pending == 0) break;
+      const int first = __ffsll((long long)pending) - 1;
+      const int64_t target = p0 + __shfl(rel, first, CXG_WAVE);
+      rbase = wave_lower_bound(ptr, n_rows + 1, target + 1) - 1;
+      load_window();
+    }
+    return row;
+  }
+};
 #endif  // __HIPCC__
 
 }  // namespace cxg

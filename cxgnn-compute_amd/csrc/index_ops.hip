@@ -6,6 +6,7 @@
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
+#include <rocprim/iterator/transform_iterator.hpp>
 
 namespace cxg {
 namespace {
@@ -44,10 +45,63 @@ __global__ void transpose_fill_kernel(const int64_t* __restrict__ ptr, int64_t n
   }
 }
 
-__global__ void row_ids_kernel(const int64_t* __restrict__ ptr, int64_t n_rows, int64_t n_edges,
-                               int64_t* __restrict__ rows) {
+// Narrow form of the transposition, for graphs whose row, column and edge counts all fit
+// 32 bits: the sort moves 4-byte keys and one 8-byte value per edge that carries the
+// edge's row next to its position, so no search by (random) position follows the sort.
+struct ColumnKey {
+  __host__ __device__ uint32_t operator()(int64_t v) const { return (uint32_t)v; }
+};
+using ColumnKeyIter = rocprim::transform_iterator<const int64_t*, ColumnKey, uint32_t>;
+
+// Row of every edge position, written as int64 row ids (MODE 0) or packed with the
+// position for the narrow transposition (MODE 1).  One wave walks kRowSpan positions.
+constexpr int kRowSpan = 8 * CXG_WAVE;
+
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void expand_rows_kernel(const int64_t* __restrict__ ptr,
+                                                             int64_t n_rows, int64_t n_edges,
+                                                             void* __restrict__ out) {
+  const int lane = lane_id();
+  const int64_t w = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+  const int64_t k0 = uniform_i64(w * kRowSpan);
+  if (k0 >= n_edges) return;
+  RowWalker walk;
+  walk.init(ptr, n_rows, (MODE == 0 ? ptr[0] : 0) + k0);   // row ids count positions from ptr[0]
+  for (int c = 0; c < kRowSpan; c += CXG_WAVE) {
+    const int64_t k = k0 + c + lane;
+    if (k0 + c >= n_edges) break;
+    const int64_t row = walk.row_of(c + lane, k < n_edges);
+    if (k < n_edges) {
+      if (MODE == 0) reinterpret_cast<int64_t*>(out)[k] = row;
+      else reinterpret_cast<uint64_t*>(out)[k] = ((uint64_t)row << 32) | (uint64_t)k;
+    }
+  }
+}
+
+// perm / idx_t from the sorted packed values (in place over `perm`), ptr_t from the
+// boundaries of the sorted keys: position k is the first edge of every column in
+// (key[k-1], key[k]], and the last position also closes the columns after its own.
+__global__ void transpose_unpack_kernel(const uint32_t* __restrict__ sorted_key, int64_t n_edges,
+                                        int64_t n_cols, int64_t* __restrict__ perm,
+                                        int64_t* __restrict__ idx_t, int64_t* __restrict__ ptr_t) {
   const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (k < n_edges) rows[k] = row_of_position(ptr, n_rows, k + ptr[0]);
+  if (k >= n_edges) return;
+  const uint64_t v = (uint64_t)perm[k];
+  perm[k] = (int64_t)(v & 0xffffffffull);
+  idx_t[k] = (int64_t)(v >> 32);
+  // (ids are < n_cols by contract; the clamp keeps a broken input from writing past ptr_t)
+  const int64_t last = n_cols - 1;
+  int64_t c = sorted_key[k], prev = k > 0 ? (int64_t)sorted_key[k - 1] : -1;
+  if (c > last) c = last;
+  if (prev > last) prev = last;
+  for (int64_t j = prev + 1; j <= c; ++j) ptr_t[j] = k;
+  if (k == n_edges - 1)
+    for (int64_t j = c + 1; j <= n_cols; ++j) ptr_t[j] = n_edges;
+}
+
+__global__ void fill_i64_kernel(int64_t* __restrict__ out, int64_t n, int64_t value) {
+  const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (k < n) out[k] = value;
 }
 
 // One wave per row: val[e] = 1 / deg(row) for the row's edges.
@@ -83,6 +137,18 @@ int bits_for(int64_t n) {
 
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
+constexpr int64_t kNarrowLimit = (int64_t)1 << 32;
+
+size_t narrow_sort_temp_bytes(int64_t n_edges, int64_t n_cols) {
+  size_t temp = 0;
+  ColumnKeyIter keys(nullptr, ColumnKey());
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, keys, (uint32_t*)nullptr,
+                                           (const uint64_t*)nullptr, (uint64_t*)nullptr,
+                                           (size_t)n_edges, 0, bits_for(n_cols > 1 ? n_cols : 2),
+                                           (hipStream_t)0);
+  return e == hipSuccess ? temp : 0;
+}
+
 }  // namespace
 }  // namespace cxg
 
@@ -96,6 +162,8 @@ size_t cxg_csr_transpose_workspace_bytes(int64_t n_edges, int64_t n_cols) {
                                            iota, (int64_t*)nullptr, (size_t)n_edges, 0,
                                            cxg::bits_for(n_cols > 1 ? n_cols : 2), (hipStream_t)0);
   if (e != hipSuccess) return 0;
+  const size_t narrow = cxg::narrow_sort_temp_bytes(n_edges, n_cols);
+  if (narrow > temp) temp = narrow;      // the narrow form's keys need half the room of the wide ones
   return cxg::align256((size_t)n_edges * sizeof(int64_t)) + cxg::align256(temp) + 256;
 }
 
@@ -114,6 +182,29 @@ int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows
   const size_t off = cxg::align256((size_t)n_edges * sizeof(int64_t));
   void* temp = reinterpret_cast<char*>(workspace) + off;
   size_t temp_bytes = workspace_bytes - off;
+  if (n_edges == 0) {
+    hipLaunchKernelGGL(cxg::fill_i64_kernel, dim3((unsigned)cxg::ceil_div(n_cols + 1, cxg::kBlock)),
+                       dim3(cxg::kBlock), 0, st, ptr_t, n_cols + 1, (int64_t)0);
+    CXG_LAUNCH_CHECK("fill_i64_kernel");
+    return CXG_OK;
+  }
+  if (n_rows < cxg::kNarrowLimit && n_cols < cxg::kNarrowLimit && n_edges < cxg::kNarrowLimit) {
+    const dim3 grid((unsigned)cxg::ceil_div(n_edges, cxg::kBlock)), block(cxg::kBlock);
+    uint64_t* packed = reinterpret_cast<uint64_t*>(idx_t);      // outputs double as sort buffers
+    uint32_t* sorted_key = reinterpret_cast<uint32_t*>(workspace);
+    const dim3 wgrid((unsigned)cxg::ceil_div(cxg::ceil_div(n_edges, cxg::kRowSpan), cxg::kBlock / CXG_WAVE));
+    hipLaunchKernelGGL(cxg::expand_rows_kernel<1>, wgrid, block, 0, st, ptr, n_rows, n_edges,
+                       (void*)packed);
+    CXG_LAUNCH_CHECK("expand_rows_kernel");
+    cxg::ColumnKeyIter keys(idx, cxg::ColumnKey());
+    CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, keys, sorted_key, packed,
+                                            reinterpret_cast<uint64_t*>(perm), (size_t)n_edges, 0,
+                                            cxg::bits_for(n_cols > 1 ? n_cols : 2), st));
+    hipLaunchKernelGGL(cxg::transpose_unpack_kernel, grid, block, 0, st, sorted_key, n_edges, n_cols,
+                       perm, idx_t, ptr_t);
+    CXG_LAUNCH_CHECK("transpose_unpack_kernel");
+    return CXG_OK;
+  }
   if (n_edges > 0) {
     rocprim::counting_iterator<int64_t> iota(0);
     CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, idx, sorted_src, iota, perm,
@@ -133,10 +224,10 @@ int cxg_csr_row_ids_i64(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
   CXG_REQUIRE(n_rows >= 0 && n_edges >= 0, CXG_ERR_ARG, "negative size");
   if (n_edges == 0) return CXG_OK;
   CXG_REQUIRE(ptr && rows, CXG_ERR_ARG, "null pointer");
-  hipLaunchKernelGGL(cxg::row_ids_kernel, dim3((unsigned)cxg::ceil_div(n_edges, cxg::kBlock)),
-                     dim3(cxg::kBlock), 0, reinterpret_cast<hipStream_t>(stream), ptr, n_rows, n_edges,
-                     rows);
-  CXG_LAUNCH_CHECK("row_ids_kernel");
+  const dim3 wgrid((unsigned)cxg::ceil_div(cxg::ceil_div(n_edges, cxg::kRowSpan), cxg::kBlock / CXG_WAVE));
+  hipLaunchKernelGGL(cxg::expand_rows_kernel<0>, wgrid, dim3(cxg::kBlock), 0,
+                     reinterpret_cast<hipStream_t>(stream), ptr, n_rows, n_edges, (void*)rows);
+  CXG_LAUNCH_CHECK("expand_rows_kernel");
   return CXG_OK;
 }
 

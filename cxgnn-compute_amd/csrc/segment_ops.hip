@@ -23,18 +23,22 @@ namespace {
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
 
-__global__ void row_ids32_kernel(const int64_t* __restrict__ ptr, int64_t n_rows, int64_t n_edges,
-                                 int32_t* __restrict__ rows) {
-  const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= n_edges) return;
-  const int64_t p = k + ptr[0];
-  int64_t lo = 0, hi = n_rows + 1;        // upper_bound(ptr[0..n_rows], p) - 1
-  while (lo < hi) {
-    const int64_t mid = (lo + hi) >> 1;
-    if (ptr[mid] <= p) lo = mid + 1;
-    else hi = mid;
+constexpr int kRowSpan = 8 * CXG_WAVE;       // positions one wave expands
+
+__global__ __launch_bounds__(256) void row_ids32_kernel(const int64_t* __restrict__ ptr, int64_t n_rows,
+                                                        int64_t n_edges, int32_t* __restrict__ rows) {
+  const int lane = lane_id();
+  const int64_t w = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int64_t k0 = uniform_i64(w * kRowSpan);
+  if (k0 >= n_edges) return;
+  RowWalker walk;
+  walk.init(ptr, n_rows, ptr[0] + k0);
+  for (int c = 0; c < kRowSpan; c += CXG_WAVE) {
+    if (k0 + c >= n_edges) break;
+    const int64_t k = k0 + c + lane;
+    const int64_t row = walk.row_of(c + lane, k < n_edges);
+    if (k < n_edges) rows[k] = (int32_t)row;
   }
-  rows[k] = (int32_t)(lo - 1);
 }
 
 __global__ void zero_f32_kernel(float* __restrict__ p, int64_t n) {
@@ -197,7 +201,8 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
   CXG_REQUIRE(n_rows < ((int64_t)1 << 31), CXG_ERR_UNSUPPORTED, "row ids do not fit int32");
   if (n_edges == 0) return CXG_OK;
   CXG_REQUIRE(ptr && rows, CXG_ERR_ARG, "null pointer");
-  hipLaunchKernelGGL(cxg::row_ids32_kernel, dim3((unsigned)cxg::ceil_div(n_edges, 256)), dim3(256), 0,
+  hipLaunchKernelGGL(cxg::row_ids32_kernel,
+                     dim3((unsigned)cxg::ceil_div(cxg::ceil_div(n_edges, cxg::kRowSpan), 4)), dim3(256), 0,
                      reinterpret_cast<hipStream_t>(stream), ptr, n_rows, n_edges, rows);
   CXG_LAUNCH_CHECK("row_ids32_kernel");
   return CXG_OK;

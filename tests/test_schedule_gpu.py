@@ -128,3 +128,72 @@ def test_schedule_helpers_at_benchmark_size():
     p3, i3 = cxgnncomp.remove_from_graph(ptr, idx, rflag)
     assert torch.equal(p3[1:] - p3[:-1], deg[~rflag])
     assert torch.equal(i3, idx[torch.repeat_interleave(~rflag, deg)])
+
+
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "no_edges", "one_hub"])
+@pytest.mark.parametrize("prefix", [False, True])
+def test_csr_transpose_bit_exact(kind, prefix):
+    """Reversed graph of all rows / of a row prefix, with more source nodes than the ids
+    that occur (trailing empty columns): ptr_t, idx_t and the stable edge order perm."""
+    from cxgnncomp_backend import _ops
+    from test_spmm_gpu import _graph
+    ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    n_rows = n // 3 if prefix else n
+    n_src = n + 37
+    want_ptr, want_idx, want_perm = oracle.csr_transpose(ptr.numpy(), idx.numpy(), n_rows, n_src)
+    announce("csr_transpose kind=%s prefix=%s" % (kind, prefix))
+    ptr_t, idx_t, perm, n_edges = _ops.csr_transpose(ptr.cuda(), idx.cuda(), n_rows, n_src)
+    torch.cuda.synchronize()
+    assert n_edges == int(ptr[n_rows])
+    assert np.array_equal(_np(ptr_t), want_ptr)
+    assert np.array_equal(_np(idx_t), want_idx)
+    assert np.array_equal(_np(perm), want_perm)
+
+
+def test_csr_transpose_leading_empty_columns():
+    """Sources 0..4 never occur, one source takes every edge."""
+    from cxgnncomp_backend import _ops
+    ptr = torch.tensor([0, 2, 2, 5])
+    idx = torch.tensor([7, 5, 9, 5, 5])
+    announce("csr_transpose leading empty columns")
+    ptr_t, idx_t, perm, n_edges = _ops.csr_transpose(ptr.cuda(), idx.cuda(), 3, 12)
+    assert n_edges == 5
+    assert _np(ptr_t).tolist() == [0, 0, 0, 0, 0, 0, 3, 3, 4, 4, 5, 5, 5]
+    assert _np(idx_t).tolist() == [0, 2, 2, 0, 2]
+    assert _np(perm).tolist() == [1, 3, 4, 0, 2]
+
+
+def _gappy_ptr(rng, n, first=0):
+    """Degrees with runs of hundreds of empty rows between occupied ones, and some hubs."""
+    deg = np.zeros(n, dtype=np.int64)
+    occupied = rng.choice(n, max(1, n // 150), replace=False)
+    deg[occupied] = rng.integers(1, 9, occupied.shape[0])
+    deg[rng.choice(n, 3)] = 1500
+    return first + np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+
+
+@pytest.mark.parametrize("case", ["gappy", "gappy_offset", "dense", "single_row", "degree_one"])
+def test_csr_row_ids_bit_exact(case):
+    """Row of every edge position, int64 and int32 forms; positions count from ptr[0]."""
+    from cxgnncomp_backend import _ops
+    rng = np.random.default_rng(len(case))
+    if case == "gappy":
+        ptr = _gappy_ptr(rng, 40000)
+    elif case == "gappy_offset":
+        ptr = _gappy_ptr(rng, 40000, first=777)
+    elif case == "dense":
+        ptr = _random_ptr(rng, 30000, 60)
+    elif case == "single_row":
+        ptr = np.array([0, 100000], dtype=np.int64)
+    else:
+        ptr = np.arange(0, 70001, dtype=np.int64)
+    n = ptr.shape[0] - 1
+    E = int(ptr[-1] - ptr[0])
+    want = np.repeat(np.arange(n, dtype=np.int64), np.diff(ptr))
+    announce("csr_row_ids case=%s" % case)
+    got = _ops.csr_row_ids(torch.from_numpy(ptr).cuda(), n, E)
+    got32 = _ops.csr_row_ids32(torch.from_numpy(ptr).cuda(), n, E)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np(got), want)
+    assert got32.dtype == torch.int32 and np.array_equal(_np(got32).astype(np.int64), want)
