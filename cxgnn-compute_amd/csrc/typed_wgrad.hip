@@ -195,19 +195,43 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
   }
 }
 
-// gw[r][k][n] = sum of the partials of relation r's chunks, in chunk order.
-__global__ void wgrad_reduce_kernel(const int64_t* __restrict__ seg, int R, int64_t rows_per_chunk,
-                                    const float* __restrict__ partial, float* __restrict__ gw,
-                                    int64_t kn) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+// gw[r][k][n] = sum of the partials of relation r's chunks, in a fixed order: the chunks
+// are cut into kReduceSlices contiguous runs, each run is summed by one thread (four
+// interleaved chains, so the loads overlap) and the runs are added in run order.
+constexpr int kReduceSlices = 4;
+
+__global__ __launch_bounds__(64 * kReduceSlices) void wgrad_reduce_kernel(
+    const int64_t* __restrict__ seg, int R, int64_t rows_per_chunk, const float* __restrict__ partial,
+    float* __restrict__ gw, int64_t kn) {
+  __shared__ float s_run[kReduceSlices][64];
+  const int el = threadIdx.x & 63, sl = threadIdx.x >> 6;
+  const int64_t e = (int64_t)blockIdx.x * 64 + el;
   const int r = blockIdx.y;
-  if (e >= kn) return;
   int64_t first = 0;
   for (int q = 0; q < r; ++q) first += (seg[q + 1] - seg[q] + rows_per_chunk - 1) / rows_per_chunk;
   const int64_t cnt = (seg[r + 1] - seg[r] + rows_per_chunk - 1) / rows_per_chunk;
-  float acc = 0.f;
-  for (int64_t c = 0; c < cnt; ++c) acc += partial[(size_t)(first + c) * kn + e];
-  gw[(size_t)r * kn + e] = acc;
+  const int64_t per = (cnt + kReduceSlices - 1) / kReduceSlices;
+  const int64_t c0 = sl * per, c1 = (c0 + per) < cnt ? (c0 + per) : cnt;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  if (e < kn) {
+    const float* p = partial + (size_t)first * kn + e;
+    int64_t c = c0;
+    for (; c + 4 <= c1; c += 4) {
+      a0 += p[(size_t)(c + 0) * kn];
+      a1 += p[(size_t)(c + 1) * kn];
+      a2 += p[(size_t)(c + 2) * kn];
+      a3 += p[(size_t)(c + 3) * kn];
+    }
+    for (; c < c1; ++c) a0 += p[(size_t)c * kn];
+  }
+  s_run[sl][el] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (sl == 0 && e < kn) {
+    float acc = s_run[0][el];
+#pragma unroll
+    for (int q = 1; q < kReduceSlices; ++q) acc += s_run[q][el];
+    gw[(size_t)r * kn + e] = acc;
+  }
 }
 
 int64_t chunk_rows(int64_t M, int N) {
@@ -257,7 +281,8 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
   else hipLaunchKernelGGL(cxg::typed_wgrad_split_kernel<3>, grid, block, 0, st, wa);
   CXG_LAUNCH_CHECK("typed_wgrad_split_kernel");
   const int64_t kn = (int64_t)K * N;
-  hipLaunchKernelGGL(cxg::wgrad_reduce_kernel, dim3((unsigned)cxg::ceil_div(kn, 256), (unsigned)R), dim3(256), 0,
+  hipLaunchKernelGGL(cxg::wgrad_reduce_kernel, dim3((unsigned)cxg::ceil_div(kn, 64), (unsigned)R),
+                     dim3(64 * cxg::kReduceSlices), 0,
                      st, seg_ptr, R, rows, reinterpret_cast<const float*>(workspace), gw, kn);
   CXG_LAUNCH_CHECK("wgrad_reduce_kernel");
   return CXG_OK;

@@ -182,11 +182,11 @@ class MySageConv(torch.nn.Module):
 
     def forward(self, x, ptr, idx, num_node):
         if self.in_channels > self.hidden_channels:
-            out = sage_mean_forward(self.lin_l(x), ptr, idx, num_node)
+            out = sage_mean_forward(linear(x, self.lin_l.weight, self.lin_l.bias), ptr, idx, num_node)
         else:
-            out = self.lin_l(sage_mean_forward(x, ptr, idx, num_node))
+            out = linear(sage_mean_forward(x, ptr, idx, num_node), self.lin_l.weight, self.lin_l.bias)
         if self.root_weight:
-            out = out + self.lin_r(x[:num_node] if num_node != 0 else x)
+            out = out + linear(x[:num_node] if num_node != 0 else x, self.lin_r.weight)
         return out
 
 
@@ -207,7 +207,7 @@ class MyGINConv(torch.nn.Module):
 
     def forward(self, x, ptr, idx, num_node):
         out = sage_mean_forward(x, ptr, idx, num_node)
-        return self.nn(out + (1 + self.eps) * x[:num_node])
+        return linear(out + (1 + self.eps) * x[:num_node], self.nn.weight)
 
 
 class MyRGCNConv(torch.nn.Module):
@@ -253,7 +253,7 @@ def _arange_ptr(n, device):
 
 class HeadDotOP(torch.autograd.Function):
     """alpha[n, h] = sum_c x[n, h, c] * att[h, c]: upstream's ``(x * att).sum(dim=-1)``
-    (cxgnncomp/graph_conv.py:460-461) without the [N, H, C] temporaries.  On the GPU it is
+    (cxgnncomp/graph_conv.py:466-467) without the [N, H, C] temporaries.  On the GPU it is
     the SDDMM of every node row against the single row ``att`` (a one-row CSR over all
     nodes); its weight gradient is a [H, N] x [N, H*C] product on the typed weight-gradient
     kernel.  Host tensors use the upstream expression."""
@@ -289,6 +289,81 @@ class HeadDotOP(torch.autograd.Function):
             if gatt is None:
                 gatt = (grad.unsqueeze(-1) * x).sum(dim=0).view_as(att)
         return gx, gatt
+
+
+_SEG_CACHE = {}
+
+
+def _one_segment(m, device):
+    """Device tensor [0, m]: the segment table of an untyped weight gradient."""
+    key = (m, device)
+    seg = _SEG_CACHE.get(key)
+    if seg is None:
+        if len(_SEG_CACHE) > 64:
+            _SEG_CACHE.clear()
+        seg = _SEG_CACHE[key] = torch.tensor([0, m], dtype=torch.int64, device=device)
+    return seg
+
+
+class LinearOP(torch.autograd.Function):
+    """``F.linear(x, weight)`` whose weight gradient g^T x, a product with one very long
+    reduction axis (every node) and a small output, runs on the typed weight-gradient
+    kernel as a single segment; the library GEMM serves the forward pass, the input
+    gradient and the shapes that kernel does not take."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        ctx.save_for_backward(x, weight)
+        return F.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        gx = gw = None
+        if ctx.needs_input_grad[0]:
+            gx = g @ weight
+        if ctx.needs_input_grad[1]:
+            x2, g2 = x.reshape(-1, x.shape[-1]).contiguous(), g.reshape(-1, g.shape[-1]).contiguous()
+            m = x2.shape[0]
+            full = _typed.typed_gemm_wgrad(x2, g2, _one_segment(m, x.device), m, 1) if m > 0 else None
+            gw = full[0].t() if full is not None else g2.t() @ x2
+        return gx, gw
+
+
+def linear(x, weight, bias=None):
+    """``F.linear`` for the conv layers; CUDA tensors take LinearOP."""
+    if not x.is_cuda:
+        return F.linear(x, weight, bias)
+    out = LinearOP.apply(x, weight)
+    return out if bias is None else out + bias
+
+
+class AttentionLogitsOP(torch.autograd.Function):
+    """Both per-node logits of a GAT layer, ``(x * att_src).sum(-1)`` over every source node
+    and ``(x[:num_dst] * att_dst).sum(-1)`` (cxgnncomp/graph_conv.py:466-467), from one
+    pass over x; the backward pass reads x once more for grad_x and both parameter
+    gradients.  Host tensors use the upstream expressions."""
+
+    @staticmethod
+    def forward(ctx, x, att_src, att_dst, num_dst):
+        ctx.save_for_backward(x, att_src, att_dst)
+        ctx.num_dst = num_dst
+        if not x.is_cuda:
+            return (x * att_src).sum(dim=-1), (x[:num_dst] * att_dst).sum(dim=-1)
+        return cxgnncomp_backend._ops.attention_logits(x.contiguous(), att_src, att_dst, num_dst)
+
+    @staticmethod
+    def backward(ctx, g_src, g_dst):
+        x, att_src, att_dst = ctx.saved_tensors
+        if not x.is_cuda:
+            gx = g_src.unsqueeze(-1) * att_src
+            gx[:ctx.num_dst] += g_dst.unsqueeze(-1) * att_dst
+            ga_src = (g_src.unsqueeze(-1) * x).sum(dim=0).view_as(att_src)
+            ga_dst = (g_dst.unsqueeze(-1) * x[:ctx.num_dst]).sum(dim=0).view_as(att_dst)
+            return gx, ga_src, ga_dst, None
+        gx, ga_src, ga_dst = cxgnncomp_backend._ops.attention_logits_bwd(
+            x.contiguous(), att_src, att_dst, g_src.contiguous(), g_dst.contiguous())
+        return gx, ga_src.view_as(att_src), ga_dst.view_as(att_dst), None
 
 
 class MyGATConv(torch.nn.Module):
@@ -349,11 +424,10 @@ class MyGATConv(torch.nn.Module):
         H, C = self.heads, self.out_channels
         assert x.dim() == 2
         x = TimerOP.apply(x, "linear1", True)
-        x_src = x_dst = F.linear(x[:num_src], self.lin_src).view(-1, H, C)
+        x_src = x_dst = linear(x[:num_src], self.lin_src).view(-1, H, C)
         x_src = TimerOP.apply(x_src, "linear1", False)
         x_src = TimerOP.apply(x_src, "sum1", True)
-        alpha_src = HeadDotOP.apply(x_src, self.att_src).view(-1, H)
-        alpha_dst = HeadDotOP.apply(x_dst[:num_dst], self.att_dst).view(-1, H)
+        alpha_src, alpha_dst = AttentionLogitsOP.apply(x_src, self.att_src, self.att_dst, num_dst)
         alpha_dst = TimerOP.apply(alpha_dst, "sum1", False)
         alpha_dst = TimerOP.apply(alpha_dst, "softmax1", True)
         edge_value = self.edge_softmax(ptr=ptr, idx=idx, att_src=alpha_src, att_dst=alpha_dst,
@@ -433,7 +507,7 @@ class MyGCNConv(torch.nn.Module):
     def forward(self, x, ptr, idx, num_node):
         x = TimerOP.apply(x, "linear", True)
         mm_before = self.in_channels > self.out_channels
-        out = self.lin(x) if mm_before else x
+        out = linear(x, self.lin.weight) if mm_before else x
         out = TimerOP.apply(out, "linear", False)
         if self.normalize:
             out = TimerOP.apply(out, "aggregation", True)
@@ -445,5 +519,5 @@ class MyGCNConv(torch.nn.Module):
         else:
             out = AggrOP.apply(out, ptr, idx, num_node)
         if not mm_before:
-            out = self.lin(out)
+            out = linear(out, self.lin.weight)
         return out + self.bias if self.bias is not None else out

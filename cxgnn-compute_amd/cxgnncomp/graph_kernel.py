@@ -31,9 +31,15 @@ class SpMMValOP(torch.autograd.Function):
         x, ptr, idx, val = ctx.saved_tensors
         grad_out = grad_out.contiguous()
         grad_x = grad_val = None
+        g = _ops.transposed(ptr, idx, ctx.n, x.shape[0])       # cached with the graph
         if ctx.needs_input_grad[0]:
-            grad_x = torch.zeros_like(x)
-            cxgnncomp_backend.spmm_multihead_bwd(ptr, idx, val, grad_out, grad_x, ctx.n)
+            # spmm_multihead_bwd adds into a zeroed tensor; writing the rows of the transposed
+            # graph directly saves the fill and the read-back of the accumulation
+            grad_x = _ops.spmm(g.ptr_t, g.idx_t, grad_out, x.shape[0], val=val, val_perm=g.perm)
         if ctx.needs_input_grad[3]:
-            grad_val = _ops.sddmm_csr(ptr, idx, x, grad_out, ctx.n)[:val.shape[0]]
+            # the kernel writes the edges of the first ctx.n rows; only a tail past them needs zeros
+            grad_val = torch.empty((idx.shape[0], val.shape[1]), dtype=torch.float32, device=x.device)
+            if g.n_edges < idx.shape[0]:
+                grad_val[g.n_edges:].zero_()
+            grad_val = _ops.sddmm_csr(ptr, idx, x, grad_out, ctx.n, out=grad_val)[:val.shape[0]]
         return grad_x, None, None, grad_val, None

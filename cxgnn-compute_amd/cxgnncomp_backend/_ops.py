@@ -314,20 +314,70 @@ def edge_softmax_fwd(ptr, idx, att_dst, att_src, n_edges, slope):
 
 
 def edge_softmax_bwd(ptr, out, mask, grad, n_dst, slope):
-    """Returns (g_dst [n_dst,H], t_edge [E,H])."""
+    """Returns (g_dst [n_dst,H], t_edge [E,H]); rows of t_edge at or past ptr[n_dst] are not
+    written (the transposed gather that consumes t_edge never reads them)."""
     lib = _lib.load()
     _req(out, "out", torch.float32, 2)
     _req(grad, "grad", torch.float32, 2)
     _req(mask, "mask", torch.bool, 2)
     heads = out.shape[1]
     g_dst = torch.empty((n_dst, heads), dtype=torch.float32, device=out.device)
-    t_edge = torch.zeros_like(out)
+    t_edge = torch.empty_like(out)
     with torch.cuda.device(out.device):
         st = lib.cxg_edge_softmax_bwd_f32(ptr.data_ptr(), _lib.ptr(out), _lib.ptr(mask), _lib.ptr(grad),
                                           _lib.ptr(g_dst), _lib.ptr(t_edge), n_dst, heads, float(slope),
                                           _lib.current_stream(out.device))
     _lib.check(st)
     return g_dst, t_edge
+
+
+def attention_logits(x, att_src, att_dst, n_dst):
+    """(x[:, h, :] . att_src[h], x[:n_dst, h, :] . att_dst[h]) for x [n_src, H, C]: both
+    per-node logits of a GAT layer from one pass over x."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 3)
+    n_src, heads, channels = x.shape
+    att_src = att_src.reshape(heads, channels).contiguous()
+    att_dst = att_dst.reshape(heads, channels).contiguous()
+    _req(att_src, "att_src", torch.float32, 2)
+    _req(att_dst, "att_dst", torch.float32, 2)
+    if not 0 <= n_dst <= n_src:
+        raise ValueError("n_dst=%d outside [0, %d]" % (n_dst, n_src))
+    out_src = torch.empty(n_src, heads, dtype=torch.float32, device=x.device)
+    out_dst = torch.empty(n_dst, heads, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_attention_logits_fwd_f32(_lib.ptr(x), att_src.data_ptr(), att_dst.data_ptr(), n_src,
+                                              n_dst, heads, channels, _lib.ptr(out_src), _lib.ptr(out_dst),
+                                              _lib.current_stream(x.device))
+    _lib.check(st)
+    return out_src, out_dst
+
+
+def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst):
+    """Gradients of ``attention_logits``: (grad_x, grad_att_src, grad_att_dst), reproducible."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 3)
+    n_src, heads, channels = x.shape
+    n_dst = g_dst.shape[0]
+    att_src = att_src.reshape(heads, channels).contiguous()
+    att_dst = att_dst.reshape(heads, channels).contiguous()
+    _req(g_src, "g_src", torch.float32, 2)
+    _req(g_dst, "g_dst", torch.float32, 2)
+    if tuple(g_src.shape) != (n_src, heads) or g_dst.shape[1] != heads or n_dst > n_src:
+        raise ValueError("gradient shapes %s / %s do not fit x %s"
+                         % (tuple(g_src.shape), tuple(g_dst.shape), tuple(x.shape)))
+    grad_x = torch.empty_like(x)
+    ga_src = torch.empty(heads, channels, dtype=torch.float32, device=x.device)
+    ga_dst = torch.empty(heads, channels, dtype=torch.float32, device=x.device)
+    ws_bytes = lib.cxg_attention_logits_workspace_bytes(n_src, heads, channels)
+    ws = _workspace(ws_bytes, x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_attention_logits_bwd_f32(_lib.ptr(x), att_src.data_ptr(), att_dst.data_ptr(),
+                                              _lib.ptr(g_src), _lib.ptr(g_dst), n_src, n_dst, heads, channels,
+                                              _lib.ptr(grad_x), ga_src.data_ptr(), ga_dst.data_ptr(),
+                                              ws.data_ptr(), ws.numel(), _lib.current_stream(x.device))
+    _lib.check(st)
+    return grad_x, ga_src, ga_dst
 
 
 def csr_row_ids32(ptr, n_rows, n_edges):

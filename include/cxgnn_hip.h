@@ -301,6 +301,30 @@ int cxg_gather_rows_f32(const float* in, const int64_t* sel, float* out,
 int cxg_head_sum_f32(const float* in, float* out, int64_t n_rows, int heads,
                      int channels, void* stream);
 
+/* Per-node attention logits of a multi-head GAT layer, both in one pass over x:
+ *   out_src[n, h] = sum_c x[n, h, c] * att_src[h, c]   for n < n_src
+ *   out_dst[n, h] = sum_c x[n, h, c] * att_dst[h, c]   for n < n_dst (<= n_src)
+ * x is [n_src, heads, channels], att_* are [heads, channels].  Replaces the two
+ * broadcast-multiply-and-sum expressions of MyGATConv.forward_many
+ * (cxgnncomp/graph_conv.py:466-467). */
+int cxg_attention_logits_fwd_f32(const float* x, const float* att_src, const float* att_dst,
+                                 int64_t n_src, int64_t n_dst, int heads, int channels,
+                                 float* out_src, float* out_dst, void* stream);
+
+size_t cxg_attention_logits_workspace_bytes(int64_t n_src, int heads, int channels);
+
+/* Gradients of the logits above for g_src [n_src, heads], g_dst [n_dst, heads]:
+ *   grad_x[n, h, c]    = g_src[n, h] * att_src[h, c] + (n < n_dst) g_dst[n, h] * att_dst[h, c]
+ *   grad_att_src[h, c] = sum_n g_src[n, h] * x[n, h, c]
+ *   grad_att_dst[h, c] = sum_{n < n_dst} g_dst[n, h] * x[n, h, c]
+ * All three outputs are overwritten; the sums run in a fixed order (reproducible).
+ * The autograd of the same two expressions (cxgnncomp/graph_conv.py:466-467). */
+int cxg_attention_logits_bwd_f32(const float* x, const float* att_src, const float* att_dst,
+                                 const float* g_src, const float* g_dst, int64_t n_src,
+                                 int64_t n_dst, int heads, int channels, float* grad_x,
+                                 float* grad_att_src, float* grad_att_dst, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Index work (bit-exact)                                                     */
 /* ------------------------------------------------------------------------- */

@@ -165,3 +165,67 @@ def test_segment_gather_sum_multi_step_spans():
     got = _ops.narrow_gather_sum(pc, ic, table.cuda(), n, rows32=rows32)
     want = oracle.spmm(ptr.numpy(), idx.numpy(), table.numpy(), n)
     assert_close(_np(got), want, RTOL, ATOL, "segment_gather_sum, multi-step spans")
+
+
+ATT_SHAPES = [(4, 64), (1, 128), (8, 16), (3, 40), (2, 7), (1, 1), (4, 256), (16, 64), (8, 512), (2, 6)]
+
+
+@pytest.mark.parametrize("shape", ATT_SHAPES)
+@pytest.mark.parametrize("n_src,n_dst", [(1, 1), (1000, 0), (1000, 333), (70001, 70001), (70001, 12345)])
+def test_attention_logits_forward_backward(shape, n_src, n_dst):
+    """Both per-node GAT logits and their three gradients against the upstream expressions
+    ``(x * att).sum(-1)`` differentiated in double precision.  Tolerance: 1e-4 relative /
+    1e-5 absolute on values scaled to O(1); the parameter gradients are sums over all
+    nodes and are compared relative to their largest entry."""
+    from cxgnncomp_backend import _ops
+    H, C = shape
+    if H * C >= 1024 and n_src > 1000:
+        n_src, n_dst = 5003, min(n_dst, 5003)
+    torch.manual_seed(H * 1000 + C + n_src)
+    x = (torch.randn(n_src, H, C) / C ** 0.5)
+    a_s, a_d = torch.randn(1, H, C), torch.randn(1, H, C)
+    gs, gd = torch.randn(n_src, H), torch.randn(n_dst, H)
+    xd = x.double().requires_grad_(True)
+    asd, add = a_s.double().requires_grad_(True), a_d.double().requires_grad_(True)
+    ref_s = (xd * asd).sum(-1)
+    ref_d = (xd[:n_dst] * add).sum(-1)
+    (ref_s * gs.double()).sum().backward(retain_graph=True)
+    (ref_d * gd.double()).sum().backward()
+    announce("attention_logits H=%d C=%d n_src=%d n_dst=%d" % (H, C, n_src, n_dst))
+    out_s, out_d = _ops.attention_logits(x.cuda(), a_s.cuda(), a_d.cuda(), n_dst)
+    torch.cuda.synchronize()
+    assert out_s.shape == (n_src, H) and out_d.shape == (n_dst, H)
+    assert_close(_np(out_s), ref_s.detach().numpy(), RTOL, ATOL, "logits src")
+    assert_close(_np(out_d), ref_d.detach().numpy(), RTOL, ATOL, "logits dst")
+    announce("attention_logits_bwd H=%d C=%d n_src=%d n_dst=%d" % (H, C, n_src, n_dst))
+    gx, ga_s, ga_d = _ops.attention_logits_bwd(x.cuda(), a_s.cuda(), a_d.cuda(), gs.cuda(), gd.cuda())
+    gx2, ga_s2, ga_d2 = _ops.attention_logits_bwd(x.cuda(), a_s.cuda(), a_d.cuda(), gs.cuda(), gd.cuda())
+    torch.cuda.synchronize()
+    assert_close(_np(gx), xd.grad.numpy(), RTOL, ATOL, "grad x")
+    for got, ref, name in ((ga_s, asd.grad, "grad att_src"), (ga_d, add.grad, "grad att_dst")):
+        ref = ref.numpy().reshape(H, C)
+        scale = max(1.0, float(np.abs(ref).max()))
+        assert_close(_np(got) / scale, ref / scale, RTOL, ATOL, name)
+    assert torch.equal(ga_s, ga_s2) and torch.equal(ga_d, ga_d2) and torch.equal(gx, gx2)
+
+
+def test_attention_logits_op_autograd():
+    """The autograd wrapper used by MyGATConv: gradients flow to x and both parameters."""
+    import cxgnncomp
+    from cxgnncomp.graph_conv import AttentionLogitsOP
+    torch.manual_seed(3)
+    n, H, C, nd = 4097, 4, 32, 1500
+    x = torch.randn(n, H, C, device="cuda", requires_grad=True)
+    a_s = torch.randn(1, H, C, device="cuda", requires_grad=True)
+    a_d = torch.randn(1, H, C, device="cuda", requires_grad=True)
+    gs, gd = torch.randn(n, H, device="cuda"), torch.randn(nd, H, device="cuda")
+    announce("AttentionLogitsOP autograd")
+    s, d = AttentionLogitsOP.apply(x, a_s, a_d, nd)
+    ((s * gs).sum() + (d * gd).sum()).backward()
+    got = [x.grad.clone(), a_s.grad.clone(), a_d.grad.clone()]
+    x.grad = a_s.grad = a_d.grad = None
+    (((x * a_s).sum(-1) * gs).sum() + ((x[:nd] * a_d).sum(-1) * gd).sum()).backward()
+    for g, r in zip(got, [x.grad, a_s.grad, a_d.grad]):
+        assert g.shape == r.shape
+        scale = max(1.0, float(r.abs().max()))
+        assert_close(_np(g) / scale, _np(r) / scale, 1e-4, 2e-5, "autograd")
