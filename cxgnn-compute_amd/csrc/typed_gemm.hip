@@ -65,25 +65,44 @@ __device__ __forceinline__ bool locate_tile(const int64_t* __restrict__ seg, int
   return false;
 }
 
-template <int BN, int MT>
-__device__ __forceinline__ void store_tile(const GemmArgs& g, const v16f (&acc)[MT],
-                                           const int64_t* s_dst, int wm, int wn, int lane, int n0) {
+// Output of one block tile.  In the 32x32 MFMA accumulator a lane holds, for its column,
+// four groups of four consecutive rows; the destination rows of a group are fetched from
+// LDS together (they are 32 contiguous bytes) and the four stores follow without waits.
+// MODE 0: store, 1: read-add-store, 2: fp32 atomic add.
+template <int BN, int MT, int MODE>
+__device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&acc)[MT],
+                                                const int64_t* s_dst, int wm, int wn, int lane, int n0) {
   const int col = n0 + wn * 32 + (lane & 31);
   if (col >= g.N) return;
+  float* const base = g.c + col;
+  const int64_t ldc = g.ldc;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int rl = (wm * MT + mt) * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-      const int64_t d = s_dst[rl];
-      if (d < 0) continue;
-      float* p = g.c + d * g.ldc + col;
-      const float v = acc[mt][i];
-      if (g.atomic) unsafeAtomicAdd(p, v);
-      else if (g.accumulate) *p += v;
-      else *p = v;
+    for (int q = 0; q < 4; ++q) {
+      const int rl0 = (wm * MT + mt) * 32 + q * 8 + (lane >> 5) * 4;
+      int64_t d[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) d[j] = s_dst[rl0 + j];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (d[j] < 0) continue;
+        float* p = base + d[j] * ldc;
+        const float v = acc[mt][q * 4 + j];
+        if (MODE == 2) unsafeAtomicAdd(p, v);
+        else if (MODE == 1) *p += v;
+        else *p = v;
+      }
     }
   }
+}
+
+template <int BN, int MT>
+__device__ __forceinline__ void store_tile(const GemmArgs& g, const v16f (&acc)[MT],
+                                           const int64_t* s_dst, int wm, int wn, int lane, int n0) {
+  if (g.atomic) store_tile_mode<BN, MT, 2>(g, acc, s_dst, wm, wn, lane, n0);
+  else if (g.accumulate) store_tile_mode<BN, MT, 1>(g, acc, s_dst, wm, wn, lane, n0);
+  else store_tile_mode<BN, MT, 0>(g, acc, s_dst, wm, wn, lane, n0);
 }
 
 __device__ __forceinline__ void load_row_maps(const GemmArgs& g, int64_t row0, int64_t row_end,
@@ -111,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_f32_kernel(GemmArgs g) {
   constexpr int WPT = BN * KC / kThreads;      // W elements per thread per chunk
   __shared__ float As[2][kBM][KC + 1];
   __shared__ float Ws[2][KC][BN];
-  __shared__ int64_t s_src[kBM], s_dst[kBM];
+  __shared__ __attribute__((aligned(16))) int64_t s_src[kBM], s_dst[kBM];
   int rel = 0;
   int64_t row0 = 0, row_end = 0;
   if (!locate_tile(g.seg, g.R, blockIdx.x, rel, row0, row_end)) return;
@@ -198,7 +217,7 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_kernel(GemmArgs g) {
   constexpr int WV = BN * KC / 8 / kThreads;  // 16-byte W vectors per thread per chunk
   __shared__ __attribute__((aligned(16))) uint16_t As[2][kBM][LD];
   __shared__ __attribute__((aligned(16))) uint16_t Wt[2][BN][LD];
-  __shared__ int64_t s_src[kBM], s_dst[kBM];
+  __shared__ __attribute__((aligned(16))) int64_t s_src[kBM], s_dst[kBM];
   int rel = 0;
   int64_t row0 = 0, row_end = 0;
   if (!locate_tile(g.seg, g.R, blockIdx.x, rel, row0, row_end)) return;
@@ -278,11 +297,21 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_kernel(GemmArgs g) {
 // Six bf16 MFMAs take 3/8 of the cycles of the fp32 MFMA for the same K, which
 // turns the K, N <= 128 typed GEMM from matrix-core bound into HBM bound.
 //
-// A block owns up to G consecutive 64-row tiles of ONE relation and keeps that
-// relation's weight slab in registers, already split and in MFMA operand layout
-// (wave w: columns 32w..32w+31), so W is fetched once per 64*G rows.  A tiles are
-// fetched as whole 16-byte-per-lane row segments, split on the way into LDS, and
-// the loads of the next two tiles are in flight while the current one is multiplied.
+// A block owns up to G consecutive 64-row tiles of ONE relation and has two kinds of
+// waves.  The four consumer waves keep the relation's weight slab in registers, already
+// split and in MFMA operand layout (wave w: columns 32w..32w+31), so W is fetched once
+// per 64*G rows; they multiply a tile out of LDS and store it.  The four producer waves
+// fetch the A rows as 16-byte-per-lane row segments, split them into their bf16 parts
+// and write the parts of the NEXT tile into the other half of a double-buffered LDS
+// area while the consumers multiply.  One barrier per tile separates the two halves.
+//
+// Why two kinds of waves: a wave's memory counter completes in order, so a wave that
+// both loads and stores cannot wait for a load without also waiting for every store it
+// issued before it -- the stores of a tile then have to drain (microseconds under a
+// write-heavy load) before the next tile can be staged.  Consumer waves never wait on
+// memory: their stores (or atomics) stay in flight for as long as the hardware queue
+// allows.  Producer waves only ever wait for their own loads.  The conversion work of
+// the producers runs on the same SIMDs in the shadow of the consumers' MFMAs.
 template <int NS>
 __device__ __forceinline__ void split_bf16(float x, __bf16 (&p)[NS]) {
 #pragma unroll
@@ -292,14 +321,27 @@ __device__ __forceinline__ void split_bf16(float x, __bf16 (&p)[NS]) {
   }
 }
 
-template <int KS, int NS>
-__global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, int G) {
+constexpr int kSplitThreads = 512;         // waves 0-3 consume, waves 4-7 produce
+constexpr int kMapSlots = 8;               // row maps of tiles t-1 .. t+5 are live at once
+constexpr int kCP = 40;                    // floats per staged output row: 32 + pad; rows r and
+                                           // r + 4 (the two halves of a wave) land 32 banks apart
+
+template <int KS, int NS, bool MAPPED>
+__global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(2)))
+void typed_gemm_split_kernel(GemmArgs g, int G) {
   constexpr int KP = KS * 16 + 8;          // padded LDS row (bf16 elements)
   constexpr int LPR = KS * 4;              // lanes per A row, one float4 each
-  constexpr int RPI = kThreads / LPR;      // rows per load instruction
+  constexpr int RPI = 256 / LPR;           // rows per load instruction (256 producer threads)
   constexpr int NLD = kBM / RPI;           // load instructions per tile
-  __shared__ __attribute__((aligned(16))) uint16_t Ap[NS][kBM][KP];
-  __shared__ int64_t s_src[3][kBM], s_dst[3][kBM];
+  typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // layout: Ap[2][NS][kBM][KP] bf16, s_src / s_dst [kMapSlots][kBM] int64, then one
+  // [kBM][kCP] fp32 staging area per consumer wave for its 64 x 32 piece of the output
+  uint16_t (*Ap)[NS][kBM][KP] = reinterpret_cast<uint16_t (*)[NS][kBM][KP]>(smem);
+  int64_t (*s_src)[kBM] = reinterpret_cast<int64_t (*)[kBM]>(smem + sizeof(uint16_t) * 2 * NS * kBM * KP);
+  int64_t (*s_dst)[kBM] = s_src + kMapSlots;
+  float (*Cw)[kCP] = reinterpret_cast<float (*)[kCP]>(reinterpret_cast<unsigned char*>(s_dst + kMapSlots)) +
+                     (size_t)(threadIdx.x >> 6 & 3) * kBM;
   const int64_t span = (int64_t)kBM * G;
   int rel = -1;
   int64_t row0 = 0, row_end = 0;
@@ -319,16 +361,85 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
       t -= nt;
     }
   }
-  if (rel < 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (rel < 0) return;                       // whole block: no barrier has been passed yet
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uniform_i32(tid >> 6);
+  const bool consumer = wave < 4;
   const int n0 = (int)(slot % n_ct) * 128;
   const int K = g.K, N = g.N;
   const int64_t rows_here = (row_end - row0) < span ? (row_end - row0) : span;
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
-  // this wave's 32 columns of W[rel], split, in B-operand layout
-  v8bf bw[NS][KS];
-  {
+  // plain stores of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
+  const bool wide_store = !g.atomic && !g.accumulate && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
+                          ((uintptr_t)g.c & 15) == 0;
+
+  // ---- producer state -------------------------------------------------------------
+  const int ptid = tid & 255;
+  const int c4 = ptid % LPR, rsub = ptid / LPR;
+  const bool k_ok = 4 * c4 < K;
+  const float* A = reinterpret_cast<const float*>(g.a);
+  float4 areg0[NLD], areg1[NLD];             // rows of the next two tiles, in flight
+  int64_t m_src = -1, m_dst = -1;            // wave 4: the maps of a tile, in flight
+  // Row maps: given (MAPPED) they are fetched by wave 4, loads issued one iteration and
+  // published the next; otherwise source and destination row are the row index itself
+  // and the table is filled without any load.
+  auto maps_issue = [&](int t) {
+    m_src = -1;
+    m_dst = -1;
+    if (wave == 4 && t < n_tiles) {
+      const int64_t gr = row0 + (int64_t)t * kBM + lane;
+      if (gr < row_end) {
+        m_src = (MAPPED && g.src) ? g.src[gr] : gr;
+        m_dst = (MAPPED && g.dst) ? g.dst[gr] : gr;
+      }
+    }
+  };
+  auto maps_commit = [&](int t) {
+    if (wave == 4 && t < n_tiles) {
+      const bool bad = m_src < 0 || m_dst < 0;
+      s_src[t % kMapSlots][lane] = bad ? -1 : m_src;
+      s_dst[t % kMapSlots][lane] = bad ? -1 : m_dst;
+    }
+  };
+  // Loads are issued unconditionally (rows and columns that do not exist are redirected
+  // to an address that does and zeroed when the tile is staged): with no branch around a
+  // load the compiler counts the loads in flight exactly and waits only for the older of
+  // the two register sets.
+  auto gload = [&](float4 (&areg)[NLD], int t) {
+    const int tc = t < n_tiles ? t : n_tiles - 1;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int64_t sidx = s_src[tc % kMapSlots][i * RPI + rsub];
+      areg[i] = *reinterpret_cast<const float4*>(A + (sidx >= 0 ? sidx : 0) * g.lda + (k_ok ? 4 * c4 : 0));
+    }
+  };
+  // split the rows held in areg and write the parts of tile t into its LDS half
+  auto stage = [&](const float4 (&areg)[NLD], int t) {
+    uint16_t (*dst)[kBM][KP] = Ap[t & 1];
+    const int tc = t < n_tiles ? t : n_tiles - 1;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int row = i * RPI + rsub;
+      const bool live = k_ok && s_src[tc % kMapSlots][row] >= 0;
+      const float v[4] = {live ? areg[i].x : 0.f, live ? areg[i].y : 0.f, live ? areg[i].z : 0.f,
+                          live ? areg[i].w : 0.f};
+      v4bf part[NS];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        __bf16 parts[NS];
+        split_bf16<NS>(v[j], parts);
+#pragma unroll
+        for (int q = 0; q < NS; ++q) part[q][j] = parts[q];
+      }
+#pragma unroll
+      for (int q = 0; q < NS; ++q) *reinterpret_cast<v4bf*>(&dst[q][row][4 * c4]) = part[q];
+    }
+  };
+
+  // ---- prologue -------------------------------------------------------------------
+  v8bf bw[NS][KS];                           // consumers: this wave's 32 columns of W[rel], split
+  if (consumer) {
     const float* W = reinterpret_cast<const float*>(g.w) + (int64_t)rel * K * N;
     const int col = n0 + wave * 32 + (lane & 31);
 #pragma unroll
@@ -343,88 +454,132 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_split_kernel(GemmArgs g, 
         for (int q = 0; q < NS; ++q) bw[q][s][j] = parts[q];
       }
     }
+  } else {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      maps_issue(t);
+      maps_commit(t);
+    }
+  }
+  __syncthreads();                           // maps of tiles 0..3 visible
+  if (!consumer) {
+    gload(areg0, 0);
+    gload(areg1, 1);
+    stage(areg0, 0);
+    gload(areg0, 2);
+    maps_issue(4);
   }
 
-  const int c4 = tid % LPR, rsub = tid / LPR;
-  const bool k_ok = 4 * c4 < K;
-  const float* A = reinterpret_cast<const float*>(g.a);
-  auto load_maps = [&](int t) {
-    if (tid < kBM && t < n_tiles) {
-      const int64_t gr = row0 + (int64_t)t * kBM + tid;
-      int64_t sidx = -1, didx = -1;
-      if (gr < row_end) {
-        sidx = g.src ? g.src[gr] : gr;
-        didx = g.dst ? g.dst[gr] : gr;
-        if (sidx < 0 || didx < 0) { sidx = -1; didx = -1; }
-      }
-      s_src[t % 3][tid] = sidx;
-      s_dst[t % 3][tid] = didx;
-    }
-  };
-  auto gload = [&](float4 (&areg)[NLD], int t) {
-    if (t >= n_tiles) return;
+  // ---- one barrier per tile ---------------------------------------------------------
+  // Iteration t, consumers: multiply tile t out of LDS half t&1, store it.
+  // Iteration t, producers: publish the maps of tile t+4 (their loads were issued an
+  // iteration ago), split tile t+1 into half (t+1)&1 (the consumers finished reading it
+  // before this iteration's barrier), start the loads of tile t+3 into the registers
+  // that tile t+1 just left, and the loads of the maps of tile t+5.
+  // (the two kinds of waves run separate loops with the same number of barriers, so the
+  // registers of one role are not live in the other)
+  if (consumer) {
+    // Plain stores leave through the wave's own LDS area in row order: a lane stores 16
+    // bytes and an instruction covers 8 rows x 128 bytes -- a quarter of the store
+    // instructions, so four times the bytes in flight for the same depth of the memory
+    // queue.  The eight pieces of tile t-1 are read back and stored between the k-steps
+    // of tile t, in the shadow of its MFMAs.
+    constexpr int PPS = 8 / KS;              // pieces per k-step
+    auto piece_read = [&](int it) -> float4 {
+      return *reinterpret_cast<const float4*>(&Cw[it * 8 + (lane >> 3)][(lane & 7) * 4]);
+    };
+    auto piece_row = [&](int it, int t) -> int64_t { return s_dst[t % kMapSlots][it * 8 + (lane >> 3)]; };
+    auto piece_store = [&](const float4& v, int64_t d) {
+      if (d >= 0) *reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wave * 32 + (lane & 7) * 4) = v;
+    };
+    for (int t = 0; t < n_tiles; ++t) {
+      __syncthreads();
+      const uint16_t (*src)[kBM][KP] = Ap[t & 1];
+      const bool drain = wide_store && t > 0;
+      float4 pv[PPS];
+      int64_t pd[PPS];
+      v16f acc[2];
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int64_t sidx = s_src[t % 3][i * RPI + rsub];
-      areg[i] = (sidx >= 0 && k_ok) ? *reinterpret_cast<const float4*>(A + sidx * g.lda + 4 * c4)
-                                    : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-  };
-  // One tile: stage its rows (already in registers) into LDS, start the loads of
-  // tile t + 2 into the same registers, multiply, store.
-  auto tile_step = [&](float4 (&areg)[NLD], int t) {
+      for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const float v[4] = {areg[i].x, areg[i].y, areg[i].z, areg[i].w};
-      typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
-      v4bf part[NS];
+        for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
+      // operands of k-step s+1 are read while step s multiplies (two register sets)
+      v8bf ap[2][2][NS];
+      auto read_ap = [&](int s) {
+        const int k = s * 16 + (lane >> 5) * 8;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        __bf16 parts[NS];
-        split_bf16<NS>(v[j], parts);
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int q = 0; q < NS; ++q) part[q][j] = parts[q];
-      }
-      const int row = i * RPI + rsub;
+          for (int q = 0; q < NS; ++q)
+            ap[s & 1][mt][q] = *reinterpret_cast<const v8bf*>(&src[q][mt * 32 + (lane & 31)][k]);
+      };
+      read_ap(0);
 #pragma unroll
-      for (int q = 0; q < NS; ++q) *reinterpret_cast<v4bf*>(&Ap[q][row][4 * c4]) = part[q];
-    }
-    load_maps(t + 2);
-    __syncthreads();
-    gload(areg, t + 2);
-    v16f acc[2];
+      for (int s = 0; s < KS; ++s) {
+        if (s + 1 < KS) read_ap(s + 1);
+        if (drain) {
+          if (s > 0) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+            for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u]);
+          }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const int row = mt * 32 + (lane & 31), k = s * 16 + (lane >> 5) * 8;
-        v8bf ap[NS];
-#pragma unroll
-        for (int q = 0; q < NS; ++q) ap[q] = *reinterpret_cast<const v8bf*>(&Ap[q][row][k]);
+          for (int u = 0; u < PPS; ++u) {
+            pv[u] = piece_read(s * PPS + u);
+            pd[u] = piece_row(s * PPS + u, t - 1);
+          }
+        }
+        // the two accumulators alternate, so consecutive MFMAs never depend on each other
 #pragma unroll
         for (int order = NS - 1; order >= 0; --order)
 #pragma unroll
           for (int i = 0; i <= order; ++i)
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[i], bw[order - i][s], acc[mt], 0, 0, 0);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+#ifdef CXG_EXP_NO_MFMA
+              if (s == 0 && i == 0 && order == 0)
+#endif
+              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s & 1][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
+            }
+      }
+      if (drain) {
+#pragma unroll
+        for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u]);
+      }
+#ifdef CXG_EXP_NO_STORE
+      if (acc[0][0] == 12345.678f && acc[1][3] == 4.5f)
+#endif
+      if (wide_store) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            Cw[mt * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)][lane & 31] = acc[mt][i];
+      } else {
+        store_tile<128, 2>(g, acc, s_dst[t % kMapSlots], 0, wave, lane, n0);
       }
     }
-    store_tile<128, 2>(g, acc, s_dst[t % 3], 0, wave, lane, n0);
-    __syncthreads();   // every wave is done with Ap before the next tile is staged
-  };
-
-  float4 areg0[NLD], areg1[NLD];
-  load_maps(0);
-  load_maps(1);
-  __syncthreads();
-  gload(areg0, 0);
-  gload(areg1, 1);
-  for (int t = 0; t < n_tiles; t += 2) {
-    tile_step(areg0, t);
-    if (t + 1 < n_tiles) tile_step(areg1, t + 1);
+    if (wide_store) {
+#ifdef CXG_EXP_NO_STORE
+      if (lane == 77)
+#endif
+#pragma unroll
+      for (int it = 0; it < 8; ++it) piece_store(piece_read(it), piece_row(it, n_tiles - 1));
+    }
+  } else {
+    // two iterations per trip, so each register set has a fixed role
+    for (int t = 0; t < n_tiles; t += 2) {
+      __syncthreads();
+      maps_commit(t + 4);
+      stage(areg1, t + 1);
+      gload(areg1, t + 3);
+      maps_issue(t + 5);
+      if (t + 1 >= n_tiles) break;
+      __syncthreads();
+      maps_commit(t + 5);
+      stage(areg0, t + 2);
+      gload(areg0, t + 4);
+      maps_issue(t + 6);
+    }
   }
 }
 
@@ -443,7 +598,7 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
   constexpr int RPI = kThreads / LPR;      // rows per load instruction
   constexpr int NLD = kBM / RPI;           // load instructions per tile
   __shared__ __attribute__((aligned(16))) uint16_t Ap[kBM][KP];
-  __shared__ int64_t s_src[3][kBM], s_dst[3][kBM];
+  __shared__ __attribute__((aligned(16))) int64_t s_src[3][kBM], s_dst[3][kBM];
   const int64_t span = (int64_t)kBM * G;
   int rel = -1;
   int64_t row0 = 0, row_end = 0;
@@ -538,6 +693,14 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
   }
 }
 
+// Dynamic LDS above the default 64 KB limit has to be enabled per kernel (once per device).
+template <typename KernelT>
+hipError_t allow_lds(KernelT kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             (int)bytes);
+}
+
 int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64_t M, int K, int N,
                int R, unsigned flags) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
@@ -570,16 +733,28 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
     const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
     CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
     const dim3 grid((unsigned)n_blocks);
+#define CXG_SPLIT_LAUNCH(KS, NSV, MAP)                                                         \
+  do {                                                                                         \
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_gemm_split_kernel<KS, NSV, MAP>, lds));            \
+    hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, NSV, MAP>), grid, dim3(cxg::kSplitThreads), lds, st, \
+                       g, G);                                                                  \
+  } while (0)
 #define CXG_SPLIT(KS)                                                                          \
   do {                                                                                         \
-    if (flags & CXG_GEMM_SPLIT_BF16X3)                                                         \
-      hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, 2>), grid, dim3(cxg::kThreads), 0, st, g, G); \
-    else                                                                                       \
-      hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, 3>), grid, dim3(cxg::kThreads), 0, st, g, G); \
+    const int ns = (flags & CXG_GEMM_SPLIT_BF16X3) ? 2 : 3;                                    \
+    const size_t lds = (size_t)2 * ns * cxg::kBM * (KS * 16 + 8) * sizeof(uint16_t) +          \
+                       (size_t)2 * cxg::kMapSlots * cxg::kBM * sizeof(int64_t) +               \
+                       (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float);                        \
+    const bool mapped = src_idx || dst_idx;                                                    \
+    if (ns == 2 && mapped) CXG_SPLIT_LAUNCH(KS, 2, true);                                      \
+    else if (ns == 2) CXG_SPLIT_LAUNCH(KS, 2, false);                                          \
+    else if (mapped) CXG_SPLIT_LAUNCH(KS, 3, true);                                            \
+    else CXG_SPLIT_LAUNCH(KS, 3, false);                                                       \
   } while (0)
     if (K <= 32) CXG_SPLIT(2);
     else if (K <= 64) CXG_SPLIT(4);
     else CXG_SPLIT(8);
+#undef CXG_SPLIT_LAUNCH
 #undef CXG_SPLIT
     CXG_LAUNCH_CHECK("typed_gemm_split_kernel");
     return CXG_OK;

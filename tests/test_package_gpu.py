@@ -365,3 +365,31 @@ def test_head_dot_op(heads, channels):
     assert_close(_np(ac.grad), ar.grad.numpy(), RTOL, 2 * ATOL, "head dot grad att")
     # host tensors take the upstream expression
     assert torch.allclose(HeadDotOP.apply(x, att), (x * att).sum(-1))
+
+
+@pytest.mark.parametrize("k,n", [(128, 256), (256, 256), (256, 40), (300, 64), (30, 16), (64, 7)])
+@pytest.mark.parametrize("rows", [1, 5000, 70001])
+def test_linear_op_matches_torch(k, n, rows):
+    """The conv layers' linear: forward and input gradient from the library GEMM, weight
+    gradient from the typed weight-gradient kernel (one launch per 128 input columns), with
+    the library GEMM for shapes it does not take.  Reference: F.linear differentiated in
+    double precision; 1e-4 relative / 2e-5 absolute on values scaled to O(1)."""
+    from cxgnncomp.graph_conv import linear
+    torch.manual_seed(k * n + rows)
+    x = torch.randn(rows, k)
+    w = torch.randn(n, k) / k ** 0.5
+    b = torch.randn(n)
+    g = torch.randn(rows, n) / max(1.0, rows ** 0.5)
+    xd, wd, bd = (t.double().requires_grad_(True) for t in (x, w, b))
+    (torch.nn.functional.linear(xd, wd, bd) * g.double()).sum().backward()
+    xc, wc, bc = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    announce("linear op k=%d n=%d rows=%d" % (k, n, rows))
+    out = linear(xc, wc, bc)
+    (out * g.cuda()).sum().backward()
+    torch.cuda.synchronize()
+    ref = torch.nn.functional.linear(xd, wd, bd).detach()
+    assert_close(out.detach().cpu().numpy(), ref.numpy(), 1e-4, 2e-5, "linear out")
+    for got, want, name in ((xc.grad, xd.grad, "grad x"), (wc.grad, wd.grad, "grad w"), (bc.grad, bd.grad, "grad b")):
+        assert got.shape == want.shape
+        scale = max(1.0, float(want.abs().max()))
+        assert_close(got.cpu().numpy() / scale, want.numpy() / scale, 1e-4, 2e-5, name)
