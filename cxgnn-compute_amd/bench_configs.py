@@ -214,7 +214,20 @@ def c3(iters):
     out = torch.empty(E, H, device="cuda")
     report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),
            E * (8 * H * C + 16) + 4 * E * H, 2 * E * H * C)
-    del x, g
+    # single-head F=128 (several edges per gather step), same graph
+    x1, g1 = x.view(N, H * C)[:, :128].contiguous(), g.view(N, H * C)[:, :128].contiguous()
+    report("c3", "sddmm_csr H=1 C=128", timeit(lambda: _ops.sddmm_csr(ptr, idx, x1, g1, N), iters),
+           E * (4 * 128 + 8) + 4 * N * 128 + 4 * E, 2 * E * 128)
+    del x1, g1
+    # per-node attention logits of the layer (both from one pass over x) and their gradients
+    a_s, a_d = torch.randn(H, C, device="cuda"), torch.randn(H, C, device="cuda")
+    gs = torch.randn(N, H, device="cuda")
+    report("c3", "attention_logits fwd H=4 C=64 (src and dst logits)",
+           timeit(lambda: _ops.attention_logits(x, a_s, a_d, N), iters), 4 * N * H * C + 8 * N * H, 4 * N * H * C)
+    report("c3", "attention_logits bwd H=4 C=64 (grad x, grad att_src, grad att_dst)",
+           timeit(lambda: _ops.attention_logits_bwd(x, a_s, a_d, gs, gs), iters), 8 * N * H * C + 8 * N * H,
+           8 * N * H * C)
+    del x, g, gs
     # the configuration's layer: GAT 128 -> 4 heads x 64, forward + backward through the
     # softmax and the edge-weighted aggregation including the edge-value gradient
     import cxgnncomp

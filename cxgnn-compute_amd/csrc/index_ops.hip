@@ -78,25 +78,27 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(const int64_t* __re
   }
 }
 
-// perm / idx_t from the sorted packed values (in place over `perm`), ptr_t from the
-// boundaries of the sorted keys: position k is the first edge of every column in
-// (key[k-1], key[k]], and the last position also closes the columns after its own.
+// perm / idx_t from the sorted packed values (in place over `perm`); ptr_t[c] = number of
+// edges whose source is < c, by a search of the sorted keys per column (one thread per
+// column: the columns may outnumber the edges by far, e.g. a sampled layer over all nodes).
 __global__ void transpose_unpack_kernel(const uint32_t* __restrict__ sorted_key, int64_t n_edges,
                                         int64_t n_cols, int64_t* __restrict__ perm,
                                         int64_t* __restrict__ idx_t, int64_t* __restrict__ ptr_t) {
   const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= n_edges) return;
-  const uint64_t v = (uint64_t)perm[k];
-  perm[k] = (int64_t)(v & 0xffffffffull);
-  idx_t[k] = (int64_t)(v >> 32);
-  // (ids are < n_cols by contract; the clamp keeps a broken input from writing past ptr_t)
-  const int64_t last = n_cols - 1;
-  int64_t c = sorted_key[k], prev = k > 0 ? (int64_t)sorted_key[k - 1] : -1;
-  if (c > last) c = last;
-  if (prev > last) prev = last;
-  for (int64_t j = prev + 1; j <= c; ++j) ptr_t[j] = k;
-  if (k == n_edges - 1)
-    for (int64_t j = c + 1; j <= n_cols; ++j) ptr_t[j] = n_edges;
+  if (k < n_edges) {
+    const uint64_t v = (uint64_t)perm[k];
+    perm[k] = (int64_t)(v & 0xffffffffull);
+    idx_t[k] = (int64_t)(v >> 32);
+  }
+  if (k <= n_cols) {
+    int64_t lo = 0, hi = n_edges;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if ((int64_t)sorted_key[mid] < k) lo = mid + 1;
+      else hi = mid;
+    }
+    ptr_t[k] = lo;
+  }
 }
 
 __global__ void fill_i64_kernel(int64_t* __restrict__ out, int64_t n, int64_t value) {
@@ -200,8 +202,9 @@ int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows
     CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, keys, sorted_key, packed,
                                             reinterpret_cast<uint64_t*>(perm), (size_t)n_edges, 0,
                                             cxg::bits_for(n_cols > 1 ? n_cols : 2), st));
-    hipLaunchKernelGGL(cxg::transpose_unpack_kernel, grid, block, 0, st, sorted_key, n_edges, n_cols,
-                       perm, idx_t, ptr_t);
+    const int64_t work = (n_edges > n_cols + 1) ? n_edges : n_cols + 1;
+    hipLaunchKernelGGL(cxg::transpose_unpack_kernel, dim3((unsigned)cxg::ceil_div(work, cxg::kBlock)), block, 0,
+                       st, sorted_key, n_edges, n_cols, perm, idx_t, ptr_t);
     CXG_LAUNCH_CHECK("transpose_unpack_kernel");
     return CXG_OK;
   }

@@ -535,9 +535,6 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
           for (int i = 0; i <= order; ++i)
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
-#ifdef CXG_EXP_NO_MFMA
-              if (s == 0 && i == 0 && order == 0)
-#endif
               acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s & 1][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
             }
       }
@@ -545,9 +542,6 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
         for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u]);
       }
-#ifdef CXG_EXP_NO_STORE
-      if (acc[0][0] == 12345.678f && acc[1][3] == 4.5f)
-#endif
       if (wide_store) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -559,9 +553,6 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       }
     }
     if (wide_store) {
-#ifdef CXG_EXP_NO_STORE
-      if (lane == 77)
-#endif
 #pragma unroll
       for (int it = 0; it < 8; ++it) piece_store(piece_read(it), piece_row(it, n_tiles - 1));
     }

@@ -197,3 +197,21 @@ def test_csr_row_ids_bit_exact(case):
     torch.cuda.synchronize()
     assert np.array_equal(_np(got), want)
     assert got32.dtype == torch.int32 and np.array_equal(_np(got32).astype(np.int64), want)
+
+
+def test_csr_transpose_far_more_columns_than_edges():
+    """A sampled layer whose sources are numbered over all nodes: 600 edges, a million columns."""
+    from cxgnncomp_backend import _ops
+    rng = np.random.default_rng(5)
+    n_rows, n_src = 40, 1000003
+    deg = rng.integers(0, 30, n_rows)
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    idx = rng.integers(0, n_src, int(ptr[-1])).astype(np.int64)
+    idx[:3] = [n_src - 1, 0, n_src - 1]
+    want_ptr, want_idx, want_perm = oracle.csr_transpose(ptr, idx, n_rows, n_src)
+    announce("csr_transpose far more columns than edges")
+    ptr_t, idx_t, perm, n_edges = _ops.csr_transpose(torch.from_numpy(ptr).cuda(), torch.from_numpy(idx).cuda(),
+                                                     n_rows, n_src)
+    assert np.array_equal(_np(ptr_t), want_ptr)
+    assert np.array_equal(_np(idx_t), want_idx)
+    assert np.array_equal(_np(perm), want_perm)
