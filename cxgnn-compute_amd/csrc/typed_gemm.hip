@@ -557,19 +557,25 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       for (int it = 0; it < 8; ++it) piece_store(piece_read(it), piece_row(it, n_tiles - 1));
     }
   } else {
-    // two iterations per trip, so each register set has a fixed role
-    for (int t = 0; t < n_tiles; t += 2) {
-      __syncthreads();
-      maps_commit(t + 4);
-      stage(areg1, t + 1);
-      gload(areg1, t + 3);
-      maps_issue(t + 5);
-      if (t + 1 >= n_tiles) break;
-      __syncthreads();
-      maps_commit(t + 5);
-      stage(areg0, t + 2);
-      gload(areg0, t + 4);
-      maps_issue(t + 6);
+    // Four iterations per trip: each register set keeps a fixed role, and the wait at the
+    // top of the loop body -- the one place where the compiler cannot tell how many
+    // younger loads are in flight and waits for all of them -- comes once in four tiles.
+    for (int t = 0; t < n_tiles; t += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; u += 2) {
+        if (t + u >= n_tiles) break;
+        __syncthreads();
+        maps_commit(t + u + 4);
+        stage(areg1, t + u + 1);
+        gload(areg1, t + u + 3);
+        maps_issue(t + u + 5);
+        if (t + u + 1 >= n_tiles) break;
+        __syncthreads();
+        maps_commit(t + u + 5);
+        stage(areg0, t + u + 2);
+        gload(areg0, t + u + 4);
+        maps_issue(t + u + 6);
+      }
     }
   }
 }
