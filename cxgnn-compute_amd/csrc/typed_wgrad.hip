@@ -117,20 +117,29 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
         s_dst[t % 3][tid] = didx;
       }
     };
+    // Loads are issued unconditionally: rows and columns that do not exist are redirected
+    // to an address that does and zeroed when the tile is staged (a select between a
+    // loaded vector and a zero vector made the compiler route the load through scratch).
     auto gload = [&](float4 (&ar)[4], float4 (&gr4)[4], int t) {
-      if (t >= n_tiles) return;
+      const int tc = t < n_tiles ? t : n_tiles - 1;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int64_t sidx = s_src[t % 3][mg * 4 + i], didx = s_dst[t % 3][mg * 4 + i];
-        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-        ar[i] = (sidx >= 0 && ka_ok) ? *reinterpret_cast<const float4*>(g.a + sidx * g.lda + 4 * c4) : z;
-        gr4[i] = (didx >= 0 && ng_ok) ? *reinterpret_cast<const float4*>(g.g + didx * g.ldg + n0 + 4 * c4) : z;
+        const int64_t sidx = s_src[tc % 3][mg * 4 + i], didx = s_dst[tc % 3][mg * 4 + i];
+        ar[i] = *reinterpret_cast<const float4*>(g.a + (sidx >= 0 ? sidx : 0) * g.lda + (ka_ok ? 4 * c4 : 0));
+        gr4[i] = *reinterpret_cast<const float4*>(g.g + (didx >= 0 ? didx : 0) * g.ldg + (ng_ok ? n0 + 4 * c4 : 0));
       }
     };
     // registers (4 rows x 4 columns) -> LDS [column][4 consecutive rows], split into parts
-    auto stage = [&](const float4 (&r4)[4], uint16_t (&dst)[NS][128][kMP]) {
-      const float v[4][4] = {{r4[0].x, r4[0].y, r4[0].z, r4[0].w}, {r4[1].x, r4[1].y, r4[1].z, r4[1].w},
-                             {r4[2].x, r4[2].y, r4[2].z, r4[2].w}, {r4[3].x, r4[3].y, r4[3].z, r4[3].w}};
+    auto stage = [&](const float4 (&r4)[4], uint16_t (&dst)[NS][128][kMP], const int64_t* rows, bool col_ok) {
+      float v[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool live = col_ok && rows[mg * 4 + i] >= 0;
+        v[i][0] = live ? r4[i].x : 0.f;
+        v[i][1] = live ? r4[i].y : 0.f;
+        v[i][2] = live ? r4[i].z : 0.f;
+        v[i][3] = live ? r4[i].w : 0.f;
+      }
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         v4bf out[NS];
@@ -146,8 +155,8 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
       }
     };
     auto tile_step = [&](float4 (&ar)[4], float4 (&gr4)[4], int t) {
-      stage(ar, At);
-      stage(gr4, Gt);
+      stage(ar, At, s_src[t % 3], ka_ok);
+      stage(gr4, Gt, s_dst[t % 3], ng_ok);
       load_maps(t + 2);
       __syncthreads();
       gload(ar, gr4, t + 2);
