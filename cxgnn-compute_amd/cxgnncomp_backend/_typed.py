@@ -168,11 +168,25 @@ def typed_linear_s2d(vin, weights, output, src_id, dst_id, types, in_feat_tile=3
 # --------------------------------------------------------------------------- #
 # fused relational aggregate + transform  (binding.cpp:46-47, 53-54)
 # --------------------------------------------------------------------------- #
-def _edge_segments(ptr, idx, rel, n, num_rel):
+def _edge_segments(ptr, idx, rel, n, num_rel, want_perm=False):
     n_edges = int(ptr[n].item())
     perm, seg = rel_segment(rel[:n_edges].contiguous(), num_rel)
     rows = _ops.csr_row_ids(ptr, n, n_edges)
+    if want_perm:
+        return n_edges, idx[:n_edges][perm], rows[perm], seg, perm
     return n_edges, idx[:n_edges][perm], rows[perm], seg
+
+
+_ARANGE_CACHE = {}
+
+
+def _edge_positions(n, device):
+    """arange(n) on the device, kept for the segment sums over per-edge rows."""
+    key = (device, )
+    t = _ARANGE_CACHE.get(key)
+    if t is None or t.shape[0] < n:
+        t = _ARANGE_CACHE[key] = torch.arange(n, dtype=torch.int64, device=device)
+    return t[:n]
 
 
 def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=None, precision=None):
@@ -229,6 +243,7 @@ def _weight_grad(x, g, src, dst, seg, shape):
 # pairs and Y fits the memory budget; sparser inputs (sampled blocks with many
 # relations) use the fused gather-GEMM-scatter launch.
 RGCN_DENSE_MAX_BYTES = 64 << 30
+RGCN_EDGE_ROWS_MAX_BYTES = 64 << 30        # per-edge rows of the sparse strategy; above: atomic scatter
 
 
 class _RelGraph:
@@ -302,13 +317,22 @@ class _RgcnFusedFunction(torch.autograd.Function):
             ctx.rg = rg
             ctx.save_for_backward(x, weights, ptr)
             return out
-        n_edges, src, dst, seg = _edge_segments(ptr, idx, rel, n, R)
+        n_edges, src, dst, seg, perm = _edge_segments(ptr, idx, rel, n, R, want_perm=True)
+        ctx.n_edges = n_edges
+        ctx.per_edge = 4 * n_edges * max(K, N) <= RGCN_EDGE_ROWS_MAX_BYTES
+        if ctx.per_edge:
+            # one output row per edge, written once in CSR order, then the plain sum over
+            # each destination's (consecutive) rows: no atomics, reproducible
+            tmp = torch.empty((n_edges, N), dtype=torch.float32, device=x.device)
+            typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=perm, out=tmp)
+            out = _ops.spmm(ptr, _edge_positions(n_edges, x.device), tmp, n, mean=mean)
+            ctx.save_for_backward(x, weights, ptr, src, dst, seg, perm, idx)
+            return out
         out = torch.zeros((n, N), dtype=torch.float32, device=x.device)
         typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=dst, out=out, atomic=True)
         if mean:
             out *= _inv_degree(ptr, n).unsqueeze(1)
         ctx.save_for_backward(x, weights, ptr, src, dst, seg)
-        ctx.n_edges = n_edges
         return out
 
     @staticmethod
@@ -336,8 +360,17 @@ class _RgcnFusedFunction(torch.autograd.Function):
                     gw = torch.mm(x.t(), gy.view(n_src, R * N))
                 gw = gw.view(K, R, N).permute(1, 0, 2).contiguous()
             return gx, None, None, gw, None, None, None
-        src, dst, seg = ctx.saved_tensors[3:]
-        if ctx.needs_input_grad[0]:
+        src, dst, seg = ctx.saved_tensors[3:6]
+        if ctx.needs_input_grad[0] and ctx.per_edge:
+            # per-edge rows g[dst(e)] @ W[rel(e)]^T in CSR order, summed per source over the
+            # reversed graph (whose edge permutation says where each source's rows are)
+            perm, idx = ctx.saved_tensors[6:8]
+            tmp = torch.empty((ctx.n_edges, K), dtype=torch.float32, device=x.device)
+            typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), seg, ctx.n_edges, src_idx=dst,
+                       dst_idx=perm, out=tmp)
+            gt = _ops.transposed(ptr, idx, n, n_src)
+            gx = _ops.spmm(gt.ptr_t, gt.perm, tmp, n_src)
+        elif ctx.needs_input_grad[0]:
             gx = torch.zeros_like(x)
             typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), seg, ctx.n_edges, src_idx=dst,
                        dst_idx=src, out=gx, atomic=True)

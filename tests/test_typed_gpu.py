@@ -165,14 +165,18 @@ def test_rgcn_fused_toy_all_ones():
     assert torch.all(out.cpu() == 3968.0)
 
 
-@pytest.mark.parametrize("strategy", ["transform_first", "gather_gemm_scatter"])
+@pytest.mark.parametrize("strategy", ["transform_first", "per_edge_rows", "gather_gemm_scatter"])
 @pytest.mark.parametrize("K,N,R", [(128, 128, 16), (64, 32, 3)])
 def test_rgcn_fused_forward_backward(K, N, R, strategy, monkeypatch):
+    """The three strategies of the fused relational layer: dense transform of every (source,
+    relation) pair, one GEMM row per edge summed per destination, atomic scatter."""
     import cxgnncomp_backend as B
     from cxgnncomp import synthetic as S
     from cxgnncomp_backend import _typed
-    if strategy == "gather_gemm_scatter":
+    if strategy != "transform_first":
         monkeypatch.setattr(_typed, "RGCN_DENSE_MAX_BYTES", 0)    # rules the dense path out
+    if strategy == "gather_gemm_scatter":
+        monkeypatch.setattr(_typed, "RGCN_EDGE_ROWS_MAX_BYTES", 0)   # and the per-edge rows
     assert _typed._use_dense(40000, 3000, R, N) == (strategy == "transform_first")
     ptr, idx, etype, _ = S.hetero_graph(3000, 40000, num_rel=R, seed=4)
     n = ptr.shape[0] - 1
