@@ -18,8 +18,8 @@ def rel_schedule(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel):
     target_r (original row ids); then a [num_rel, L] table, L = len(num_node_in_layer)-1,
     whose entry [r, l] is the number of kept rows among the first num_node_in_layer[l]
     rows.  Returns the 3*num_rel + 1 tensors in that order, on the inputs' device
-    (upstream works on CPU tensors); graphs on the GPU use the library's edge filter
-    once per relation."""
+    (upstream works on CPU tensors); graphs on the GPU are handled for all relations at
+    once after one stable sort by relation."""
     n = csr_ptr.shape[0] - 1
     num_rel = int(num_rel)
     if csr_ptr.is_cuda:
@@ -65,16 +65,40 @@ def _rel_schedule_device(csr_ptr, csr_idx, rel, num_node_in_layer, num_rel, n):
             break
         reached.append(i + 1)
         pos = i
-    at = torch.tensor(reached, dtype=torch.int64, device=csr_ptr.device)
-    table = torch.zeros((num_rel, max(num_layer, 0)), dtype=torch.int64, device=csr_ptr.device)
-    rel32 = rel.to(torch.int32).contiguous()
+    dev = csr_ptr.device
+    table = torch.zeros((num_rel, max(num_layer, 0)), dtype=torch.int64, device=dev)
+    e = int(csr_ptr[n].item()) if n > 0 else 0
+    if e == 0:
+        empty = torch.zeros(0, dtype=torch.int64, device=dev)
+        out = []
+        for r in range(num_rel):
+            out += [torch.zeros(1, dtype=torch.int64, device=dev), empty, empty]
+        out.append(table)
+        return out
+    # All relations at once.  A stable sort by relation keeps each relation's edges in
+    # their original (row-major) order, so within a relation the rows of its edges are
+    # non-decreasing: the kept rows and their edge counts are the runs of the combined
+    # key relation * n + row.
+    from . import _typed
+    rel32 = rel[:e].to(torch.int32).contiguous()
+    perm, seg = _typed.rel_segment(rel32, num_rel)
+    rows = _ops.csr_row_ids(csr_ptr, n, e)
+    r_rows = rows[perm]
+    r_idx = csr_idx[:e][perm]
+    key = rel32.to(torch.int64)[perm] * n + r_rows
+    uniq, counts = torch.unique_consecutive(key, return_counts=True)
+    bounds = torch.searchsorted(uniq, torch.arange(num_rel + 1, dtype=torch.int64, device=dev) * n)
+    ends = torch.cat([counts.new_zeros(1), torch.cumsum(counts, 0)])
+    target_all = uniq % n
+    if reached:
+        at = torch.tensor(reached, dtype=torch.int64, device=dev)
+        q = torch.arange(num_rel, dtype=torch.int64, device=dev).unsqueeze(1) * n + at.unsqueeze(0)
+        table[:, :len(reached)] = torch.searchsorted(uniq, q) - bounds[:num_rel].unsqueeze(1)
+    seg_h, bounds_h = seg.tolist(), bounds.tolist()
     out = []
     for r in range(num_rel):
-        sub_ptr, sub_idx, target, row_off = _ops.filter_edges(csr_ptr, csr_idx, rel=rel32, keep_rel=r,
-                                                              want_target=True)
-        out += [sub_ptr, sub_idx, target]
-        if reached:
-            table[r, :len(reached)] = row_off[at]
+        e0, e1, u0, u1 = seg_h[r], seg_h[r + 1], bounds_h[r], bounds_h[r + 1]
+        out += [ends[u0:u1 + 1] - e0, r_idx[e0:e1], target_all[u0:u1]]
     out.append(table)
     return out
 
