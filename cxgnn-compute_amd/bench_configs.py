@@ -174,6 +174,40 @@ def c2(iters):
             h.sum().backward()
         report("c2", "3-layer GCN fwd+bwd, %s aggregation" % ("1/deg-weighted" if normalize else "sum"),
                timeit(step, iters))
+    del convs, bns, xg
+    # the remaining aggregation entry points of the backend on the same graph, F = 128
+    import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
+    E, F = idx.shape[0], 128
+    xe = torch.randn(E, F, device="cuda")
+    dest = _ops.csr_row_ids(ptr, n, E)
+    report("c2", "gather (edge -> node sum, rows grouped by destination once) F=128", timeit(lambda: B.gather(xe, dest, n), iters),
+           E * (4 * F + 8) + 8 * n * F, E * F)
+    del xe
+    mask = (torch.rand(E, device="cuda") < 0.5)
+    out = torch.zeros(n, F, device="cuda")
+    report("c2", "selective_aggr (half of the edges masked) F=128",
+           timeit(lambda: B.selective_aggr(x, ptr, idx, mask, out, n), iters),
+           spmm_bytes(n, E, F) // 2 + E + 4 * n * F, E * F)
+    gsel = torch.zeros(n, F, device="cuda")
+    report("c2", "selective_aggr_bwd F=128", timeit(lambda: B.selective_aggr_bwd(out, ptr, idx, mask, gsel, n), iters),
+           spmm_bytes(n, E, F) // 2 + 9 * E + 4 * n * F, E * F)
+    import cxgnncomp
+    gp, gtar = cxgnncomp.neighbor_grouping(ptr, 32)
+    out.zero_()
+    report("c2", "target_aggr over neighbor groups of 32 (%d groups) F=128" % gtar.shape[0],
+           timeit(lambda: B.target_aggr(x, gp, idx, gtar, out, gtar.shape[0]), iters),
+           spmm_bytes(gtar.shape[0], E, F) + 8 * gtar.shape[0], 2 * E * F)
+    xs = torch.randn(n, device="cuda")
+    report("c2", "spmv (unit values)", timeit(lambda: B.spmv(ptr, idx, xs, n), iters), E * 12 + 12 * n, E)
+    report("c2", "edge_value_degree", timeit(lambda: B.edge_value_degree(ptr, n, E), iters), 8 * n + 4 * E)
+    p32, i32 = ptr.int(), idx.int()
+    report("c2", "GSpMM_u MAX (int32 CSR) F=128", timeit(lambda: B.GSpMM_u(p32, i32, x, B.REDUCEOP.MAX), iters),
+           E * (4 * F + 4) + 4 * n * F, E * F)
+    ev = torch.rand(E, device="cuda")
+    report("c2", "GSpMM_u_e SUM x MUL (int32 CSR) F=128",
+           timeit(lambda: B.GSpMM_u_e(p32, i32, ev, x, B.REDUCEOP.SUM, B.COMPUTEOP.MUL), iters),
+           E * (4 * F + 8) + 4 * n * F, 2 * E * F)
 
 
 def c3(iters):
@@ -336,6 +370,42 @@ def c4(iters):
     _last_spread = tuple((E / N) * v for v in _last_spread)
     report("c4", "torch.mm [1M,128]x[128,128] x 20 (library GEMM of the same flops, no gather, for scale)",
            t_mm, E * 8 * K, flops, MFMA_F32)
+    # the remaining relational entry points
+    xr = torch.randn(R * (N // R), K, device="cuda") / 8         # [R * nodes, F] pre-transformed features
+    nodes_r = N // R
+    idx_r = idx % nodes_r
+    report("c4", "aggr_rel forward (relation-offset gather) F=128",
+           timeit(lambda: B.aggr_rel(xr, ptr, idx_r, rel32, N, R), iters), spmm_bytes(N, E, K) + 4 * E, E * K)
+    xrg = xr.clone().requires_grad_(True)
+    gn = torch.randn(N, K, device="cuda") / 16
+
+    def aggr_rel_step():
+        xrg.grad = None
+        B.aggr_rel(xrg, ptr, idx_r, rel32, N, R).backward(gn)
+    report("c4", "aggr_rel forward + backward (gather over the transposed combined index) F=128", timeit(aggr_rel_step, iters))
+    del xr, xrg
+    oe2 = torch.zeros(E, K, device="cuda")
+    report("c4", "typed_linear_s2e (out[e] += x[src[e]] W[type[e]]), 6 bf16 products",
+           timeit(lambda: B.typed_linear_s2e(x, w, oe2, idx, rel32), max(2, iters // 2)),
+           E * (4 * K + 8 * K + 12) + 4 * R * K * K, flops)
+    del oe2
+    on = torch.zeros(N, K, device="cuda")
+    report("c4", "typed_linear_s2d (atomic out[dst[e]] += x[src[e]] W[type[e]])",
+           timeit(lambda: B.typed_linear_s2d(x, w, on, idx, rows, rel32), max(2, iters // 2)),
+           fused_bytes, flops)
+    del on
+    from cxgnncomp.typed_linear import TypedLinearE2EOP
+    xeg = torch.randn(E, K, device="cuda").requires_grad_(True)
+    wg = w.clone().requires_grad_(True)
+    pre = TypedLinearE2EOP.preprocess(w, etype)
+    ge = torch.randn(E, K, device="cuda") / 16
+
+    def e2e_step():
+        xeg.grad = None
+        wg.grad = None
+        TypedLinearE2EOP.apply(xeg, wg, etype, pre).backward(ge)
+    report("c4", "TypedLinearE2EOP forward + backward (edge-level x, preprocessed)", timeit(e2e_step, max(2, iters // 3)))
+    del xeg, ge, pre
     layer = cxgnncomp.MyRGCNConv(K, K, R).cuda()
     xg = x.clone().requires_grad_(True)
 

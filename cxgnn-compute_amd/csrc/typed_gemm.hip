@@ -370,8 +370,8 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const int64_t rows_here = (row_end - row0) < span ? (row_end - row0) : span;
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
-  // plain stores of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
-  const bool wide_store = !g.atomic && !g.accumulate && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
+  // stores (or read-add-stores) of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
+  const bool wide_store = !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
                           ((uintptr_t)g.c & 15) == 0;
 
   // ---- producer state -------------------------------------------------------------
@@ -489,8 +489,16 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       return *reinterpret_cast<const float4*>(&Cw[it * 8 + (lane >> 3)][(lane & 7) * 4]);
     };
     auto piece_row = [&](int it, int t) -> int64_t { return s_dst[t % kMapSlots][it * 8 + (lane >> 3)]; };
+    const bool add_old = g.accumulate != 0;
     auto piece_store = [&](const float4& v, int64_t d) {
-      if (d >= 0) *reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wave * 32 + (lane & 7) * 4) = v;
+      if (d < 0) return;
+      float4* const p = reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wave * 32 + (lane & 7) * 4);
+      if (add_old) {
+        const float4 o = *p;
+        *p = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
+      } else {
+        *p = v;
+      }
     };
     for (int t = 0; t < n_tiles; ++t) {
       __syncthreads();

@@ -39,14 +39,16 @@ def _segments(rel, num_rel):
 
 
 def typed_matmul(a, b, rel, num_valid_item=-1, src_idx=None, dst_idx=None, seq_output=False,
-                 bf16=False):
+                 bf16=False, covers_output=False):
     """c[out_row(i)] = a[in_row(i)] @ b[rel[i]].
 
     no index:                 in_row = out_row = i
     src_idx only:             in_row = out_row = src_idx[i]      ("single index")
     src_idx, seq_output:      in_row = src_idx[i], out_row = i
     src_idx and dst_idx:      in_row = src_idx[i], out_row = dst_idx[i]
-    Rows with a negative (or out-of-range) index are skipped.
+    Rows with a negative (or out-of-range) index are skipped; output rows no input row maps
+    to are zero.  ``covers_output=True`` is the caller's promise that every output row is
+    written (e.g. the index is a permutation), which saves the zero fill of the output.
     """
     assert a.shape[1] == b.shape[1], "incompatible dimensions"
     assert a.is_contiguous(), "matrix A must be contiguous"
@@ -85,6 +87,6 @@ def typed_matmul(a, b, rel, num_valid_item=-1, src_idx=None, dst_idx=None, seq_o
         dst = torch.where(n_rows_eff < n_out, n_rows_eff, torch.full_like(n_rows_eff, -1))
     if src is not None:
         src = torch.where(src < a.shape[0], src, torch.full_like(src, -1))
-    c = torch.zeros((n_out, N), device=a.device, dtype=torch.float32)
+    c = (torch.empty if covers_output else torch.zeros)((n_out, N), device=a.device, dtype=torch.float32)
     _typed.typed_gemm(a, b, seg, n_rows, src_idx=src, dst_idx=dst, out=c, bf16=bf16)
     return c

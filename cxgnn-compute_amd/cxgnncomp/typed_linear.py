@@ -79,8 +79,9 @@ class TypedLinearE2EOP(torch.autograd.Function):
             sorted_types, num_item, indices, count = TypedLinearE2EOP.preprocess(weights, types, thres)
         x = x.contiguous()
         weights = weights.contiguous()
-        # padding rows carry indices >= num_item; typed_matmul drops them
-        output = typed_matmul(x, weights, sorted_types, num_item, indices)
+        # padding rows carry indices >= num_item; typed_matmul drops them.  The real rows
+        # are a permutation of 0..num_item-1, so every output row is written.
+        output = typed_matmul(x, weights, sorted_types, num_item, indices, covers_output=True)
         ctx.save_for_backward(x, weights, types, indices, sorted_types)
         ctx.num_item = num_item
         return output[:num_item]
@@ -92,7 +93,7 @@ class TypedLinearE2EOP(torch.autograd.Function):
         grad_x = grad_w = None
         if ctx.needs_input_grad[0]:
             wt = torch.transpose(weights, 1, 2).contiguous()
-            grad_x = typed_matmul(grad_out, wt, sorted_types, ctx.num_item, indices)
+            grad_x = typed_matmul(grad_out, wt, sorted_types, ctx.num_item, indices, covers_output=True)
         if ctx.needs_input_grad[1]:
             perm, seg = _typed.rel_segment(types.contiguous(), weights.shape[0])
             grad_w = _weight_grad(x, grad_out, perm, seg, weights.shape)

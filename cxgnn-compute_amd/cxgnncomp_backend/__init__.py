@@ -215,7 +215,10 @@ def spmv(ptr, idx, input, num_dst):
 # gather (edge -> node scatter-add)  (binding.cpp:19)
 # --------------------------------------------------------------------------- #
 class _GatherFunction(torch.autograd.Function):
-    """GatherFunction (src/cpp/src/aggr.cu:395-448)."""
+    """GatherFunction (src/cpp/src/aggr.cu:395-448).  Upstream adds every edge row to its
+    node with atomics; here the edge positions are grouped by destination once per
+    destination array (one stable sort, cached) and every node sums its own rows --
+    several times faster than fp32 atomics at these widths, and reproducible."""
 
     @staticmethod
     def forward(ctx, input, dest, num_node):
@@ -223,7 +226,13 @@ class _GatherFunction(torch.autograd.Function):
         if n <= 0:
             raise ValueError("num_node must be > 0")
         ctx.save_for_backward(dest)
-        return _ops.scatter_add_rows(input.contiguous(), dest, n)
+        input = input.contiguous()
+        if input.dim() != 2 or input.shape[0] != dest.shape[0]:
+            raise ValueError("input must be [num_edge, F] with one row per entry of dest")
+        if dest.shape[0] == 0:
+            return torch.zeros((n, input.shape[1]), dtype=torch.float32, device=input.device)
+        g = _ops.dest_groups(dest, n)
+        return _ops.spmm(g.ptr, g.perm, input, n)
 
     @staticmethod
     def backward(ctx, grad_out):

@@ -137,6 +137,7 @@ _GRAPH_CACHE_CAP = 8
 
 def clear_graph_cache():
     _GRAPH_CACHE.clear()
+    _DEST_CACHE.clear()
 
 
 def set_graph_cache_capacity(n):
@@ -184,6 +185,35 @@ def transposed(ptr, idx, n_rows, n_src):
         _GRAPH_CACHE[key] = g
         while len(_GRAPH_CACHE) > _GRAPH_CACHE_CAP:
             _GRAPH_CACHE.popitem(last=False)
+    return g
+
+
+class DestGroups:
+    """Edge positions grouped by destination: ptr [n+1] and perm [E] (stable), kept with the
+    destination array they were built from."""
+
+    __slots__ = ("ptr", "perm", "_keep")
+
+    def __init__(self, ptr, perm, keep):
+        self.ptr, self.perm, self._keep = ptr, perm, keep
+
+
+_DEST_CACHE = collections.OrderedDict()
+
+
+def dest_groups(dest, n_rows):
+    """Cached DestGroups of an edge -> node destination array (one stable sort)."""
+    key = (dest.data_ptr(), dest.shape[0], dest._version, n_rows, dest.device.index)
+    g = _DEST_CACHE.get(key)
+    if g is not None:
+        _DEST_CACHE.move_to_end(key)
+        return g
+    ptr, _, perm = coo_to_csr(dest, dest, n_rows)
+    g = DestGroups(ptr, perm, dest)
+    if _GRAPH_CACHE_CAP > 0:
+        _DEST_CACHE[key] = g
+        while len(_DEST_CACHE) > _GRAPH_CACHE_CAP:
+            _DEST_CACHE.popitem(last=False)
     return g
 
 

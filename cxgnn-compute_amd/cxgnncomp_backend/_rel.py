@@ -1,6 +1,8 @@
 """Masked / targeted / relational aggregation of the reference backend
 (binding.cpp:26-31, 45-47) on top of cxg_spmm_ext_f32 and
 cxg_spmm_scatter_atomic_f32."""
+import collections
+
 import torch
 
 from . import _lib, _ops
@@ -96,8 +98,31 @@ def target_aggr_backward(grad_in, ptr, idx, targets, grad_out, num_node):
     spmm_ext(g.ptr_t, g.idx_t, grad_in, grad_out.shape[0], grad_out, accumulate=True, src_map=targets)
 
 
+_KEY_CACHE = collections.OrderedDict()
+
+
+def _rel_keys(idx, etype, n_edges, stride, num_rel):
+    """Combined row index etype[e] * stride + idx[e] of every edge, kept per (idx, etype):
+    with it the relational gather is the plain SpMM, and its transposed graph (cached
+    like any other) gives the backward pass without atomics."""
+    key = (idx.data_ptr(), etype.data_ptr(), idx._version, etype._version, n_edges, stride, idx.device.index)
+    k = _KEY_CACHE.get(key)
+    if k is not None:
+        _KEY_CACHE.move_to_end(key)
+        return k[0]
+    rel64 = etype[:n_edges].to(torch.int64)
+    if n_edges and (int(rel64.min()) < 0 or int(rel64.max()) >= num_rel):
+        raise ValueError("relation ids must lie in [0, %d)" % num_rel)
+    k = rel64 * stride + idx[:n_edges]
+    _KEY_CACHE[key] = (k, idx, etype)
+    while len(_KEY_CACHE) > 4:
+        _KEY_CACHE.popitem(last=False)
+    return k
+
+
 class _AggrRelFunction(torch.autograd.Function):
-    """AggrRelFunction (src/cpp/src/rel_spmm.cu:37-136)."""
+    """AggrRelFunction (src/cpp/src/rel_spmm.cu:37-136).  Upstream's backward scatters with
+    atomics; here it is the gather over the transposed graph of the combined index."""
 
     @staticmethod
     def forward(ctx, input, ptr, idx, etype, num_node, num_rel):
@@ -107,19 +132,18 @@ class _AggrRelFunction(torch.autograd.Function):
         num_rel = int(num_rel)
         if input.shape[0] % num_rel != 0:
             raise ValueError("input rows (%d) must be num_rel (%d) x nodes" % (input.shape[0], num_rel))
-        ctx.save_for_backward(ptr, idx, etype)
-        ctx.n, ctx.num_rel, ctx.shape = n, num_rel, input.shape
-        out = torch.empty((n, input.shape[1]), dtype=torch.float32, device=input.device)
-        return spmm_ext(ptr, idx, input.contiguous(), n, out, rel=etype,
-                        rel_stride=input.shape[0] // num_rel)
+        stride = input.shape[0] // num_rel
+        n_edges = int(ptr[n].item())
+        keys = _rel_keys(idx, etype, n_edges, stride, num_rel)
+        ctx.save_for_backward(ptr, keys)
+        ctx.n, ctx.rows = n, input.shape[0]
+        return _ops.spmm(ptr, keys, input.contiguous(), n)
 
     @staticmethod
     def backward(ctx, grad_out):
-        ptr, idx, etype = ctx.saved_tensors
-        gx = torch.zeros(ctx.shape, dtype=torch.float32, device=grad_out.device)
-        scatter_atomic(ptr, idx, grad_out.contiguous(), gx, ctx.n, rel=etype,
-                       rel_stride=ctx.shape[0] // ctx.num_rel)
-        return gx, None, None, None, None, None
+        ptr, keys = ctx.saved_tensors
+        g = _ops.transposed(ptr, keys, ctx.n, ctx.rows)
+        return _ops.spmm(g.ptr_t, g.idx_t, grad_out.contiguous(), ctx.rows), None, None, None, None, None
 
 
 def aggr_rel(input, ptr, idx, etype, num_node, num_rel):
