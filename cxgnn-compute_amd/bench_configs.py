@@ -406,6 +406,29 @@ def c4(iters):
         TypedLinearE2EOP.apply(xeg, wg, etype, pre).backward(ge)
     report("c4", "TypedLinearE2EOP forward + backward (edge-level x, preprocessed)", timeit(e2e_step, max(2, iters // 3)))
     del xeg, ge, pre
+    from cxgnncomp.typed_linear import (TypedLinearS2DAggrMMOP, TypedLinearS2DMMAggrOP, TypedLinearS2DSort,
+                                        TypedLinearS2EOP)
+    pre_s2e = TypedLinearS2EOP.preprocess(w, etype, idx, 256)
+    report("c4", "TypedLinearS2EOP forward (node-level x gathered per edge, preprocessed)",
+           timeit(lambda: TypedLinearS2EOP.apply(x, w, etype, idx, pre_s2e), max(2, iters // 3)),
+           E * (4 * K + 4 * K + 16) + 4 * R * K * K, flops)
+    del pre_s2e
+    xr1 = x.clone().requires_grad_(True)
+    wr1 = w.clone().requires_grad_(True)
+
+    def op_step(op):
+        def run():
+            xr1.grad = None
+            wr1.grad = None
+            op(xr1, wr1, ptr, idx, etype, N).backward(gn)
+        return run
+    report("c4", "RGCNOP = TypedLinearS2DMMAggrOP fwd+bwd (16 x dense transform + masked aggregation)",
+           timeit(op_step(TypedLinearS2DMMAggrOP.apply), max(2, iters // 3)))
+    report("c4", "RGCNOP2 = TypedLinearS2DAggrMMOP fwd+bwd (16 x masked aggregation + dense transform)",
+           timeit(op_step(TypedLinearS2DAggrMMOP.apply), max(2, iters // 3)))
+    report("c4", "RGCNOP_sorted = TypedLinearS2DSort fwd+bwd (torch ops over relation segments, as upstream)",
+           timeit(op_step(TypedLinearS2DSort), 2))
+    del xr1, wr1
     layer = cxgnncomp.MyRGCNConv(K, K, R).cuda()
     xg = x.clone().requires_grad_(True)
 

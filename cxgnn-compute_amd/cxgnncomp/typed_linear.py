@@ -129,8 +129,9 @@ class TypedLinearS2EOP(torch.autograd.Function):
         x = x.contiguous()
         weights = weights.contiguous()
         ctx.save_for_backward(x, weights, types, src_idx)
+        # every real edge row is written exactly once (indices is a permutation of them)
         output = typed_matmul(x, weights, sorted_types, num_item, new_src_idx[indices].contiguous(),
-                              indices)
+                              indices, covers_output=True)
         return output[:num_item]
 
     @staticmethod
@@ -141,9 +142,13 @@ class TypedLinearS2EOP(torch.autograd.Function):
         perm, seg = _typed.rel_segment(types[:n].contiguous(), weights.shape[0])
         grad_x = grad_w = None
         if ctx.needs_input_grad[0]:
-            grad_x = torch.zeros_like(x)
+            # per-edge rows g[e] @ W[type[e]]^T, then every source sums its own rows (the
+            # edge positions grouped by source are kept with src_idx): no atomics
+            per_edge = torch.empty((n, x.shape[1]), dtype=torch.float32, device=x.device)
             _typed.typed_gemm(grad_out, torch.transpose(weights, 1, 2).contiguous(), seg, n, src_idx=perm,
-                              dst_idx=src_idx[perm], out=grad_x, atomic=True)
+                              dst_idx=perm, out=per_edge)
+            groups = _ops.dest_groups(src_idx[:n], x.shape[0])
+            grad_x = _ops.spmm(groups.ptr, groups.perm, per_edge, x.shape[0])
         if ctx.needs_input_grad[1]:
             grad_w = _typed._weight_grad(x, grad_out, src_idx[perm].contiguous(), perm, seg, weights.shape)
         return grad_x, grad_w, None, None, None, None, None
