@@ -422,11 +422,11 @@ def c4(iters):
             wr1.grad = None
             op(xr1, wr1, ptr, idx, etype, N).backward(gn)
         return run
-    report("c4", "RGCNOP = TypedLinearS2DMMAggrOP fwd+bwd (16 x dense transform + masked aggregation)",
+    report("c4", "RGCNOP = TypedLinearS2DMMAggrOP fwd+bwd (transform all nodes for all relations, then aggregate)",
            timeit(op_step(TypedLinearS2DMMAggrOP.apply), max(2, iters // 3)))
-    report("c4", "RGCNOP2 = TypedLinearS2DAggrMMOP fwd+bwd (16 x masked aggregation + dense transform)",
+    report("c4", "RGCNOP2 = TypedLinearS2DAggrMMOP fwd+bwd (aggregate per (destination, relation), then transform)",
            timeit(op_step(TypedLinearS2DAggrMMOP.apply), max(2, iters // 3)))
-    report("c4", "RGCNOP_sorted = TypedLinearS2DSort fwd+bwd (torch ops over relation segments, as upstream)",
+    report("c4", "TypedLinearS2DSort fwd+bwd (relation-segmented edges, one typed GEMM)",
            timeit(op_step(TypedLinearS2DSort), 2))
     del xr1, wr1
     layer = cxgnncomp.MyRGCNConv(K, K, R).cuda()

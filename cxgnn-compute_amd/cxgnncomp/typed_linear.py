@@ -154,65 +154,61 @@ class TypedLinearS2EOP(torch.autograd.Function):
         return grad_x, grad_w, None, None, None, None, None
 
 
-class TypedLinearS2DMMAggrOP(torch.autograd.Function):
-    """RGCN layer as R x (dense transform of all nodes, masked aggregation) (:191-221)."""
+def TypedLinearS2DMMAggrOP_apply(x, weights, ptr, idx, rel, num_center):
+    return _typed._RgcnFusedFunction.apply(x, ptr, idx, weights, rel, num_center, False, True)
 
-    @staticmethod
-    def forward(ctx, x, weights, ptr, idx, rel, num_center):
-        ctx.save_for_backward(x, weights, ptr, idx, rel)
-        output = torch.zeros([num_center, weights.shape[-1]], device=x.device)
-        for i in range(weights.shape[0]):
-            cxgnncomp_backend.selective_aggr(torch.mm(x, weights[i]), ptr, idx, (rel == i), output,
-                                             num_center)
-        return output
 
-    @staticmethod
-    def backward(ctx, grad_out):
-        x, weights, ptr, idx, rel = ctx.saved_tensors
-        grad_out = grad_out.contiguous()
-        grad_x = torch.zeros_like(x)
-        grad_weights = []
-        num_center = grad_out.shape[0]
-        for i in range(weights.shape[0]):
-            g_sel = torch.zeros([x.shape[0], grad_out.shape[-1]], device=x.device)
-            cxgnncomp_backend.selective_aggr_bwd(grad_out, ptr, idx, (rel == i), g_sel, num_center)
-            grad_x += torch.mm(g_sel, weights[i].t())
-            grad_weights.append(torch.mm(x.t(), g_sel))
-        return grad_x, torch.stack(grad_weights), None, None, None, None
+class TypedLinearS2DMMAggrOP:
+    """RGCN layer as "transform every node with every relation's weight, then aggregate"
+    (:191-221; upstream: one torch.mm and one masked aggregation per relation).  Here the R
+    transforms are one dense typed GEMM against the concatenated weights and the R masked
+    aggregations one SpMM over the combined (source, relation) index -- the same values in
+    two launches; gradients for x and the weights."""
+
+    apply = staticmethod(TypedLinearS2DMMAggrOP_apply)
 
 
 class TypedLinearS2DAggrMMOP(torch.autograd.Function):
-    """RGCN layer as R x (masked aggregation, dense transform of the centers) (:224-258)."""
+    """RGCN layer as "aggregate per relation, then transform the centers" (:224-258;
+    upstream: one masked aggregation and one torch.mm per relation).  The R masked
+    aggregations are one SpMM into rows keyed by (destination, relation) and the R
+    transforms one GEMM [n, R*K] x [R*K, N]; the backward pass mirrors it."""
 
     @staticmethod
     def forward(ctx, x, weights, ptr, idx, rel, num_center):
-        output = torch.zeros([num_center, weights.shape[-1]], device=x.device)
-        aggr_outputs = []
-        for i in range(weights.shape[0]):
-            aggr = torch.zeros([num_center, weights.shape[-2]], device=x.device)
-            cxgnncomp_backend.selective_aggr(x, ptr, idx, (rel == i), aggr, num_center)
-            output += torch.mm(aggr, weights[i])
-            aggr_outputs.append(aggr)
-        ctx.save_for_backward(x, weights, ptr, idx, rel, torch.stack(aggr_outputs))
-        return output
+        n = int(num_center)
+        x = x.contiguous()
+        weights = weights.contiguous()
+        R, K, N = weights.shape
+        ptr_dr, idx_dr = _typed.dst_rel_graph(ptr, idx, rel, n, R)
+        z = _ops.spmm(ptr_dr, idx_dr, x, n * R)                     # [n*R, K]
+        ctx.save_for_backward(x, weights, ptr_dr, idx_dr, z)
+        ctx.n = n
+        return torch.mm(z.view(n, R * K), weights.view(R * K, N))
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, weights, ptr, idx, rel, aggr_outputs = ctx.saved_tensors
+        x, weights, ptr_dr, idx_dr, z = ctx.saved_tensors
         grad_out = grad_out.contiguous()
-        grad_x = torch.zeros_like(x)
-        grad_weights = []
-        num_center = grad_out.shape[0]
-        for i in range(weights.shape[0]):
-            grad_mm = torch.mm(grad_out, weights[i].t())
-            grad_weights.append(torch.mm(aggr_outputs[i].t(), grad_out))
-            cxgnncomp_backend.selective_aggr_bwd(grad_mm, ptr, idx, (rel == i), grad_x, num_center)
-        return grad_x, torch.stack(grad_weights), None, None, None, None
+        R, K, N = weights.shape
+        n = ctx.n
+        grad_x = grad_w = None
+        if ctx.needs_input_grad[0]:
+            gz = torch.mm(grad_out, weights.view(R * K, N).t())         # [n, R*K]
+            g = _ops.transposed(ptr_dr, idx_dr, n * R, x.shape[0])
+            grad_x = _ops.spmm(g.ptr_t, g.idx_t, gz.view(n * R, K), x.shape[0])
+        if ctx.needs_input_grad[1]:
+            grad_w = torch.mm(z.view(n, R * K).t(), grad_out).view(R, K, N)
+        return grad_x, grad_w, None, None, None, None
 
 
 def TypedLinearS2DSort(x, weights, ptr, idx, rel, num_center, count=None):
-    """Pure-torch relation-segmented RGCN (auto-differentiable; runs on CPU tensors too)
-    (:262-310)."""
+    """Relation-segmented RGCN (:262-310): upstream sorts the edges by relation and runs one
+    gather + F.linear + index_add_ per relation in torch.  GPU tensors take the fused
+    relational layer, which segments the edges the same way (stable sort by relation) and
+    does the R products in one typed GEMM; CPU tensors run the torch composition."""
+    if x.is_cuda:
+        return _typed._RgcnFusedFunction.apply(x, ptr, idx, weights, rel, num_center, False, False)
     dst = torch.repeat_interleave(torch.arange(num_center, device=x.device),
                                   ptr[1:num_center + 1] - ptr[:num_center])
     num_rel = weights.shape[0]

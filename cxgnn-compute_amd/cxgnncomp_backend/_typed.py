@@ -296,7 +296,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
     gradients are computed here."""
 
     @staticmethod
-    def forward(ctx, x, ptr, idx, weights, rel, num_node, mean=False):
+    def forward(ctx, x, ptr, idx, weights, rel, num_node, mean=False, force_dense=False):
         n = as_int(num_node)
         if n == 0:
             n = ptr.shape[0] - 1
@@ -308,7 +308,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
         n_src = x.shape[0]
         ctx.n, ctx.mean = n, mean
         n_edges = int(ptr[n].item())
-        ctx.dense = _use_dense(n_edges, n_src, R, N)
+        ctx.dense = force_dense or _use_dense(n_edges, n_src, R, N)
         if ctx.dense:
             rg = _rel_graph(ptr, idx, rel, n, n_src, R)
             wcat = weights.permute(1, 0, 2).reshape(1, K, R * N).contiguous()
@@ -359,7 +359,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
                 if gw is None:
                     gw = torch.mm(x.t(), gy.view(n_src, R * N))
                 gw = gw.view(K, R, N).permute(1, 0, 2).contiguous()
-            return gx, None, None, gw, None, None, None
+            return gx, None, None, gw, None, None, None, None
         src, dst, seg = ctx.saved_tensors[3:6]
         if ctx.needs_input_grad[0] and ctx.per_edge:
             # per-edge rows g[dst(e)] @ W[rel(e)]^T in CSR order, summed per source over the
@@ -376,7 +376,29 @@ class _RgcnFusedFunction(torch.autograd.Function):
                        dst_idx=src, out=gx, atomic=True)
         if ctx.needs_input_grad[3]:
             gw = _weight_grad(x, grad_out, src, dst, seg, weights.shape)
-        return gx, None, None, gw, None, None, None
+        return gx, None, None, gw, None, None, None, None
+
+
+_DST_REL_CACHE = collections.OrderedDict()
+
+
+def dst_rel_graph(ptr, idx, rel, n, R):
+    """CSR with one row per (destination, relation) pair, row d * R + r holding the sources of
+    d's edges of relation r in their original order: (ptr_dr [n*R+1], idx_dr [E]); cached per
+    (ptr, idx, rel).  The aggregate-then-transform RGCN sums into these rows."""
+    key = (ptr.data_ptr(), idx.data_ptr(), rel.data_ptr(), ptr.shape[0], idx.shape[0], n, R,
+           ptr._version, idx._version, rel._version, ptr.device.index)
+    hit = _DST_REL_CACHE.get(key)
+    if hit is not None:
+        _DST_REL_CACHE.move_to_end(key)
+        return hit[0], hit[1]
+    e = int(ptr[n].item())
+    rows = _ops.csr_row_ids(ptr, n, e)
+    ptr_dr, idx_dr, _ = _ops.coo_to_csr(idx[:e].contiguous(), rows * R + rel[:e].to(torch.int64), n * R)
+    _DST_REL_CACHE[key] = (ptr_dr, idx_dr, (ptr, idx, rel))
+    while len(_DST_REL_CACHE) > _REL_CACHE_CAP:
+        _DST_REL_CACHE.popitem(last=False)
+    return ptr_dr, idx_dr
 
 
 def _inv_degree(ptr, n):

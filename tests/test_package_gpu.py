@@ -183,6 +183,30 @@ def test_rgcn_op_variants(opname):
     assert_close(_np(wg.grad) / sc, want_gw / sc, RTOL, 2 * ATOL, opname + " grad w")
 
 
+def test_rgcn_sorted_variant_on_gpu():
+    """TypedLinearS2DSort with GPU tensors: same values and gradients as the torch composition
+    of the reference (restated in oracle/pyref.py) in double precision."""
+    import cxgnncomp
+    ptr, idx, etype = _hetero()
+    n = ptr.shape[0] - 1
+    K, N, R = 64, 32, 5
+    torch.manual_seed(23)
+    x = torch.randn(n, K) / 16
+    w = torch.randn(R, K, N) / 2
+    g = torch.randn(n, N) / 4
+    want, want_gx, want_gw = _rgcn_reference(x, w, ptr, idx, etype, n, g)
+    for fn in (cxgnncomp.TypedLinearS2DSort,):
+        xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+        announce("%s on GPU tensors" % fn.__name__)
+        out = fn(xg, wg, ptr.cuda(), idx.cuda(), etype.cuda(), n)
+        out.backward(g.cuda())
+        torch.cuda.synchronize()
+        assert_close(_np(out), want, RTOL, 2 * ATOL, "sorted fwd")
+        assert_close(_np(xg.grad), want_gx, RTOL, 2 * ATOL, "sorted grad x")
+        sc = float(np.abs(want_gw).max())
+        assert_close(_np(wg.grad) / sc, want_gw / sc, RTOL, 2 * ATOL, "sorted grad w")
+
+
 def test_rgcn_named_variants_and_prune_path():
     import cxgnncomp
     import cxgnncomp_backend as B
