@@ -144,6 +144,15 @@ def _typed_rows(vin, weights, output, types, src_id, dst_id, atomic):
         return
     perm, seg = rel_segment(types[:num].contiguous(), weights.shape[0])
     src = perm if src_id is None else src_id[perm]
+    if atomic and 4 * num * weights.shape[2] <= RGCN_EDGE_ROWS_MAX_BYTES:
+        # several rows share a destination: instead of fp32 atomics, one product row per
+        # input row (written once, in input order), then every destination sums its own
+        # rows (positions grouped by destination once per dst_id array) and adds them
+        per_row = torch.empty((num, weights.shape[2]), dtype=torch.float32, device=vin.device)
+        typed_gemm(vin, weights, seg, num, src_idx=src, dst_idx=perm, out=per_row)
+        groups = _ops.dest_groups(dst_id[:num], output.shape[0])
+        output += _ops.spmm(groups.ptr, groups.perm, per_row, output.shape[0])
+        return
     dst = perm if dst_id is None else dst_id[perm]
     typed_gemm(vin, weights, seg, num, src_idx=src, dst_idx=dst, out=output, accumulate=True,
                atomic=atomic)
