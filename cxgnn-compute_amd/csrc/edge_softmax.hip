@@ -1,8 +1,9 @@
 // Per-destination edge softmax (GAT attention) and other row reductions over
 // narrow per-edge data (a few floats per edge) for gfx950.
 //
-// Work decomposition ("three-tier row blocks").  A block of 4 wavefronts owns 256
-// consecutive rows, 64 per wave.
+// Two work decompositions.
+// "Three-tier row blocks" (narrow_gather_sum, and the softmax with a head count that is
+// not 1, 2, 4 or 8).  A block of 4 wavefronts owns 256 consecutive rows, 64 per wave.
 //   * rows of at most kShortDeg edges: one row per lane;
 //   * rows of at most kWaveDeg edges: one row at a time by a whole wave, lanes
 //     striding over the row's edges, wave reduction at the end;
@@ -10,6 +11,10 @@
 //     reduction, so that a 17k-edge hub is a chain of ~70 steps instead of ~270.
 // Power-law graphs have millions of degree-1..8 rows and a few hundred rows with
 // more than 10k edges; each tier keeps its lanes busy on its share.
+// "Edge-parallel walk" (the softmax with 1, 2, 4 or 8 heads): rows of at most kWaveDeg
+// edges are visited one EDGE per lane, 64 consecutive edges at a time, with segmented
+// scans for the per-row reductions (see SegmentWalk); longer rows as above.  Every
+// per-edge array is then read and written in whole contiguous lines.
 //
 //   forward  (edge_softmax_fwd, src/cpp/src/edge_softmax.cu:3-42):
 //     t = leaky_relu(att_dst[r,h] + att_src[idx[e],h]);  out = softmax_row(t);
@@ -163,7 +168,7 @@ struct BlockScope {
 
 // short_fn(r, begin, end): one lane per short row.  coop_fn(scope, r, begin, end):
 // wave-uniform (WaveScope) or block-uniform (BlockScope) arguments.
-template <class ShortFn, class CoopFn>
+template <int TIERS = kTiers, class ShortFn, class CoopFn>
 __device__ __forceinline__ void tiered_rows(const int64_t* __restrict__ ptr, int64_t n_rows,
                                             ShortFn short_fn, CoopFn coop_fn) {
   __shared__ unsigned long long s_very_long[kWavesPerBlock];
@@ -176,9 +181,9 @@ __device__ __forceinline__ void tiered_rows(const int64_t* __restrict__ ptr, int
   int64_t b = 0, e = 0;
   if (valid) { b = ptr[r]; e = ptr[r + 1]; }
   const int64_t deg = e - b;
-  if ((kTiers & 1) && valid && deg <= kShortDeg) short_fn(r, b, e);
-  uint64_t todo = __ballot((kTiers & 2) && valid && deg > kShortDeg && deg <= kWaveDeg);
-  const uint64_t very_long = __ballot((kTiers & 4) && valid && deg > kWaveDeg);
+  if ((TIERS & 1) && valid && deg <= kShortDeg) short_fn(r, b, e);
+  uint64_t todo = __ballot((TIERS & 2) && valid && deg > kShortDeg && deg <= kWaveDeg);
+  const uint64_t very_long = __ballot((TIERS & 4) && valid && deg > kWaveDeg);
   WaveScope ws{lane};
   while (todo) {
     const int l = __ffsll((unsigned long long)todo) - 1;
@@ -360,6 +365,247 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_kernel(
   }
 }
 
+// ----------------------------------------------------------------------------
+// Edge-parallel walk.  A wave owns 64 consecutive rows and visits their edges 64 at a
+// time, one edge per lane, so that idx, out and mask are read and written as whole
+// contiguous lines whatever the degrees are.  Lane l also keeps the running state of
+// row l.  Per chunk of 64 positions:
+//   * the row of a lane's edge = the number of row ends at or before its position, by a
+//     six-step search through lane shuffles of the 64 ends;
+//   * a lane's segment = the lanes of the chunk that hold edges of the same row, known
+//     from that row's begin and end; a reduction over a segment is a scan bounded by the
+//     segment's first lane, its last lane then holds the total;
+//   * the lane that owns a row pulls the total from the last lane of the row's segment.
+// The order of every floating-point sum is fixed by the positions alone.  Rows of more
+// than kWaveDeg edges are stepped over (the walk jumps to their end) and left to the
+// whole block.
+struct SegmentWalk {
+  int64_t eb;                   // first edge of the wave
+  int total;                    // number of edges of its 64 rows
+  int begin_rel, end_rel;       // of the lane's own row, relative to eb
+  uint64_t long_mask;           // rows left to the block
+  int lane;
+
+  __device__ __forceinline__ void init(const int64_t* __restrict__ ptr, int64_t n_rows, int64_t first_row) {
+    lane = lane_id();
+    const int64_t r = first_row + lane;
+    const int64_t b = ptr[r < n_rows ? r : n_rows], e = ptr[r + 1 < n_rows ? r + 1 : n_rows];
+    eb = bcast_i64(b, 0);
+    const int64_t all = bcast_i64(e, CXG_WAVE - 1) - eb;
+    long_mask = __ballot(e - b > kWaveDeg);
+    if (all >= (int64_t)1 << 30) {           // positions are kept in 32 bits: leave such a wave to the block
+      long_mask = __ballot(e > b);
+      total = 0;
+      begin_rel = end_rel = 0;
+    } else {
+      total = (int)all;
+      begin_rel = (int)(b - eb);
+      end_rel = (int)(e - eb);
+    }
+  }
+  // One chunk at wave-uniform position `pos`.  Returns false (and moves pos to the end of
+  // the row) when the chunk starts inside a stepped-over row.  Otherwise: `row` = the
+  // lane's row (0..63), `act` = the lane holds an edge of a row handled here, `lo` / `hi`
+  // = the first / last lane of its segment; pos moves on by 64.
+  __device__ __forceinline__ bool chunk(int& pos, int& row, bool& act, int& lo, int& hi) const {
+    const int rel = pos + lane;
+    int cnt = 0;
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1)
+      if (__shfl(end_rel, cnt + step - 1, CXG_WAVE) <= rel) cnt += step;
+    row = cnt;
+    const int rb = __shfl(begin_rel, row, CXG_WAVE), re = __shfl(end_rel, row, CXG_WAVE);
+    const int row_first = uniform_i32(row);
+    if ((long_mask >> row_first) & 1) {
+      pos = uniform_i32(re);
+      return false;
+    }
+    act = rel < total && !((long_mask >> row) & 1);
+    const int l = rb - pos, h = re - pos;
+    lo = l > 0 ? l : 0;
+    hi = (h < CXG_WAVE ? h : CXG_WAVE) - 1;
+    pos += CXG_WAVE;
+    return true;
+  }
+  // first / last lane of the chunk at `at` holding the lane's OWN row; last = -1: none
+  __device__ __forceinline__ void own_segment(int at, int& first, int& last) const {
+    const int l = begin_rel - at, h = end_rel - at;
+    first = l > 0 ? l : 0;
+    last = (h < CXG_WAVE ? h : CXG_WAVE) - 1;
+    if (((long_mask >> lane) & 1) || h <= 0 || l >= CXG_WAVE || end_rel == begin_rel) last = -1;
+  }
+};
+
+// Inclusive scans over the lanes [lo, lane] of a segment, by data-parallel primitives:
+// four shifts inside each row of 16 lanes, then the last lane of row 0 / 2 to rows 1 / 3
+// and the last lane of row 1 to rows 2 and 3.  A lane takes a contribution only when
+// the lanes it stands for belong to its segment.
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <class Op, int N> __device__ __forceinline__ void segment_scan(float (&v)[N], int lane, int lo, Op op) {
+  const int in_row = lane & 15, row_start = lane & ~15;
+  const int lo_row = lo > row_start ? lo - row_start : 0;   // first lane of the segment inside this row of 16
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    float o;
+    o = dpp_f32<0x111>(v[i]); if (in_row - 1 >= lo_row) v[i] = op(v[i], o);   // row_shr:1
+    o = dpp_f32<0x112>(v[i]); if (in_row - 2 >= lo_row) v[i] = op(v[i], o);   // row_shr:2
+    o = dpp_f32<0x114>(v[i]); if (in_row - 4 >= lo_row) v[i] = op(v[i], o);   // row_shr:4
+    o = dpp_f32<0x118>(v[i]); if (in_row - 8 >= lo_row) v[i] = op(v[i], o);   // row_shr:8
+    o = dpp_f32<0x142>(v[i]); if ((lane & 16) && lo < row_start) v[i] = op(v[i], o);          // row_bcast:15
+    o = dpp_f32<0x143>(v[i]); if (lane >= 32 && lo < 32) v[i] = op(v[i], o);                 // row_bcast:31
+  }
+}
+struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+struct OpSum { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+// Rows left to the whole block: every wave announces its mask, then the block takes the
+// rows one at a time.  `rows_per_wave` consecutive rows per wave from `block_row0`.
+template <class CoopFn>
+__device__ __forceinline__ void block_rows(const int64_t* __restrict__ ptr, int64_t block_row0, int rows_per_wave,
+                                           uint64_t wave_mask, CoopFn coop_fn) {
+  __shared__ unsigned long long s_mask[kWavesPerBlock];
+  __shared__ float s_red[kWavesPerBlock * 2 * kMaxRed];
+  if (lane_id() == 0) s_mask[threadIdx.x >> 6] = wave_mask;
+  __syncthreads();
+  BlockScope bs{(int)threadIdx.x, s_red};
+  for (int w = 0; w < kWavesPerBlock; ++w) {
+    unsigned long long m = s_mask[w];
+    while (m) {
+      const int l = __ffsll(m) - 1;
+      m &= m - 1;
+      const int64_t rr = block_row0 + (int64_t)w * rows_per_wave + l;
+      coop_fn(bs, rr, (int64_t)ptr[rr], (int64_t)ptr[rr + 1]);
+    }
+  }
+}
+
+template <int H>
+__global__ __launch_bounds__(kBlock) void edge_softmax_fwd_walk_kernel(
+    const int64_t* __restrict__ ptr, const int64_t* __restrict__ idx,
+    const float* __restrict__ att_dst, const float* __restrict__ att_src, float* __restrict__ out,
+    uint8_t* __restrict__ mask, int64_t n_rows, float slope) {
+  const int lane = lane_id();
+  const int64_t block_row0 = (int64_t)blockIdx.x * kBlock;
+  const int64_t first_row = block_row0 + (int64_t)uniform_i32(threadIdx.x >> 6) * CXG_WAVE;
+  SegmentWalk w;
+  w.init(ptr, n_rows, first_row < n_rows ? first_row : n_rows);
+  float m[H], s[H];                          // of row first_row + lane
+#pragma unroll
+  for (int h = 0; h < H; ++h) { m[h] = kMaxInit; s[h] = 0.f; }
+  // sweep 1: logits parked in `out`, the rows' max and sum of exp
+  for (int pos = 0; pos < w.total;) {
+    int row, lo, hi, first, last;
+    bool act;
+    const int at = pos;
+    if (!w.chunk(pos, row, act, lo, hi)) continue;
+    const int rel = at + lane;
+    const int64_t k = w.eb + (rel < w.total ? rel : w.total - 1);
+    const int64_t r = first_row + row;
+    float a[H], d[H], t[H], mx[H], p[H];
+    load_f<H>(att_src + idx[k] * H, a);
+    load_f<H>(att_dst + (r < n_rows ? r : n_rows - 1) * H, d);
+#pragma unroll
+    for (int h = 0; h < H; ++h) mx[h] = t[h] = leaky(d[h] + a[h], slope);
+    if (act) store_f<H>(out + k * H, t);
+    segment_scan(mx, lane, lo, OpMax());
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      mx[h] = __shfl(mx[h], hi, CXG_WAVE);               // the segment's max on all its lanes
+      p[h] = __expf(t[h] - mx[h]);
+    }
+    segment_scan(p, lane, lo, OpSum());
+    w.own_segment(at, first, last);
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const float m2 = __shfl(mx[h], last < 0 ? 0 : last, CXG_WAVE);
+      const float s2 = __shfl(p[h], last < 0 ? 0 : last, CXG_WAVE);
+      if (last >= 0) merge_max_sum(m[h], s[h], m2, s2);
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < H; ++h) s[h] = 1.0f / s[h];
+  // sweep 2: the same lane revisits the same edges
+  for (int pos = 0; pos < w.total;) {
+    int row, lo, hi;
+    bool act;
+    const int at = pos;
+    if (!w.chunk(pos, row, act, lo, hi)) continue;
+    const int rel = at + lane;
+    const int64_t k = w.eb + (rel < w.total ? rel : w.total - 1);
+    float t[H], o[H];
+    bool mk[H];
+    load_f<H>(out + k * H, t);
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const float mr = __shfl(m[h], row, CXG_WAVE), sr = __shfl(s[h], row, CXG_WAVE);
+      o[h] = __expf(t[h] - mr) * sr;
+      mk[h] = t[h] > 0.f;
+    }
+    if (act) {
+      store_f<H>(out + k * H, o);
+      store_b<H>(mask + k * H, mk);
+    }
+  }
+
+  // rows of more than kWaveDeg edges: one at a time by the whole block
+  auto coop_fn = [&](auto sc, int64_t r, int64_t b, int64_t e) {
+    float d[H], bm[H], bsum[H];
+    load_f<H>(att_dst + r * H, d);
+#pragma unroll
+    for (int h = 0; h < H; ++h) { bm[h] = kMaxInit; bsum[h] = 0.f; }
+    for (int64_t k = b + sc.li; k < e; k += kU * sc.nl) {
+      int64_t kk[kU], src[kU];
+      float a[kU][H];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        kk[u] = k + u * sc.nl;
+        src[u] = idx[kk[u] < e ? kk[u] : e - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) load_f<H>(att_src + src[u] * H, a[u]);
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (kk[u] < e) {
+          float t[H];
+#pragma unroll
+          for (int h = 0; h < H; ++h) {
+            t[h] = leaky(d[h] + a[u][h], slope);
+            online_add(bm[h], bsum[h], t[h]);
+          }
+          store_f<H>(out + kk[u] * H, t);
+        }
+    }
+    sc.template combine_max_sum<H>(bm, bsum);
+#pragma unroll
+    for (int h = 0; h < H; ++h) bsum[h] = 1.0f / bsum[h];
+    for (int64_t k = b + sc.li; k < e; k += kU * sc.nl) {
+      int64_t kk[kU];
+      float t[kU][H];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        kk[u] = k + u * sc.nl;
+        load_f<H>(out + (kk[u] < e ? kk[u] : b + sc.li) * H, t[u]);   // written by this thread above
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (kk[u] < e) {
+          float o[H];
+          bool mk[H];
+#pragma unroll
+          for (int h = 0; h < H; ++h) {
+            o[h] = __expf(t[u][h] - bm[h]) * bsum[h];
+            mk[h] = t[u][h] > 0.f;
+          }
+          store_f<H>(out + kk[u] * H, o);
+          store_b<H>(mask + kk[u] * H, mk);
+        }
+    }
+  };
+  block_rows(ptr, block_row0, CXG_WAVE, w.long_mask, coop_fn);
+}
+
 template <int H>
 __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
     const int64_t* __restrict__ ptr, const float* __restrict__ out, const uint8_t* __restrict__ mask,
@@ -448,6 +694,142 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
   }
 }
 
+// Backward as an edge-parallel walk (see SegmentWalk): s = sum_row out*g, then
+// t = out*(g-s)*(mask ? 1 : slope) per edge and g_dst = sum_row t where the row has both
+// signs.
+template <int H>
+__global__ __launch_bounds__(kBlock) void edge_softmax_bwd_walk_kernel(
+    const int64_t* __restrict__ ptr, const float* __restrict__ out, const uint8_t* __restrict__ mask,
+    const float* __restrict__ grad, float* __restrict__ g_dst, float* __restrict__ t_edge,
+    int64_t n_rows, float slope) {
+  const int lane = lane_id();
+  const int64_t block_row0 = (int64_t)blockIdx.x * kBlock;
+  const int64_t first_row = block_row0 + (int64_t)uniform_i32(threadIdx.x >> 6) * CXG_WAVE;
+  SegmentWalk w;
+  w.init(ptr, n_rows, first_row < n_rows ? first_row : n_rows);
+  float s[H], dsum[H];                       // of row first_row + lane
+  unsigned seen = 0;                         // bit h: a positive logit seen, bit H + h: a negative one
+#pragma unroll
+  for (int h = 0; h < H; ++h) { s[h] = 0.f; dsum[h] = 0.f; }
+  // sweep 1: s = sum out*g
+  for (int pos = 0; pos < w.total;) {
+    int row, lo, hi, first, last;
+    bool act;
+    const int at = pos;
+    if (!w.chunk(pos, row, act, lo, hi)) continue;
+    const int rel = at + lane;
+    const int64_t k = w.eb + (rel < w.total ? rel : w.total - 1);
+    float o[H], g[H], v[H];
+    load_f<H>(out + k * H, o);
+    load_f<H>(grad + k * H, g);
+#pragma unroll
+    for (int h = 0; h < H; ++h) v[h] = o[h] * g[h];
+    segment_scan(v, lane, lo, OpSum());
+    w.own_segment(at, first, last);
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const float x = __shfl(v[h], last < 0 ? 0 : last, CXG_WAVE);
+      if (last >= 0) s[h] += x;
+    }
+  }
+  // sweep 2: per-edge values, their row sums, the signs seen in each row
+  for (int pos = 0; pos < w.total;) {
+    int row, lo, hi, first, last;
+    bool act;
+    const int at = pos;
+    if (!w.chunk(pos, row, act, lo, hi)) continue;
+    const int rel = at + lane;
+    const int64_t k = w.eb + (rel < w.total ? rel : w.total - 1);
+    float o[H], g[H], t[H];
+    bool mk[H];
+    load_f<H>(out + k * H, o);
+    load_f<H>(grad + k * H, g);
+    load_b<H>(mask + k * H, mk);
+    w.own_segment(at, first, last);
+    const uint64_t own = last < 0 ? 0ull : ((~0ull >> (CXG_WAVE - 1 - last)) & (~0ull << first));
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const float sr = __shfl(s[h], row, CXG_WAVE);
+      t[h] = o[h] * (g[h] - sr) * (mk[h] ? 1.0f : slope);
+      const uint64_t pos_m = __ballot(act && mk[h]), neg_m = __ballot(act && !mk[h]);
+      if (pos_m & own) seen |= 1u << h;
+      if (neg_m & own) seen |= 1u << (H + h);
+    }
+    if (act) store_f<H>(t_edge + k * H, t);
+    segment_scan(t, lane, lo, OpSum());
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const float x = __shfl(t[h], last < 0 ? 0 : last, CXG_WAVE);
+      if (last >= 0) dsum[h] += x;
+    }
+  }
+  if (first_row + lane < n_rows && !((w.long_mask >> lane) & 1)) {
+    float gd[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) gd[h] = ((seen >> h) & (seen >> (H + h)) & 1u) ? dsum[h] : 0.f;
+    store_f<H>(g_dst + (first_row + lane) * H, gd);
+  }
+
+  // rows of more than kWaveDeg edges: one at a time by the whole block
+  auto coop_fn = [&](auto sc, int64_t r, int64_t b, int64_t e) {
+    float bs[H], bd[H], flags[H];
+    int pos[H], neg[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) { bs[h] = 0.f; bd[h] = 0.f; pos[h] = 0; neg[h] = 0; }
+    for (int64_t k = b + sc.li; k < e; k += kU * sc.nl) {
+      int64_t kk[kU];
+      float o[kU][H], g[kU][H];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        kk[u] = k + u * sc.nl;
+        const int64_t c = kk[u] < e ? kk[u] : b + sc.li;
+        load_f<H>(out + c * H, o[u]);
+        load_f<H>(grad + c * H, g[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (kk[u] < e)
+#pragma unroll
+          for (int h = 0; h < H; ++h) bs[h] += o[u][h] * g[u][h];
+    }
+    sc.template sum_n<H>(bs);
+    for (int64_t k = b + sc.li; k < e; k += kU * sc.nl) {
+      int64_t kk[kU];
+      float o[kU][H], g[kU][H];
+      bool mk[kU][H];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        kk[u] = k + u * sc.nl;
+        const int64_t c = kk[u] < e ? kk[u] : b + sc.li;
+        load_f<H>(out + c * H, o[u]);
+        load_f<H>(grad + c * H, g[u]);
+        load_b<H>(mask + c * H, mk[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (kk[u] < e) {
+          float t[H];
+#pragma unroll
+          for (int h = 0; h < H; ++h) {
+            t[h] = o[u][h] * (g[u][h] - bs[h]);
+            if (!mk[u][h]) { t[h] *= slope; neg[h] = 1; } else { pos[h] = 1; }
+            bd[h] += t[h];
+          }
+          store_f<H>(t_edge + kk[u] * H, t);
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < H; ++h) flags[h] = (float)(pos[h] + 2 * neg[h]);   // 1: positive seen, 2: negative seen
+    sc.template sum_n<H>(bd);
+    sc.template or_n<H>(flags);
+    if (sc.leader()) {
+#pragma unroll
+      for (int h = 0; h < H; ++h) g_dst[r * H + h] = ((int)flags[h] == 3) ? bd[h] : 0.f;
+    }
+  };
+  block_rows(ptr, block_row0, CXG_WAVE, w.long_mask, coop_fn);
+}
+
 // out[r, 0..W) = sum_{k in row r} in[sel[k], 0..W)   (sel == nullptr: in[k]).
 template <int W>
 __global__ __launch_bounds__(kBlock) void narrow_gather_sum_kernel(
@@ -505,14 +887,16 @@ int cxg_edge_softmax_fwd_f32(const int64_t* ptr, const int64_t* idx, const float
   CXG_REQUIRE(idx && att_src && out && mask, CXG_ERR_ARG, "null idx/att_src/out/mask");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   dim3 grid = cxg::row_grid(n_dst), block(cxg::kBlock);
-#define CXG_FWD(HH)                                                                         \
-  hipLaunchKernelGGL(cxg::edge_softmax_fwd_kernel<HH>, grid, block, 0, st, ptr, idx, att_dst, \
-                     att_src, out, mask, n_dst, heads, slope)
+#define CXG_FWD(HH)                                                                              \
+  hipLaunchKernelGGL(cxg::edge_softmax_fwd_walk_kernel<HH>, grid, block, 0, st, ptr, idx, att_dst, \
+                     att_src, out, mask, n_dst, slope)
   if (heads == 1) CXG_FWD(1);
   else if (heads == 2) CXG_FWD(2);
   else if (heads == 4) CXG_FWD(4);
   else if (heads == 8) CXG_FWD(8);
-  else CXG_FWD(0);
+  else
+    hipLaunchKernelGGL(cxg::edge_softmax_fwd_kernel<0>, grid, block, 0, st, ptr, idx, att_dst, att_src,
+                       out, mask, n_dst, heads, slope);
 #undef CXG_FWD
   CXG_LAUNCH_CHECK("edge_softmax_fwd_kernel");
   return CXG_OK;
@@ -527,14 +911,16 @@ int cxg_edge_softmax_bwd_f32(const int64_t* ptr, const float* out, const uint8_t
   CXG_REQUIRE(out && mask && grad && t_edge, CXG_ERR_ARG, "null out/mask/grad/t_edge");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   dim3 grid = cxg::row_grid(n_dst), block(cxg::kBlock);
-#define CXG_BWD(HH)                                                                          \
-  hipLaunchKernelGGL(cxg::edge_softmax_bwd_kernel<HH>, grid, block, 0, st, ptr, out, mask, grad, \
-                     g_dst, t_edge, n_dst, heads, slope)
+#define CXG_BWD(HH)                                                                              \
+  hipLaunchKernelGGL(cxg::edge_softmax_bwd_walk_kernel<HH>, grid, block, 0, st, ptr, out, mask, grad, \
+                     g_dst, t_edge, n_dst, slope)
   if (heads == 1) CXG_BWD(1);
   else if (heads == 2) CXG_BWD(2);
   else if (heads == 4) CXG_BWD(4);
   else if (heads == 8) CXG_BWD(8);
-  else CXG_BWD(0);
+  else
+    hipLaunchKernelGGL(cxg::edge_softmax_bwd_kernel<0>, grid, block, 0, st, ptr, out, mask, grad, g_dst,
+                       t_edge, n_dst, heads, slope);
 #undef CXG_BWD
   CXG_LAUNCH_CHECK("edge_softmax_bwd_kernel");
   return CXG_OK;

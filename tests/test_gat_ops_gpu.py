@@ -116,6 +116,48 @@ def test_spmv_and_edge_value_degree(kind):
     assert np.array_equal(_np(ev), oracle.edge_value_degree(ptr.numpy(), n, E))
 
 
+@pytest.mark.parametrize("heads", [1, 2, 4, 8])
+def test_edge_softmax_degrees_at_the_step_boundaries(heads):
+    """Rows whose lengths sit on either side of what the kernels switch on: 64 edges (one
+    step of a wave), 512 edges (rows handed to the whole block), empty rows between them,
+    a long row first and last in a wave's 64 rows, and a row count that fills neither the
+    last wave nor the last block."""
+    import cxgnncomp_backend as B
+    pattern = [64, 0, 63, 1, 65, 512, 513, 0, 0, 128, 511, 2, 127, 129, 0, 700, 3, 64, 64, 1, 0, 0, 31, 33]
+    deg = torch.tensor((pattern * 15)[:331], dtype=torch.int64)
+    deg[0] = 900        # a row left to the block, first of its wave
+    deg[63] = 600       # ... and last of its wave
+    deg[64] = 0
+    deg[330] = 1500     # the very last row
+    n = deg.shape[0]
+    ptr = torch.zeros(n + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(deg, 0)
+    E = int(ptr[-1])
+    g0 = torch.Generator().manual_seed(5)
+    idx = torch.randint(0, n, (E,), generator=g0)
+    att_dst = torch.randn(n, heads, generator=g0) * 3
+    att_src = torch.randn(n, heads, generator=g0) * 3
+    slope = 0.2
+    ad = att_dst.cuda().requires_grad_(True)
+    asr = att_src.cuda().requires_grad_(True)
+    announce("edge_attention boundary degrees H=%d" % heads)
+    out = B.edge_attention(ptr=ptr.cuda(), idx=idx.cuda(), att_dst=ad, att_src=asr, num_edge=E, relu_l=slope)
+    g = torch.randn(E, heads, generator=g0)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    p, i = ptr.numpy(), idx.numpy()
+    ref, mask = oracle.edge_softmax_fwd(p, i, att_dst.numpy(), att_src.numpy(), E, slope)
+    assert_close(_np(out), ref, 2e-4, 1e-6, "softmax fwd")
+    gd, gs = oracle.edge_softmax_bwd(p, i, g.numpy(), mask, ref, n, n, slope)
+    assert_close(_np(ad.grad), gd, 1e-3, 2e-5, "grad att_dst")
+    assert_close(_np(asr.grad), gs, 1e-3, 2e-5, "grad att_src")
+    # a second run gives the same bits
+    ad2 = att_dst.cuda().requires_grad_(True)
+    out2 = B.edge_attention(ptr=ptr.cuda(), idx=idx.cuda(), att_dst=ad2, att_src=asr.detach(), num_edge=E, relu_l=slope)
+    out2.backward(g.cuda())
+    assert torch.equal(out, out2) and torch.equal(ad.grad, ad2.grad)
+
+
 @pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
 @pytest.mark.parametrize("width", [1, 2, 4, 8])
 @pytest.mark.parametrize("with_sel", [True, False])
