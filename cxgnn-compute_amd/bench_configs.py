@@ -158,10 +158,12 @@ def c2(iters):
     cxgnncomp.set_timers()                       # MyGCNConv brackets its phases with TimerOP, as upstream
     n = 169343
     x = torch.randn(n, 128, device="cuda")
-    for normalize in (False, True):
+    for normalize, own_bn in ((False, True), (True, True), (False, False)):
         convs = [cxgnncomp.MyGCNConv(128, 256, normalize).cuda(), cxgnncomp.MyGCNConv(256, 256, normalize).cuda(),
                  cxgnncomp.MyGCNConv(256, 40, normalize).cuda()]
-        bns = [torch.nn.BatchNorm1d(256).cuda(), torch.nn.BatchNorm1d(256).cuda()]
+        # between the layers, as GNN._between: the library's BatchNorm1d with the ReLU fused, or torch's own
+        bn_cls = cxgnncomp.BatchNorm1d if own_bn else torch.nn.BatchNorm1d
+        bns = [bn_cls(256).cuda(), bn_cls(256).cuda()]
         xg = x.clone().requires_grad_(True)
 
         def step():
@@ -170,10 +172,19 @@ def c2(iters):
             for li, conv in enumerate(convs):
                 h = conv(h, ptr, idx, n)
                 if li < 2:
-                    h = torch.relu(bns[li](h))
+                    h = bns[li](h, relu=True) if own_bn else torch.relu(bns[li](h))
             h.sum().backward()
-        report("c2", "3-layer GCN fwd+bwd, %s aggregation" % ("1/deg-weighted" if normalize else "sum"),
+        report("c2", "3-layer GCN fwd+bwd, %s aggregation%s" % ("1/deg-weighted" if normalize else "sum",
+                                                                "" if own_bn else ", torch.nn.BatchNorm1d + relu"),
                timeit(step, iters))
+    bn = cxgnncomp.BatchNorm1d(256).cuda()
+    hb = torch.randn(n, 256, device="cuda").requires_grad_(True)
+    gb = torch.randn(n, 256, device="cuda")
+    report("c2", "BatchNorm1d + ReLU forward, [169343, 256]", timeit(lambda: bn(hb, relu=True), iters), 2 * 3 * n * 256 * 4 // 3)
+    yb = bn(hb, relu=True)
+    report("c2", "BatchNorm1d + ReLU backward, [169343, 256]",
+           timeit(lambda: torch.autograd.grad(yb, hb, gb, retain_graph=True), iters), 5 * n * 256 * 4)
+    del bn, hb, gb, yb
     del convs, bns, xg
     # the remaining aggregation entry points of the backend on the same graph, F = 128
     import cxgnncomp_backend as B

@@ -20,5 +20,6 @@ from .schedule import (neighbor_grouping, neighbor_grouping_gpu, partition_2d, r
 from .batch import Batch, PyGBatch
 from .util import global_tuner
 from .graph_kernel import SpMMValOP
+from .batchnorm import BatchNorm1d
 from .model import GNN, SAGE, GCN, GIN, GAT, RGCN
 from . import synthetic  # noqa: F401

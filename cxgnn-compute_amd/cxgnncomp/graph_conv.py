@@ -186,7 +186,7 @@ class MySageConv(torch.nn.Module):
         else:
             out = linear(sage_mean_forward(x, ptr, idx, num_node), self.lin_l.weight, self.lin_l.bias)
         if self.root_weight:
-            out = out + linear(x[:num_node] if num_node != 0 else x, self.lin_r.weight)
+            out = linear(x[:num_node] if num_node != 0 else x, self.lin_r.weight, addend=out)
         return out
 
 
@@ -306,20 +306,24 @@ def _one_segment(m, device):
 
 
 class LinearOP(torch.autograd.Function):
-    """``F.linear(x, weight)`` whose weight gradient g^T x, a product with one very long
-    reduction axis (every node) and a small output, runs on the typed weight-gradient
-    kernel as a single segment; the library GEMM serves the forward pass, the input
-    gradient and the shapes that kernel does not take."""
+    """``F.linear(x, weight, bias) (+ addend)`` whose weight gradient g^T x, a product with
+    one very long reduction axis (every node) and a small output, runs on the typed
+    weight-gradient kernel as a single segment; the library GEMM serves the forward pass
+    (bias and addend go into its epilogue instead of separate element-wise passes), the
+    input gradient and the shapes that kernel does not take."""
 
     @staticmethod
-    def forward(ctx, x, weight):
+    def forward(ctx, x, weight, bias=None, addend=None):
         ctx.save_for_backward(x, weight)
-        return F.linear(x, weight)
+        if addend is None:
+            return F.linear(x, weight, bias)
+        out = torch.addmm(addend, x, weight.t())
+        return out if bias is None else out.add_(bias)
 
     @staticmethod
     def backward(ctx, g):
         x, weight = ctx.saved_tensors
-        gx = gw = None
+        gx = gw = gb = None
         if ctx.needs_input_grad[0]:
             gx = g @ weight
         if ctx.needs_input_grad[1]:
@@ -327,15 +331,18 @@ class LinearOP(torch.autograd.Function):
             m = x2.shape[0]
             full = _typed.typed_gemm_wgrad(x2, g2, _one_segment(m, x.device), m, 1) if m > 0 else None
             gw = full[0].t() if full is not None else g2.t() @ x2
-        return gx, gw
+        if ctx.needs_input_grad[2]:
+            gb = g.reshape(-1, g.shape[-1]).sum(dim=0)
+        return gx, gw, gb, (g if ctx.needs_input_grad[3] else None)
 
 
-def linear(x, weight, bias=None):
-    """``F.linear`` for the conv layers; CUDA tensors take LinearOP."""
-    if not x.is_cuda:
-        return F.linear(x, weight, bias)
-    out = LinearOP.apply(x, weight)
-    return out if bias is None else out + bias
+def linear(x, weight, bias=None, addend=None):
+    """``F.linear(x, weight, bias)``, plus ``addend`` where given, for the conv layers; CUDA
+    tensors take LinearOP."""
+    if not x.is_cuda or (addend is not None and x.dim() != 2):
+        out = F.linear(x, weight, bias)
+        return out if addend is None else addend + out
+    return LinearOP.apply(x, weight, bias, addend)
 
 
 class AttentionLogitsOP(torch.autograd.Function):
@@ -519,5 +526,5 @@ class MyGCNConv(torch.nn.Module):
         else:
             out = AggrOP.apply(out, ptr, idx, num_node)
         if not mm_before:
-            out = linear(out, self.lin.weight)
+            return linear(out, self.lin.weight, self.bias)
         return out + self.bias if self.bias is not None else out

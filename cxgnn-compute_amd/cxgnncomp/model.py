@@ -15,6 +15,7 @@ import torch.nn.functional as F
 
 import cxgnncomp_backend
 
+from .batchnorm import BatchNorm1d
 from .graph_conv import MyGATConv, MyGCNConv, MyGINConv, MyRGCNConv, MySageConv
 
 
@@ -36,7 +37,7 @@ class GNN(torch.nn.Module):
         self.graph_type = graph_type
         self.num_layer = num_layer
         self.dropout = dropout
-        self.bns = torch.nn.ModuleList(torch.nn.BatchNorm1d(hidden_channels) for _ in range(num_layer - 1))
+        self.bns = torch.nn.ModuleList(BatchNorm1d(hidden_channels) for _ in range(num_layer - 1))
         self.init_convs(**kwargs)
 
     def init_convs(self, **kwargs):
@@ -63,7 +64,7 @@ class GNN(torch.nn.Module):
         return batch.ptr.shape[0] - 1
 
     def _between(self, x, i):
-        x = F.relu(self.bns[i](x))
+        x = self.bns[i](x, relu=True)              # = F.relu(bn(x)), upstream model.py:66-67
         return F.dropout(x, p=self.dropout, training=self.training)
 
     def layer(self, conv, x, batch, i):

@@ -410,6 +410,75 @@ def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst):
     return grad_x, ga_src, ga_dst
 
 
+def _bn_vec(t, name, c, device):
+    if t is None:
+        return None
+    _req(t, name, torch.float32, 1)
+    if t.shape[0] != c or t.device != device:
+        raise ValueError("%s must hold %d floats on %s" % (name, c, device))
+    return t
+
+
+def batchnorm_stats(x, eps):
+    """Column statistics of x [n, c]: (mean, 1/sqrt(biased var + eps), unbiased var)."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 2)
+    n, c = x.shape
+    if n < 1 or c < 1:
+        raise ValueError("batch statistics need at least one row and one column, got %s" % (tuple(x.shape),))
+    mean = torch.empty(c, dtype=torch.float32, device=x.device)
+    invstd = torch.empty_like(mean)
+    var_unbiased = torch.empty_like(mean)
+    ws = _workspace(lib.cxg_batchnorm_workspace_bytes(n, c), x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_batchnorm_stats_f32(_lib.ptr(x), n, c, x.stride(0), float(eps), mean.data_ptr(),
+                                         invstd.data_ptr(), var_unbiased.data_ptr(), ws.data_ptr(), ws.numel(),
+                                         _lib.current_stream(x.device))
+    _lib.check(st)
+    return mean, invstd, var_unbiased
+
+
+def batchnorm_apply(x, mean, invstd, gamma=None, beta=None, relu=False):
+    """(x - mean) * invstd * gamma + beta per column of x [n, c], then max(., 0) if relu."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 2)
+    n, c = x.shape
+    if c < 1:
+        raise ValueError("x has no columns")
+    mean, invstd = _bn_vec(mean, "mean", c, x.device), _bn_vec(invstd, "invstd", c, x.device)
+    gamma, beta = _bn_vec(gamma, "gamma", c, x.device), _bn_vec(beta, "beta", c, x.device)
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_batchnorm_apply_f32(_lib.ptr(x), n, c, x.stride(0), mean.data_ptr(), invstd.data_ptr(),
+                                         _lib.ptr(gamma), _lib.ptr(beta), _lib.ptr(y), y.stride(0), int(bool(relu)),
+                                         _lib.current_stream(x.device))
+    _lib.check(st)
+    return y
+
+
+def batchnorm_bwd(x, dy, mean, invstd, gamma=None, beta=None, relu=False):
+    """Gradients of batchnorm_apply over batch statistics: (dx, dgamma, dbeta)."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 2)
+    _req(dy, "dy", torch.float32, 2)
+    n, c = x.shape
+    if tuple(dy.shape) != (n, c) or n < 1 or c < 1:
+        raise ValueError("dy %s does not fit x %s" % (tuple(dy.shape), tuple(x.shape)))
+    mean, invstd = _bn_vec(mean, "mean", c, x.device), _bn_vec(invstd, "invstd", c, x.device)
+    gamma, beta = _bn_vec(gamma, "gamma", c, x.device), _bn_vec(beta, "beta", c, x.device)
+    dx = torch.empty_like(x)
+    dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
+    dbeta = torch.empty_like(dgamma)
+    ws = _workspace(lib.cxg_batchnorm_workspace_bytes(n, c), x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_batchnorm_bwd_f32(_lib.ptr(x), _lib.ptr(dy), n, c, x.stride(0), dy.stride(0), mean.data_ptr(),
+                                       invstd.data_ptr(), _lib.ptr(gamma), _lib.ptr(beta), int(bool(relu)),
+                                       _lib.ptr(dx), dx.stride(0), dgamma.data_ptr(), dbeta.data_ptr(),
+                                       ws.data_ptr(), ws.numel(), _lib.current_stream(x.device))
+    _lib.check(st)
+    return dx, dgamma, dbeta
+
+
 def csr_row_ids32(ptr, n_rows, n_edges):
     """int32 row id of every edge position (the edge-parallel kernels' row lookup)."""
     lib = _lib.load()

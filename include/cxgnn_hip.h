@@ -325,6 +325,31 @@ int cxg_attention_logits_bwd_f32(const float* x, const float* att_src, const flo
                                  float* grad_att_src, float* grad_att_dst, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
+/* Batch normalisation over the rows of x[n, c] (row stride ldx), the layer the upstream
+ * models put between two convolutions (torch.nn.BatchNorm1d, cxgnncomp/model.py:28 and
+ * its use followed by F.relu in GNN.forward_cxg, cxgnncomp/model.py:66-67).  Three calls:
+ *   stats : mean[c], invstd[c] = 1/sqrt(biased variance + eps), var_unbiased[c] (may be
+ *           NULL; the value the running variance is updated with); needs n >= 1;
+ *   apply : y = (x - mean) * invstd * gamma + beta, then max(., 0) when relu != 0
+ *           (gamma / beta may be NULL: 1 / 0); also serves evaluation mode with the
+ *           running statistics;
+ *   bwd   : dbeta[c] = sum dy, dgamma[c] = sum dy * xhat, dx = gamma * invstd *
+ *           (dy - dbeta/n - xhat * dgamma/n); with relu != 0, dy counts only where the
+ *           forward output was positive (recomputed from x, gamma, beta).
+ * workspace: cxg_batchnorm_workspace_bytes(n, c) bytes of device memory (per-block
+ * partial statistics).  Results do not depend on the run (fixed merge order). */
+size_t cxg_batchnorm_workspace_bytes(int64_t n, int c);
+int cxg_batchnorm_stats_f32(const float* x, int64_t n, int c, int64_t ldx, float eps, float* mean,
+                            float* invstd, float* var_unbiased, void* workspace,
+                            size_t workspace_bytes, void* stream);
+int cxg_batchnorm_apply_f32(const float* x, int64_t n, int c, int64_t ldx, const float* mean,
+                            const float* invstd, const float* gamma, const float* beta, float* y,
+                            int64_t ldy, int relu, void* stream);
+int cxg_batchnorm_bwd_f32(const float* x, const float* dy, int64_t n, int c, int64_t ldx,
+                          int64_t lddy, const float* mean, const float* invstd, const float* gamma,
+                          const float* beta, int relu, float* dx, int64_t lddx, float* dgamma,
+                          float* dbeta, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Index work (bit-exact)                                                     */
 /* ------------------------------------------------------------------------- */

@@ -224,3 +224,46 @@ def topo_sort(ptr, idx, degree):
         elif not q:
             break
     return out, len(out)
+
+
+def batchnorm_fwd(x, gamma, beta, eps, relu=False):
+    """torch.nn.BatchNorm1d in training mode as the reference's models use it
+    (cxgnncomp/model.py:28, :66-67, there followed by F.relu): per column,
+    y = (x - mean) / sqrt(biased var + eps) * gamma + beta, in float64.  Returns
+    (y, mean, biased var, unbiased var); the running statistics are updated with the mean
+    and the unbiased variance."""
+    x = np.asarray(x, dtype=np.float64)
+    n = x.shape[0]
+    mean = x.mean(axis=0)
+    var = ((x - mean) ** 2).mean(axis=0)
+    y = (x - mean) / np.sqrt(var + eps)
+    if gamma is not None:
+        y = y * np.asarray(gamma, dtype=np.float64)
+    if beta is not None:
+        y = y + np.asarray(beta, dtype=np.float64)
+    if relu:
+        y = np.maximum(y, 0.0)
+    return y, mean, var, var * n / max(n - 1, 1)
+
+
+def batchnorm_bwd(x, dy, gamma, beta, eps, relu=False, active=None):
+    """Gradient of batchnorm_fwd (batch statistics are functions of x): with
+    xhat = (x - mean) / sqrt(var + eps), dbeta = sum dy, dgamma = sum dy * xhat,
+    dx = gamma / sqrt(var + eps) * (dy - mean(dy) - xhat * mean(dy * xhat)); with relu,
+    dy is first zeroed where the forward output is not positive (``active``, if given, says
+    where it is positive instead of the recomputation: for outputs within rounding of 0).
+    float64."""
+    x = np.asarray(x, dtype=np.float64)
+    dy = np.asarray(dy, dtype=np.float64)
+    mean = x.mean(axis=0)
+    var = ((x - mean) ** 2).mean(axis=0)
+    invstd = 1.0 / np.sqrt(var + eps)
+    xhat = (x - mean) * invstd
+    g = np.ones(x.shape[1]) if gamma is None else np.asarray(gamma, dtype=np.float64)
+    if relu:
+        y = xhat * g + (0.0 if beta is None else np.asarray(beta, dtype=np.float64))
+        dy = np.where((y > 0) if active is None else active, dy, 0.0)
+    dbeta = dy.sum(axis=0)
+    dgamma = (dy * xhat).sum(axis=0)
+    dx = g * invstd * (dy - dy.mean(axis=0) - xhat * (dy * xhat).mean(axis=0))
+    return dx, dgamma, dbeta

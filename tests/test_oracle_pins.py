@@ -469,3 +469,37 @@ def test_topo_sort_restatement_on_dags_and_hand_cases():
     assert pyref.topo_sort([0, 1, 2, 3], [1, 2, 0], [1, 1, 1]) == ([0, 1, 2], 3)
     # counters the release rule cannot start from (running minimum starts at n)
     assert pyref.topo_sort([0, 1, 2], [1, 0], [2, 3]) == ([], 0)
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("affine", [True, False])
+def test_batchnorm_restatement_matches_torch_and_autograd(relu, affine):
+    """pyref.batchnorm_fwd / batchnorm_bwd against torch's own batch_norm (a library
+    routine, float64 on the CPU) and its autograd, plus the closed-form properties: the
+    normalised columns have zero mean and variance var/(var+eps), dx sums to zero per column."""
+    rng = np.random.default_rng(3)
+    n, c, eps = 257, 12, 1e-5
+    x = rng.normal(size=(n, c)) * rng.uniform(0.1, 30, size=c) + rng.normal(size=c) * 50
+    dy = rng.normal(size=(n, c))
+    gamma = rng.uniform(0.5, 2, size=c) if affine else None
+    beta = rng.normal(size=c) if affine else None
+    xt = torch.tensor(x, requires_grad=True)
+    gt = torch.tensor(gamma, requires_grad=True) if affine else None
+    bt = torch.tensor(beta, requires_grad=True) if affine else None
+    rm, rv = torch.zeros(c, dtype=torch.float64), torch.ones(c, dtype=torch.float64)
+    yt = torch.nn.functional.batch_norm(xt, rm, rv, gt, bt, training=True, momentum=1.0, eps=eps)
+    if relu:
+        yt = torch.relu(yt)
+    yt.backward(torch.tensor(dy))
+    y, mean, var, var_unbiased = pyref.batchnorm_fwd(x, gamma, beta, eps, relu)
+    assert np.allclose(y, yt.detach().numpy(), rtol=1e-10, atol=1e-10)
+    assert np.allclose(mean, rm.numpy(), rtol=1e-12) and np.allclose(var_unbiased, rv.numpy(), rtol=1e-12)
+    dx, dgamma, dbeta = pyref.batchnorm_bwd(x, dy, gamma, beta, eps, relu)
+    assert np.allclose(dx, xt.grad.numpy(), rtol=1e-8, atol=1e-10)
+    if affine:
+        assert np.allclose(dgamma, gt.grad.numpy(), rtol=1e-9, atol=1e-10)
+        assert np.allclose(dbeta, bt.grad.numpy(), rtol=1e-9, atol=1e-10)
+    assert np.allclose(dx.sum(axis=0), 0, atol=1e-9)
+    if not relu and not affine:
+        assert np.allclose(y.mean(axis=0), 0, atol=1e-12)
+        assert np.allclose(y.var(axis=0), var / (var + eps), rtol=1e-12)
