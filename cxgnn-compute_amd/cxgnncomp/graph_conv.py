@@ -13,7 +13,7 @@ import torch.nn.functional as F
 from torch.nn import Parameter
 
 import cxgnncomp_backend
-from cxgnncomp_backend import _typed
+from cxgnncomp_backend import _ops, _typed
 from cxgnncomp_backend import (aggr_rel, aggr_rgcn_direct_func, edge_attention, gather,
                                sage_mean_forward, sage_sum_forward, sage_sum_forward_edge_value,
                                selective_aggr, selective_aggr_bwd)
@@ -181,6 +181,9 @@ class MySageConv(torch.nn.Module):
             self.lin_r.reset_parameters()
 
     def forward(self, x, ptr, idx, num_node):
+        if x.is_cuda and x.dim() == 2:
+            return SageLayerOP.apply(x, self.lin_l.weight, self.lin_l.bias,
+                                     self.lin_r.weight if self.root_weight else None, ptr, idx, num_node)
         if self.in_channels > self.hidden_channels:
             out = sage_mean_forward(linear(x, self.lin_l.weight, self.lin_l.bias), ptr, idx, num_node)
         else:
@@ -305,6 +308,72 @@ def _one_segment(m, device):
     return seg
 
 
+def _weight_grad(x, g):
+    """g^T x, the weight gradient of ``F.linear(x, w)``: one very long reduction axis, on the
+    typed weight-gradient kernel as a single segment."""
+    x2, g2 = x.reshape(-1, x.shape[-1]).contiguous(), g.reshape(-1, g.shape[-1]).contiguous()
+    m = x2.shape[0]
+    full = _typed.typed_gemm_wgrad(x2, g2, _one_segment(m, x.device), m, 1) if m > 0 else None
+    return full[0].t() if full is not None else g2.t() @ x2      # shapes that kernel does not take
+
+
+class SageLayerOP(torch.autograd.Function):
+    """``MySageConv.forward`` on CUDA tensors as one autograd node: mean aggregation and
+    ``lin_l`` in the cheaper order, plus the root term ``lin_r(x[:num_node])`` added by the
+    GEMM in place.  The backward pass writes the input gradient once (the transposed
+    aggregation fills every source row, the root term is added in place on the first
+    rows) instead of autograd's zero-padded slice gradient and a full-size add."""
+
+    @staticmethod
+    def forward(ctx, x, w_l, b_l, w_r, ptr, idx, num_node):
+        n = int(num_node) if int(num_node) != 0 else ptr.shape[0] - 1
+        x = x.contiguous()
+        mm_first = w_l.shape[1] > w_l.shape[0]
+        aggr = None
+        if mm_first:
+            out = _ops.spmm(ptr, idx, F.linear(x, w_l, b_l), n, mean=True)
+        else:
+            aggr = _ops.spmm(ptr, idx, x, n, mean=True)
+            out = F.linear(aggr, w_l, b_l)
+        if w_r is not None:
+            out.addmm_(x[:n], w_r.t())
+        ctx.n, ctx.mm_first = n, mm_first
+        ctx.save_for_backward(x, w_l, w_r, ptr, idx, aggr)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w_l, w_r, ptr, idx, aggr = ctx.saved_tensors
+        n, n_src = ctx.n, x.shape[0]
+        g = g.contiguous()
+        need_x, need_wl, need_bl, need_wr = ctx.needs_input_grad[:4]
+        gx = gw_l = gb_l = gw_r = None
+        if need_x or ctx.mm_first:
+            tg = _ops.transposed(ptr, idx, n, n_src)
+            inv = _ops.inv_degree_transposed(tg, ptr, n)
+        if ctx.mm_first:
+            g_t = _ops.spmm(tg.ptr_t, tg.idx_t, g, n_src, val=inv)
+            if need_wl:
+                gw_l = _weight_grad(x, g_t)
+            if need_bl:
+                gb_l = g_t.sum(dim=0)
+            if need_x:
+                gx = g_t @ w_l
+        else:
+            if need_wl:
+                gw_l = _weight_grad(aggr, g)
+            if need_bl:
+                gb_l = g.sum(dim=0)
+            if need_x:
+                gx = _ops.spmm(tg.ptr_t, tg.idx_t, g @ w_l, n_src, val=inv)
+        if w_r is not None:
+            if need_wr:
+                gw_r = _weight_grad(x[:n], g)
+            if need_x:
+                gx[:n].addmm_(g, w_r)
+        return gx, gw_l, gb_l, gw_r, None, None, None
+
+
 class LinearOP(torch.autograd.Function):
     """``F.linear(x, weight, bias) (+ addend)`` whose weight gradient g^T x, a product with
     one very long reduction axis (every node) and a small output, runs on the typed
@@ -327,10 +396,7 @@ class LinearOP(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             gx = g @ weight
         if ctx.needs_input_grad[1]:
-            x2, g2 = x.reshape(-1, x.shape[-1]).contiguous(), g.reshape(-1, g.shape[-1]).contiguous()
-            m = x2.shape[0]
-            full = _typed.typed_gemm_wgrad(x2, g2, _one_segment(m, x.device), m, 1) if m > 0 else None
-            gw = full[0].t() if full is not None else g2.t() @ x2
+            gw = _weight_grad(x, g)
         if ctx.needs_input_grad[2]:
             gb = g.reshape(-1, g.shape[-1]).sum(dim=0)
         return gx, gw, gb, (g if ctx.needs_input_grad[3] else None)

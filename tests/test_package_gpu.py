@@ -295,12 +295,17 @@ def test_conv_layers_forward_backward():
         out.sum().backward()
         torch.cuda.synchronize()
         x64 = x.double().requires_grad_(True)
-        params = {k: v.detach().double().cpu() for k, v in layer.named_parameters()}
+        params = {k: v.detach().double().cpu().requires_grad_(True) for k, v in layer.named_parameters()}
         ref = ref_fn(x64, params)
         ref.sum().backward()
         assert_close(_np(out), ref.detach().numpy(), 2e-4, 2e-5, name + " fwd")
         sc = max(1.0, float(x64.grad.abs().max()))
         assert_close(_np(xg.grad) / sc, x64.grad.numpy() / sc, 2e-4, 2e-5, name + " grad x")
+        for k, v in layer.named_parameters():
+            if params[k].grad is None:
+                continue
+            sc = max(1.0, float(params[k].grad.abs().max()))
+            assert_close(_np(v.grad) / sc, params[k].grad.numpy() / sc, 2e-4, 2e-5, name + " grad " + k)
 
     inv = torch.where(deg > 0, 1.0 / deg.clamp(min=1), torch.zeros_like(deg))
     check(cxgnncomp.MyGCNConv(32, 48), lambda t, P: agg(t) @ P["lin.weight"].T + P["bias"], (pc, ic, n), "GCN sum")
@@ -309,6 +314,11 @@ def test_conv_layers_forward_backward():
     check(cxgnncomp.MySageConv(32, 48),
           lambda t, P: (agg(t) * inv[:, None]) @ P["lin_l.weight"].T + P["lin_l.bias"] + t @ P["lin_r.weight"].T,
           (pc, ic, n), "SAGE mean")
+    check(cxgnncomp.MySageConv(32, 16),
+          lambda t, P: agg(t @ P["lin_l.weight"].T + P["lin_l.bias"]) * inv[:, None] + t @ P["lin_r.weight"].T,
+          (pc, ic, n), "SAGE mean, linear first")
+    check(cxgnncomp.MySageConv(32, 40, root_weight=False, bias=False),
+          lambda t, P: (agg(t) * inv[:, None]) @ P["lin_l.weight"].T, (pc, ic, n), "SAGE mean, no root, no bias")
     check(cxgnncomp.MyGINConv(32, 24),
           lambda t, P: (agg(t) * inv[:, None] + (1 + P["eps"]) * t) @ P["nn.weight"].T, (pc, ic, n), "GIN")
 
@@ -417,3 +427,53 @@ def test_linear_op_matches_torch(k, n, rows):
         assert got.shape == want.shape
         scale = max(1.0, float(want.abs().max()))
         assert_close(got.cpu().numpy() / scale, want.numpy() / scale, 1e-4, 2e-5, name)
+
+
+@pytest.mark.parametrize("widths", [(24, 40), (40, 24)])
+def test_sage_layer_on_a_row_prefix(widths):
+    """MySageConv on a sampled-batch layer: num_node destination rows over more source rows
+    (the root term reads x[:num_node]); output, input gradient and every parameter gradient
+    against the float64 composition, and a frozen input (no input gradient asked for)."""
+    import cxgnncomp
+    torch.manual_seed(4)
+    n_src, n_dst, fin, fout = 900, 300, widths[0], widths[1]
+    deg = torch.randint(0, 9, (n_dst,))
+    deg[5] = 0
+    ptr = torch.zeros(n_dst + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(deg, 0)
+    E = int(ptr[-1])
+    idx = torch.randint(0, n_src, (E,))
+    dst = torch.repeat_interleave(torch.arange(n_dst), deg)
+    x = torch.randn(n_src, fin)
+    layer = cxgnncomp.MySageConv(fin, fout).cuda()
+    xg = x.cuda().requires_grad_(True)
+    announce("SageLayerOP prefix rows %s" % (widths,))
+    out = layer(xg, ptr.cuda(), idx.cuda(), n_dst)
+    w = torch.randn(n_dst, fout)
+    (out * w.cuda()).sum().backward()
+    torch.cuda.synchronize()
+    P = {k: v.detach().double().cpu().requires_grad_(True) for k, v in layer.named_parameters()}
+    x64 = x.double().requires_grad_(True)
+    inv = torch.where(deg > 0, 1.0 / deg.clamp(min=1).double(), torch.zeros(n_dst, dtype=torch.float64))
+
+    def mean_aggr(t):
+        return torch.zeros(n_dst, t.shape[1], dtype=t.dtype).index_add_(0, dst, t[idx]) * inv[:, None]
+    if fin > fout:
+        ref = mean_aggr(x64 @ P["lin_l.weight"].T + P["lin_l.bias"])
+    else:
+        ref = mean_aggr(x64) @ P["lin_l.weight"].T + P["lin_l.bias"]
+    ref = ref + x64[:n_dst] @ P["lin_r.weight"].T
+    (ref * w.double()).sum().backward()
+    assert_close(_np(out), ref.detach().numpy(), 2e-4, 2e-5, "fwd")
+    assert_close(_np(xg.grad), x64.grad.numpy(), 2e-4, 2e-5, "grad x")
+    for k, v in layer.named_parameters():
+        sc = max(1.0, float(P[k].grad.abs().max()))
+        assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "grad " + k)
+    # frozen input: parameter gradients only
+    layer.zero_grad()
+    out2 = layer(x.cuda(), ptr.cuda(), idx.cuda(), n_dst)
+    (out2 * w.cuda()).sum().backward()
+    assert torch.equal(out2, out)
+    for k, v in layer.named_parameters():
+        sc = max(1.0, float(P[k].grad.abs().max()))
+        assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "frozen input, grad " + k)
