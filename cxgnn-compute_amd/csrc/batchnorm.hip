@@ -14,7 +14,8 @@
 // first row, so that a column mean far from zero costs no accuracy), merged pairwise (Chan) over the
 // TY row offsets in LDS, written as one partial row per block and merged again, in block
 // order, by a second kernel (one wave per column).  Grid sizes depend on the shape only,
-// so results are reproducible bit for bit.
+// so results are reproducible bit for bit.  The same layout serves the plain column sum
+// (the bias gradient of a linear layer, g.sum(0)).
 #include "cxg_common.hpp"
 
 namespace cxg {
@@ -295,6 +296,53 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_dx_kernel(
   }
 }
 
+// partial[b][col] = sum of x[r, col] over the rows of block b (the bias gradient of a linear layer)
+template <int V>
+__global__ __launch_bounds__(kBnThreads) void column_sum_partial_kernel(
+    const float* __restrict__ x, int64_t n, int c, int64_t ldx, int tx_shift, int64_t rows_per_block,
+    float* __restrict__ partial) {
+  __shared__ float s_a[kBnThreads * V];
+  const BnBlock b(n, c, V, tx_shift, rows_per_block);
+  float sa[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) sa[i] = 0.f;
+  if (b.live) {
+    for (int64_t r = b.r_begin + b.ty_i; r < b.r_end; r += b.ty) {
+      float v[V];
+      load_v<V>(x + r * ldx + (int64_t)b.slot * V, v);
+#pragma unroll
+      for (int i = 0; i < V; ++i) sa[i] += v[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < V; ++i) s_a[threadIdx.x * V + i] = sa[i];
+  __syncthreads();
+  if (b.ty_i == 0 && b.live) {
+    const int tx = 1 << tx_shift;
+    for (int j = 1; j < b.ty; ++j) {
+      const int t = j * tx + b.tx_i;
+#pragma unroll
+      for (int i = 0; i < V; ++i) sa[i] += s_a[t * V + i];
+    }
+    store_v<V>(partial + (size_t)blockIdx.x * c + (size_t)b.slot * V, sa);
+  }
+}
+
+__global__ __launch_bounds__(kBnThreads) void column_sum_final_kernel(
+    const float* __restrict__ partial, int row_blocks, int c, float* __restrict__ out) {
+  const int lane = lane_id();
+  const int col = blockIdx.x * (kBnThreads / CXG_WAVE) + (threadIdx.x >> 6);
+  if (col >= c) return;
+  const int per = (row_blocks + CXG_WAVE - 1) / CXG_WAVE;
+  float a = 0.f;
+  for (int b = lane * per; b < (lane + 1) * per && b < row_blocks; ++b) a += partial[(size_t)b * c + col];
+  for (int s = 1; s < CXG_WAVE; s <<= 1) {
+    const float a2 = __shfl_down(a, s, CXG_WAVE);
+    if ((lane & (2 * s - 1)) == 0) a += a2;
+  }
+  if (lane == 0) out[col] = a;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
@@ -390,6 +438,37 @@ int cxg_batchnorm_bwd_f32(const float* x, const float* dy, int64_t n, int c, int
   else { if (relu) CXG_BN_DX(1, true); else CXG_BN_DX(1, false); }
 #undef CXG_BN_DX
   CXG_LAUNCH_CHECK("bn_bwd_dx_kernel");
+  return CXG_OK;
+}
+
+int cxg_column_sum_f32(const float* x, int64_t n, int c, int64_t ldx, float* out, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  CXG_REQUIRE(n >= 0 && c >= 1 && ldx >= c, CXG_ERR_ARG, "column_sum: bad n/c/ldx");
+  CXG_REQUIRE(out, CXG_ERR_ARG, "column_sum: null out");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (n == 0) {
+    CXG_HIP_CHECK(hipMemsetAsync(out, 0, (size_t)c * sizeof(float), st));
+    return CXG_OK;
+  }
+  CXG_REQUIRE(x && workspace, CXG_ERR_ARG, "column_sum: null x/workspace");
+  CXG_REQUIRE(workspace_bytes >= cxg_batchnorm_workspace_bytes(n, c), CXG_ERR_ARG,
+              "column_sum: workspace of %zu bytes, %zu needed", workspace_bytes,
+              cxg_batchnorm_workspace_bytes(n, c));
+  const bool v4 = c % 4 == 0 && ldx % 4 == 0 && cxg::aligned16(x);
+  const cxg::BnGeom g = cxg::bn_geometry(n, c, v4);
+  float* partial = static_cast<float*>(workspace);
+  dim3 grid(g.row_blocks, g.col_tiles), block(cxg::kBnThreads);
+  if (v4)
+    hipLaunchKernelGGL(cxg::column_sum_partial_kernel<4>, grid, block, 0, st, x, n, c, ldx, g.tx_shift,
+                       g.rows_per_block, partial);
+  else
+    hipLaunchKernelGGL(cxg::column_sum_partial_kernel<1>, grid, block, 0, st, x, n, c, ldx, g.tx_shift,
+                       g.rows_per_block, partial);
+  CXG_LAUNCH_CHECK("column_sum_partial_kernel");
+  const int waves = cxg::kBnThreads / CXG_WAVE;
+  hipLaunchKernelGGL(cxg::column_sum_final_kernel, dim3((c + waves - 1) / waves), block, 0, st, partial,
+                     g.row_blocks, c, out);
+  CXG_LAUNCH_CHECK("column_sum_final_kernel");
   return CXG_OK;
 }
 

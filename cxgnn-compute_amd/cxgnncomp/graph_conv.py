@@ -356,14 +356,14 @@ class SageLayerOP(torch.autograd.Function):
             if need_wl:
                 gw_l = _weight_grad(x, g_t)
             if need_bl:
-                gb_l = g_t.sum(dim=0)
+                gb_l = _ops.column_sum(g_t)
             if need_x:
                 gx = g_t @ w_l
         else:
             if need_wl:
                 gw_l = _weight_grad(aggr, g)
             if need_bl:
-                gb_l = g.sum(dim=0)
+                gb_l = _ops.column_sum(g)
             if need_x:
                 gx = _ops.spmm(tg.ptr_t, tg.idx_t, g @ w_l, n_src, val=inv)
         if w_r is not None:
@@ -398,7 +398,7 @@ class LinearOP(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             gw = _weight_grad(x, g)
         if ctx.needs_input_grad[2]:
-            gb = g.reshape(-1, g.shape[-1]).sum(dim=0)
+            gb = _ops.column_sum(g.reshape(-1, g.shape[-1]).contiguous())
         return gx, gw, gb, (g if ctx.needs_input_grad[3] else None)
 
 

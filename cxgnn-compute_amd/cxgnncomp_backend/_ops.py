@@ -479,6 +479,22 @@ def batchnorm_bwd(x, dy, mean, invstd, gamma=None, beta=None, relu=False):
     return dx, dgamma, dbeta
 
 
+def column_sum(x):
+    """x.sum(0) of a 2-D fp32 tensor, in a fixed order (bias gradients)."""
+    lib = _lib.load()
+    _req(x, "x", torch.float32, 2)
+    n, c = x.shape
+    if c < 1:
+        raise ValueError("x has no columns")
+    out = torch.empty(c, dtype=torch.float32, device=x.device)
+    ws = _workspace(lib.cxg_batchnorm_workspace_bytes(n, c), x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_column_sum_f32(_lib.ptr(x), n, c, x.stride(0), out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                    _lib.current_stream(x.device))
+    _lib.check(st)
+    return out
+
+
 def csr_row_ids32(ptr, n_rows, n_edges):
     """int32 row id of every edge position (the edge-parallel kernels' row lookup)."""
     lib = _lib.load()

@@ -350,6 +350,13 @@ int cxg_batchnorm_bwd_f32(const float* x, const float* dy, int64_t n, int c, int
                           const float* beta, int relu, float* dx, int64_t lddx, float* dgamma,
                           float* dbeta, void* workspace, size_t workspace_bytes, void* stream);
 
+/* out[c] = sum over the n rows of x[n, c] (row stride ldx): the bias gradient of the
+ * layers' linear maps (autograd's g.sum(0) for lin_l.bias of MySageConv,
+ * cxgnncomp/graph_conv.py:130 and :142-152, and the bias of MyGCNConv, :622-623).  workspace:
+ * cxg_batchnorm_workspace_bytes(n, c) bytes.  Fixed summation order. */
+int cxg_column_sum_f32(const float* x, int64_t n, int c, int64_t ldx, float* out, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Index work (bit-exact)                                                     */
 /* ------------------------------------------------------------------------- */

@@ -124,3 +124,18 @@ def test_batchnorm_module_matches_torch_module(relu):
     assert torch.allclose(ours(x3), torch.nn.functional.batch_norm(x3, None, None, ours.weight, ours.bias, True),
                           rtol=1e-4, atol=1e-5)
     assert ours.state_dict().keys() == ref.state_dict().keys()
+
+
+@pytest.mark.parametrize("shape", SHAPES + [(0, 12)])
+def test_column_sum_against_float64(shape):
+    from cxgnncomp_backend import _ops
+    n, c = shape
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(n, c, generator=g) * 3 + 0.5
+    announce("column_sum n=%d c=%d" % (n, c))
+    xc = x.cuda()
+    got = _ops.column_sum(xc)
+    want = x.double().sum(dim=0).numpy()
+    scale = np.sqrt(max(n, 1)) * 3
+    assert np.all(np.abs(got.cpu().numpy() - want) <= 1e-4 * np.abs(want) + 1e-5 * scale)
+    assert torch.equal(got, _ops.column_sum(xc))
