@@ -128,7 +128,7 @@ __global__ void att_logits_fwd_generic_kernel(AttArgs a) {
   if (n < a.n_dst) a.out_dst[u] = pd;
 }
 
-template <int V>
+template <int V, bool ACC>
 __global__ void att_logits_bwd_kernel(AttArgs a) {
   using vec_t = typename Vec<V>::type;
   extern __shared__ float s_part[];            // [2][blockDim][V]
@@ -142,20 +142,25 @@ __global__ void att_logits_bwd_kernel(AttArgs a) {
   const int64_t begin = (int64_t)blockIdx.x * a.rows_per_block;
   const int64_t end = (begin + a.rows_per_block) < a.n_src ? (begin + a.rows_per_block) : a.n_src;
   for (int64_t n0 = begin + ro; n0 < end; n0 += kRowsInFlight * stride) {
-    vec_t xv[kRowsInFlight];
+    vec_t xv[kRowsInFlight], old[kRowsInFlight];
     float gs[kRowsInFlight], gd[kRowsInFlight];
 #pragma unroll
     for (int u = 0; u < kRowsInFlight; ++u) {
       const int64_t n = n0 + u * stride;
       const bool in = n < end;
       xv[u] = in ? *reinterpret_cast<const vec_t*>(a.x + n * F + j * V) : vzero<V>();
+      if (ACC) old[u] = in ? *reinterpret_cast<const vec_t*>(a.grad_x + n * F + j * V) : vzero<V>();
       gs[u] = in ? a.g_src[n * a.heads + h] : 0.f;
       gd[u] = (in && n < a.n_dst) ? a.g_dst[n * a.heads + h] : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < kRowsInFlight; ++u) {
       const int64_t n = n0 + u * stride;
-      if (n < end) *reinterpret_cast<vec_t*>(a.grad_x + n * F + j * V) = axpby(gs[u], as, gd[u], ad);
+      if (n < end) {
+        vec_t gx = axpby(gs[u], as, gd[u], ad);
+        if (ACC) fma_into(gx, 1.f, old[u]);
+        *reinterpret_cast<vec_t*>(a.grad_x + n * F + j * V) = gx;
+      }
       fma_into(acc_s, gs[u], xv[u]);
       fma_into(acc_d, gd[u], xv[u]);
     }
@@ -291,9 +296,9 @@ size_t cxg_attention_logits_workspace_bytes(int64_t n_src, int heads, int channe
 
 int cxg_attention_logits_bwd_f32(const float* x, const float* att_src, const float* att_dst,
                                  const float* g_src, const float* g_dst, int64_t n_src, int64_t n_dst,
-                                 int heads, int channels, float* grad_x, float* grad_att_src,
-                                 float* grad_att_dst, void* workspace, size_t workspace_bytes,
-                                 void* stream) {
+                                 int heads, int channels, float* grad_x, int accumulate,
+                                 float* grad_att_src, float* grad_att_dst, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
   int rc = cxg::check_shape(n_src, n_dst, heads, channels);
   if (rc) return rc;
   CXG_REQUIRE(att_src && att_dst && grad_att_src && grad_att_dst, CXG_ERR_ARG, "null pointer");
@@ -316,8 +321,10 @@ int cxg_attention_logits_bwd_f32(const float* x, const float* att_src, const flo
   cxg::block_shape(a.slots, n_src, &a, &blocks);
   const dim3 grid(blocks), block(a.slots * a.rpb);
   const size_t lds = (size_t)2 * block.x * v * sizeof(float);
-  if (v == 4) hipLaunchKernelGGL(cxg::att_logits_bwd_kernel<4>, grid, block, lds, st, a);
-  else hipLaunchKernelGGL(cxg::att_logits_bwd_kernel<1>, grid, block, lds, st, a);
+  if (v == 4 && accumulate) hipLaunchKernelGGL((cxg::att_logits_bwd_kernel<4, true>), grid, block, lds, st, a);
+  else if (v == 4) hipLaunchKernelGGL((cxg::att_logits_bwd_kernel<4, false>), grid, block, lds, st, a);
+  else if (accumulate) hipLaunchKernelGGL((cxg::att_logits_bwd_kernel<1, true>), grid, block, lds, st, a);
+  else hipLaunchKernelGGL((cxg::att_logits_bwd_kernel<1, false>), grid, block, lds, st, a);
   CXG_LAUNCH_CHECK("att_logits_bwd_kernel");
   hipLaunchKernelGGL(cxg::att_partial_reduce_kernel, dim3((unsigned)cxg::ceil_div(2 * F, 64)),
                      dim3(64 * cxg::kReduceSlices), 0,

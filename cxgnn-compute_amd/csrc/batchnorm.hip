@@ -446,8 +446,11 @@ int cxg_column_sum_f32(const float* x, int64_t n, int c, int64_t ldx, float* out
   CXG_REQUIRE(n >= 0 && c >= 1 && ldx >= c, CXG_ERR_ARG, "column_sum: bad n/c/ldx");
   CXG_REQUIRE(out, CXG_ERR_ARG, "column_sum: null out");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (n == 0) {
-    CXG_HIP_CHECK(hipMemsetAsync(out, 0, (size_t)c * sizeof(float), st));
+  const int waves = cxg::kBnThreads / CXG_WAVE;
+  if (n == 0) {                                  // no rows: the merge of zero partial rows writes the zeros
+    hipLaunchKernelGGL(cxg::column_sum_final_kernel, dim3((c + waves - 1) / waves), dim3(cxg::kBnThreads), 0, st,
+                       static_cast<const float*>(nullptr), 0, c, out);
+    CXG_LAUNCH_CHECK("column_sum_final_kernel");
     return CXG_OK;
   }
   CXG_REQUIRE(x && workspace, CXG_ERR_ARG, "column_sum: null x/workspace");
@@ -465,7 +468,6 @@ int cxg_column_sum_f32(const float* x, int64_t n, int c, int64_t ldx, float* out
     hipLaunchKernelGGL(cxg::column_sum_partial_kernel<1>, grid, block, 0, st, x, n, c, ldx, g.tx_shift,
                        g.rows_per_block, partial);
   CXG_LAUNCH_CHECK("column_sum_partial_kernel");
-  const int waves = cxg::kBnThreads / CXG_WAVE;
   hipLaunchKernelGGL(cxg::column_sum_final_kernel, dim3((c + waves - 1) / waves), block, 0, st, partial,
                      g.row_blocks, c, out);
   CXG_LAUNCH_CHECK("column_sum_final_kernel");

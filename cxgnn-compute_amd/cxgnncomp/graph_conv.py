@@ -439,6 +439,60 @@ class AttentionLogitsOP(torch.autograd.Function):
         return gx, ga_src.view_as(att_src), ga_dst.view_as(att_dst), None
 
 
+class GatLayerOP(torch.autograd.Function):
+    """``MyGATConv.forward_many`` (several heads) on CUDA tensors as one autograd node: linear
+    map, both attention logits, fused edge softmax, edge-weighted aggregation, head
+    concatenation or mean, bias.  The backward pass runs the same kernels as the separate
+    nodes do, but the two gradients of the transformed features -- from the aggregation
+    and from the logits -- meet in one buffer (the logits kernel adds into what the
+    transposed aggregation wrote) instead of two tensors and a full-size add, and the
+    intermediate views cost no copies."""
+
+    @staticmethod
+    def forward(ctx, x, w, att_src, att_dst, bias, ptr, idx, num_dst, num_src, num_edge, slope, heads, concat):
+        H, C = heads, w.shape[0] // heads
+        xs = F.linear(x[:num_src], w).view(-1, H, C)
+        a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
+        ev, mask = _ops.edge_softmax_fwd(ptr, idx, a_dst, a_src, num_edge, slope)
+        out = _ops.spmm(ptr, idx, xs, num_dst, val=ev)
+        out = out.view(-1, H * C) if concat else out.mean(dim=1)
+        if bias is not None:
+            out.add_(bias)
+        ctx.save_for_backward(x, w, att_src, att_dst, xs, ev, mask, ptr, idx)
+        ctx.dims = (num_dst, num_src, H, C, concat, float(slope), bias is not None)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, w, att_src, att_dst, xs, ev, mask, ptr, idx = ctx.saved_tensors
+        num_dst, num_src, H, C, concat, slope, has_bias = ctx.dims
+        g = g.contiguous()
+        g_bias = _ops.column_sum(g) if has_bias and ctx.needs_input_grad[4] else None
+        if concat:
+            g3 = g.view(-1, H, C)
+        else:
+            g3 = (g / H).unsqueeze(1).expand(-1, H, -1).contiguous()
+        tg = _ops.transposed(ptr, idx, num_dst, xs.shape[0])
+        g_xs = _ops.spmm(tg.ptr_t, tg.idx_t, g3, xs.shape[0], val=ev, val_perm=tg.perm)
+        g_ev = torch.empty((idx.shape[0], H), dtype=torch.float32, device=g.device)
+        if tg.n_edges < idx.shape[0]:
+            g_ev[tg.n_edges:].zero_()
+        g_ev = _ops.sddmm_csr(ptr, idx, xs, g3, num_dst, out=g_ev)[:ev.shape[0]]
+        g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope)
+        g_asrc = _ops.narrow_gather_sum(tg.ptr_t, tg.perm, t_edge, xs.shape[0], rows32=_ops.rows32_transposed(tg))
+        _, g_att_src, g_att_dst = _ops.attention_logits_bwd(xs, att_src, att_dst, g_asrc, g_adst, add_to=g_xs)
+        g_xs2 = g_xs.view(-1, H * C)
+        g_x = g_w = None
+        if ctx.needs_input_grad[0]:
+            g_x = g_xs2 @ w
+            if g_x.shape[0] < x.shape[0]:
+                g_x = torch.cat([g_x, g_x.new_zeros(x.shape[0] - g_x.shape[0], g_x.shape[1])])
+        if ctx.needs_input_grad[1]:
+            g_w = _weight_grad(x[:num_src], g_xs2)
+        return (g_x, g_w, g_att_src.view_as(att_src), g_att_dst.view_as(att_dst), g_bias,
+                None, None, None, None, None, None, None, None)
+
+
 class MyGATConv(torch.nn.Module):
 
     def __init__(self, in_channels, out_channels, heads=1, concat=False, negative_slope=0.2,
@@ -496,6 +550,11 @@ class MyGATConv(torch.nn.Module):
     def forward_many(self, x, ptr, idx, num_dst, num_src, num_edge):
         H, C = self.heads, self.out_channels
         assert x.dim() == 2
+        if x.is_cuda and self.edge_softmax_schedule == "fused" and C % 4 == 0:
+            x = TimerOP.apply(x, "gat layer", True)
+            out = GatLayerOP.apply(x, self.lin_src, self.att_src, self.att_dst, self.bias, ptr, idx, int(num_dst),
+                                   int(num_src), int(num_edge), self.negative_slope, H, self.concat)
+            return TimerOP.apply(out, "gat layer", False)
         x = TimerOP.apply(x, "linear1", True)
         x_src = x_dst = linear(x[:num_src], self.lin_src).view(-1, H, C)
         x_src = TimerOP.apply(x_src, "linear1", False)

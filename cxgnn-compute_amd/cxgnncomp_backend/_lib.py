@@ -69,7 +69,8 @@ SIGNATURES = {
     "cxg_coo_to_csr_i64": (_I32, [_P, _P, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
     "cxg_attention_logits_fwd_f32": (_I32, [_P, _P, _P, _I64, _I64, _I32, _I32, _P, _P, _P]),
     "cxg_attention_logits_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
-    "cxg_attention_logits_bwd_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _P, _P, _P, _SZ, _P]),
+    "cxg_attention_logits_bwd_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _I32, _P, _P, _P, _SZ,
+                                            _P]),
     "cxg_batchnorm_workspace_bytes": (_SZ, [_I64, _I32]),
     "cxg_column_sum_f32": (_I32, [_P, _I64, _I32, _I64, _P, _P, _SZ, _P]),
     "cxg_batchnorm_stats_f32": (_I32, [_P, _I64, _I32, _I64, _F32, _P, _P, _P, _P, _SZ, _P]),

@@ -383,8 +383,9 @@ def attention_logits(x, att_src, att_dst, n_dst):
     return out_src, out_dst
 
 
-def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst):
-    """Gradients of ``attention_logits``: (grad_x, grad_att_src, grad_att_dst), reproducible."""
+def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst, add_to=None):
+    """Gradients of ``attention_logits``: (grad_x, grad_att_src, grad_att_dst), reproducible.
+    ``add_to`` (shaped like x) receives grad_x added in place and is returned as grad_x."""
     lib = _lib.load()
     _req(x, "x", torch.float32, 3)
     n_src, heads, channels = x.shape
@@ -396,7 +397,11 @@ def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst):
     if tuple(g_src.shape) != (n_src, heads) or g_dst.shape[1] != heads or n_dst > n_src:
         raise ValueError("gradient shapes %s / %s do not fit x %s"
                          % (tuple(g_src.shape), tuple(g_dst.shape), tuple(x.shape)))
-    grad_x = torch.empty_like(x)
+    if add_to is not None:
+        _req(add_to, "add_to", torch.float32, 3)
+        if add_to.shape != x.shape or add_to.device != x.device:
+            raise ValueError("add_to %s does not fit x %s" % (tuple(add_to.shape), tuple(x.shape)))
+    grad_x = torch.empty_like(x) if add_to is None else add_to
     ga_src = torch.empty(heads, channels, dtype=torch.float32, device=x.device)
     ga_dst = torch.empty(heads, channels, dtype=torch.float32, device=x.device)
     ws_bytes = lib.cxg_attention_logits_workspace_bytes(n_src, heads, channels)
@@ -404,7 +409,8 @@ def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst):
     with torch.cuda.device(x.device):
         st = lib.cxg_attention_logits_bwd_f32(_lib.ptr(x), att_src.data_ptr(), att_dst.data_ptr(),
                                               _lib.ptr(g_src), _lib.ptr(g_dst), n_src, n_dst, heads, channels,
-                                              _lib.ptr(grad_x), ga_src.data_ptr(), ga_dst.data_ptr(),
+                                              _lib.ptr(grad_x), int(add_to is not None), ga_src.data_ptr(),
+                                              ga_dst.data_ptr(),
                                               ws.data_ptr(), ws.numel(), _lib.current_stream(x.device))
     _lib.check(st)
     return grad_x, ga_src, ga_dst

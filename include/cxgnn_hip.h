@@ -317,13 +317,15 @@ size_t cxg_attention_logits_workspace_bytes(int64_t n_src, int heads, int channe
  *   grad_x[n, h, c]    = g_src[n, h] * att_src[h, c] + (n < n_dst) g_dst[n, h] * att_dst[h, c]
  *   grad_att_src[h, c] = sum_n g_src[n, h] * x[n, h, c]
  *   grad_att_dst[h, c] = sum_{n < n_dst} g_dst[n, h] * x[n, h, c]
- * All three outputs are overwritten; the sums run in a fixed order (reproducible).
+ * grad_att_* are overwritten; grad_x is overwritten, or, with accumulate != 0, added to
+ * (the layer's other gradient of x, from the aggregation, is already there: autograd's
+ * sum of the two).  The sums run in a fixed order (reproducible).
  * The autograd of the same two expressions (cxgnncomp/graph_conv.py:466-467). */
 int cxg_attention_logits_bwd_f32(const float* x, const float* att_src, const float* att_dst,
                                  const float* g_src, const float* g_dst, int64_t n_src,
                                  int64_t n_dst, int heads, int channels, float* grad_x,
-                                 float* grad_att_src, float* grad_att_dst, void* workspace,
-                                 size_t workspace_bytes, void* stream);
+                                 int accumulate, float* grad_att_src, float* grad_att_dst,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* Batch normalisation over the rows of x[n, c] (row stride ldx), the layer the upstream
  * models put between two convolutions (torch.nn.BatchNorm1d, cxgnncomp/model.py:28 and

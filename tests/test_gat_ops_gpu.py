@@ -249,6 +249,12 @@ def test_attention_logits_forward_backward(shape, n_src, n_dst):
         scale = max(1.0, float(np.abs(ref).max()))
         assert_close(_np(got) / scale, ref / scale, RTOL, ATOL, name)
     assert torch.equal(ga_s, ga_s2) and torch.equal(ga_d, ga_d2) and torch.equal(gx, gx2)
+    # adding into an existing gradient of x
+    base = torch.randn(n_src, H, C, generator=torch.Generator().manual_seed(8))
+    acc = base.cuda()
+    gx3, ga_s3, _ = _ops.attention_logits_bwd(x.cuda(), a_s.cuda(), a_d.cuda(), gs.cuda(), gd.cuda(), add_to=acc)
+    assert gx3.data_ptr() == acc.data_ptr() and torch.equal(ga_s3, ga_s)
+    assert_close(_np(acc), base.numpy() + xd.grad.numpy(), RTOL, ATOL, "grad x added in place")
 
 
 def test_attention_logits_op_autograd():
