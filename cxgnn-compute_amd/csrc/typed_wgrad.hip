@@ -14,9 +14,10 @@
 // row-consecutive bf16 values as one 8-byte LDS store into [column][row] order.
 //
 // Split over the rows: a block owns `rows_per_chunk` rows of one relation and one
-// 128-column tile of G, keeps the 128 x 128 partial in registers (wave w: output
-// rows 32w .. 32w+31) and writes it to a partial buffer; a second kernel adds the
-// partials of each relation in chunk order -- no atomics, deterministic.
+// 128-column tile of G, keeps the 128 x 128 partial in the registers of its four
+// consumer waves (wave w: output rows 32w .. 32w+31) and writes it to a partial buffer;
+// a second kernel adds the partials of each relation in chunk order -- no atomics,
+// deterministic.
 //
 // Replaces the weight-gradient half of TypedLinearE2EOP.backward /
 // TypedLinearS2DMMAggrOP.backward (cxgnncomp/typed_linear.py:114-137,205-221),
@@ -71,11 +72,30 @@ __device__ __forceinline__ bool locate_chunk(const int64_t* __restrict__ seg, in
   return false;
 }
 
+// 768 threads in three groups of four waves, so that the conversion work (vector ALU, LDS
+// stores) of the next tile runs beside the matrix instructions of the current one on
+// every SIMD:
+//   waves 4-7 load 32 rows of A two tiles ahead, split them into bf16 parts and stage
+//     tile t+1 into one half of the double-buffered LDS; waves 8-11 do the same for G;
+//   waves 0-3 (consumers) multiply tile t from the other half, 32 output rows each.
+// One barrier per tile.  Each role has its own loop: the register needs differ (staging
+// registers against accumulators) and a common loop would hold the union.
+constexpr int kWgThreads = 768;
+constexpr int kMapSlots = 4;             // tiles of row maps in LDS
+
 template <int NS>
-__global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g) {
-  __shared__ __attribute__((aligned(16))) uint16_t At[NS][128][kMP];   // [part][k][row]
-  __shared__ __attribute__((aligned(16))) uint16_t Gt[NS][128][kMP];   // [part][n][row]
-  __shared__ int64_t s_src[3][kMT], s_dst[3][kMT];
+constexpr size_t wgrad_lds_bytes() { return (size_t)2 * 2 * NS * 128 * kMP * sizeof(uint16_t); }
+
+template <int NS>
+__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(3)))
+void typed_wgrad_split_kernel(WgradArgs g) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t s_tiles[];
+  typedef uint16_t (*tile_t)[128][kMP];                       // [part][column][row]
+  // s_tiles: At[2][NS][128][kMP], then Gt[2][NS][128][kMP]
+  auto tile_buf = [&](int operand, int b) -> tile_t {
+    return reinterpret_cast<tile_t>(s_tiles + (size_t)(2 * operand + b) * NS * 128 * kMP);
+  };
+  __shared__ int64_t s_map[2][kMapSlots][kMT];                // [operand][tile slot][row]
   // The column tiles of one row chunk get consecutive slots of one XCD (blocks go to
   // the 8 XCDs round-robin by index), so the chunk's A rows are fetched into one L2.
   const int n_ct = (g.N + 127) / 128;
@@ -85,52 +105,53 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
   int rel = 0;
   int64_t row0 = 0, row_end = 0;
   const bool have = locate_chunk(g.seg, g.R, g.rows_per_chunk, chunk, rel, row0, row_end);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = uniform_i32(tid >> 6);
   const int K = g.K, N = g.N;
-  float* const part = g.partial + ((size_t)chunk * K) * (size_t)N;
-  v16f acc[4];
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[nb][i] = 0.f;
+  const int64_t rows_here = !have ? 0 : ((row_end - row0) < g.rows_per_chunk ? (row_end - row0) : g.rows_per_chunk);
+  const int n_tiles = (int)((rows_here + kMT - 1) / kMT);
 
-  if (have) {
-    const int64_t rows_here = (row_end - row0) < g.rows_per_chunk ? (row_end - row0) : g.rows_per_chunk;
-    const int n_tiles = (int)((rows_here + kMT - 1) / kMT);
-    // float4 column and group of 4 rows of this thread: 8 lanes run along a row (128
-    // contiguous bytes per global load), the other lane bits select the row group, so
-    // the transposed 8-byte LDS stores of a wave spread over the banks (2-way conflicts
-    // at most with the 80-byte pitch) instead of piling onto four of them.
-    const int c4 = wave * 8 + (lane & 7), mg = lane >> 3;
-    const bool ka_ok = 4 * c4 < K;
-    const bool ng_ok = n0 + 4 * c4 < N;               // N % 4 == 0 is required
+  if (wave >= 4) {
+    // ---- producers: operand 0 = A (waves 4-7), operand 1 = G (waves 8-11) ---------------
+    if (n_tiles == 0) return;
+    const int operand = (wave - 4) >> 2, pwave = (wave - 4) & 3, ptid = tid - 256 - operand * 256;
+    // float4 column and group of 4 rows of this thread.  The low lane bits select the row
+    // group and the high ones the column: the 16 lanes the LDS serves together then
+    // write 8 row groups of 2 columns, 32 different banks with the 80-byte pitch (with
+    // the bits the other way round four lanes met in every bank), while a global load
+    // still covers 8 rows with 128 contiguous bytes each.
+    const int c4 = pwave * 8 + (lane >> 3), mg = lane & 7;
+    const bool col_ok = operand ? (n0 + 4 * c4 < N) : (4 * c4 < K);      // N % 4 == 0 is required
+    const float* const base = operand ? g.g + (col_ok ? n0 + 4 * c4 : 0) : g.a + (col_ok ? 4 * c4 : 0);
+    const int64_t ld = operand ? g.ldg : g.lda;
+    const int64_t* const map = operand ? g.dst : g.src;
     auto load_maps = [&](int t) {
-      if (tid < kMT && t < n_tiles) {
-        const int64_t gr = row0 + (int64_t)t * kMT + tid;
-        int64_t sidx = -1, didx = -1;
+      if (ptid < kMT && t < n_tiles) {
+        const int64_t gr = row0 + (int64_t)t * kMT + ptid;
+        int64_t ridx = -1;
         if (gr < row_end) {
-          sidx = g.src ? g.src[gr] : gr;
-          didx = g.dst ? g.dst[gr] : gr;
-          if (sidx < 0 || didx < 0) { sidx = -1; didx = -1; }
+          // a negative entry in either map drops the row from the product
+          const int64_t sidx = g.src ? g.src[gr] : gr, didx = g.dst ? g.dst[gr] : gr;
+          ridx = (sidx < 0 || didx < 0) ? -1 : (operand ? didx : sidx);
         }
-        s_src[t % 3][tid] = sidx;
-        s_dst[t % 3][tid] = didx;
+        s_map[operand][t % kMapSlots][ptid] = ridx;
       }
     };
     // Loads are issued unconditionally: rows and columns that do not exist are redirected
     // to an address that does and zeroed when the tile is staged (a select between a
     // loaded vector and a zero vector made the compiler route the load through scratch).
-    auto gload = [&](float4 (&ar)[4], float4 (&gr4)[4], int t) {
+    auto gload = [&](float4 (&r4)[4], int t) {
       const int tc = t < n_tiles ? t : n_tiles - 1;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int64_t sidx = s_src[tc % 3][mg * 4 + i], didx = s_dst[tc % 3][mg * 4 + i];
-        ar[i] = *reinterpret_cast<const float4*>(g.a + (sidx >= 0 ? sidx : 0) * g.lda + (ka_ok ? 4 * c4 : 0));
-        gr4[i] = *reinterpret_cast<const float4*>(g.g + (didx >= 0 ? didx : 0) * g.ldg + (ng_ok ? n0 + 4 * c4 : 0));
+        const int64_t ridx = s_map[operand][tc % kMapSlots][mg * 4 + i];
+        r4[i] = *reinterpret_cast<const float4*>(base + (ridx >= 0 ? ridx : 0) * ld);
       }
     };
     // registers (4 rows x 4 columns) -> LDS [column][4 consecutive rows], split into parts
-    auto stage = [&](const float4 (&r4)[4], uint16_t (&dst)[NS][128][kMP], const int64_t* rows, bool col_ok) {
+    auto stage_tile = [&](const float4 (&r4)[4], int t) {
+      if (t >= n_tiles) return;
+      const tile_t dst = tile_buf(operand, t & 1);
+      const int64_t* rows = s_map[operand][t % kMapSlots];
       float v[4][4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -154,12 +175,43 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
         for (int q = 0; q < NS; ++q) *reinterpret_cast<v4bf*>(&dst[q][4 * c4 + c][mg * 4]) = out[q];
       }
     };
-    auto tile_step = [&](float4 (&ar)[4], float4 (&gr4)[4], int t) {
-      stage(ar, At, s_src[t % 3], ka_ok);
-      stage(gr4, Gt, s_dst[t % 3], ng_ok);
-      load_maps(t + 2);
+    float4 r0[4], r1[4];
+    load_maps(0);
+    load_maps(1);
+    load_maps(2);
+    __syncthreads();                                   // #1: the first maps are there
+    gload(r0, 0);
+    gload(r1, 1);
+    stage_tile(r0, 0);
+    gload(r0, 2);
+    __syncthreads();                                   // #2: tile 0 is staged
+    // iteration t: stage tile t+1, maps of tile t+3, barrier, load tile t+3
+    for (int t = 0; t < n_tiles; t += 2) {
+      stage_tile(r1, t + 1);
+      load_maps(t + 3);
       __syncthreads();
-      gload(ar, gr4, t + 2);
+      gload(r1, t + 3);
+      if (t + 1 >= n_tiles) break;
+      stage_tile(r0, t + 2);
+      load_maps(t + 4);
+      __syncthreads();
+      gload(r0, t + 4);
+    }
+    return;
+  }
+
+  // ---- consumers --------------------------------------------------------------------
+  float* const part = g.partial + ((size_t)chunk * K) * (size_t)N;
+  v16f acc[4];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[nb][i] = 0.f;
+  if (n_tiles > 0) {
+    __syncthreads();                                   // #1
+    __syncthreads();                                   // #2
+    for (int t = 0; t < n_tiles; ++t) {
+      const tile_t At = tile_buf(0, t & 1), Gt = tile_buf(1, t & 1);
 #pragma unroll
       for (int ms = 0; ms < kMT / 16; ++ms) {
         const int m = ms * 16 + (lane >> 5) * 8;
@@ -178,17 +230,7 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
               acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[order - i], acc[nb], 0, 0, 0);
         }
       }
-      __syncthreads();   // every wave is done with At / Gt before the next tile is staged
-    };
-    float4 a0[4], g0[4], a1[4], g1[4];
-    load_maps(0);
-    load_maps(1);
-    __syncthreads();
-    gload(a0, g0, 0);
-    gload(a1, g1, 1);
-    for (int t = 0; t < n_tiles; t += 2) {
-      tile_step(a0, g0, t);
-      if (t + 1 < n_tiles) tile_step(a1, g1, t + 1);
+      __syncthreads();   // tile t+1 is staged, and every wave is done with tile t
     }
   }
   // partial[chunk][k][n] (zeros for chunk numbers past the last relation)
@@ -202,6 +244,14 @@ __global__ __launch_bounds__(kThreads) void typed_wgrad_split_kernel(WgradArgs g
       if (k < K) part[(size_t)k * N + col] = acc[nb][i];
     }
   }
+}
+
+// Dynamic LDS above the default 64 KB limit has to be enabled per kernel.
+template <typename KernelT>
+hipError_t allow_lds(KernelT kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             (int)bytes);
 }
 
 // gw[r][k][n] = sum of the partials of relation r's chunks, in a fixed order: the chunks
@@ -285,9 +335,14 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
   CXG_REQUIRE(chunks * n_ct < ((int64_t)1 << 31), CXG_ERR_UNSUPPORTED, "too many chunks for one launch");
   cxg::WgradArgs wa{a, lda, g, ldg, src_idx, dst_idx, seg_ptr, reinterpret_cast<float*>(workspace),
                     M, K, N, R, rows};
-  const dim3 grid((unsigned)(chunks * n_ct)), block(cxg::kThreads);
-  if (flags & CXG_GEMM_SPLIT_BF16X3) hipLaunchKernelGGL(cxg::typed_wgrad_split_kernel<2>, grid, block, 0, st, wa);
-  else hipLaunchKernelGGL(cxg::typed_wgrad_split_kernel<3>, grid, block, 0, st, wa);
+  const dim3 grid((unsigned)(chunks * n_ct)), block(cxg::kWgThreads);
+  if (flags & CXG_GEMM_SPLIT_BF16X3) {
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_wgrad_split_kernel<2>, cxg::wgrad_lds_bytes<2>()));
+    hipLaunchKernelGGL(cxg::typed_wgrad_split_kernel<2>, grid, block, cxg::wgrad_lds_bytes<2>(), st, wa);
+  } else {
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_wgrad_split_kernel<3>, cxg::wgrad_lds_bytes<3>()));
+    hipLaunchKernelGGL(cxg::typed_wgrad_split_kernel<3>, grid, block, cxg::wgrad_lds_bytes<3>(), st, wa);
+  }
   CXG_LAUNCH_CHECK("typed_wgrad_split_kernel");
   const int64_t kn = (int64_t)K * N;
   hipLaunchKernelGGL(cxg::wgrad_reduce_kernel, dim3((unsigned)cxg::ceil_div(kn, 64), (unsigned)R),
