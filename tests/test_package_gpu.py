@@ -477,3 +477,48 @@ def test_sage_layer_on_a_row_prefix(widths):
     for k, v in layer.named_parameters():
         sc = max(1.0, float(P[k].grad.abs().max()))
         assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "frozen input, grad " + k)
+
+
+@pytest.mark.parametrize("concat", [True, False])
+def test_gat_layer_on_a_row_prefix(concat):
+    """MyGATConv (several heads, one autograd node on CUDA) on a sampled-batch layer: num_dst
+    destination rows over num_src source rows of a longer x; output and every gradient against
+    the float64 composition of the upstream expressions."""
+    import cxgnncomp
+    cxgnncomp.set_timers()               # MyGATConv brackets its phases with TimerOP, as upstream
+    torch.manual_seed(6)
+    n_all, n_src, n_dst, fin, H, C = 700, 600, 200, 24, 4, 8
+    deg = torch.randint(0, 12, (n_dst,))
+    deg[3] = 0
+    ptr = torch.zeros(n_dst + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(deg, 0)
+    E = int(ptr[-1])
+    idx = torch.randint(0, n_src, (E,))
+    dst = torch.repeat_interleave(torch.arange(n_dst), deg)
+    x = torch.randn(n_all, fin)
+    layer = cxgnncomp.MyGATConv(fin, C, heads=H, concat=concat).cuda()
+    with torch.no_grad():
+        layer.bias.normal_()
+    xg = x.cuda().requires_grad_(True)
+    announce("GatLayerOP prefix rows concat=%s" % concat)
+    out = layer(xg, ptr.cuda(), idx.cuda(), n_dst, n_src, E)
+    w = torch.randn(*out.shape)
+    (out * w.cuda()).sum().backward()
+    torch.cuda.synchronize()
+    P = {k: v.detach().double().cpu().requires_grad_(True) for k, v in layer.named_parameters()}
+    x64 = x.double().requires_grad_(True)
+    xs = (x64[:n_src] @ P["lin_src"].T).view(-1, H, C)
+    a_s = (xs * P["att_src"]).sum(-1)
+    a_d = (xs[:n_dst] * P["att_dst"]).sum(-1)
+    ev = pyref.edge_softmax_opwise(ptr, idx, a_s, a_d, E, 0.2)
+    ref = torch.zeros(n_dst, H, C, dtype=torch.float64).index_add_(0, dst, xs[idx] * ev.unsqueeze(-1))
+    ref = (ref.view(-1, H * C) if concat else ref.mean(dim=1)) + P["bias"]
+    (ref * w.double()).sum().backward()
+    assert out.shape == ref.shape
+    assert_close(_np(out), ref.detach().numpy(), 2e-4, 2e-5, "fwd")
+    assert xg.grad.shape == x.shape and float(xg.grad[n_src:].abs().max()) == 0.0
+    sc = max(1.0, float(x64.grad.abs().max()))
+    assert_close(_np(xg.grad) / sc, x64.grad.numpy() / sc, 2e-4, 2e-5, "grad x")
+    for k, v in layer.named_parameters():
+        sc = max(1.0, float(P[k].grad.abs().max()))
+        assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "grad " + k)
