@@ -239,7 +239,7 @@ def _weight_grad(x, g, src, dst, seg, shape):
         b, e = bounds[r], bounds[r + 1]
         if e > b:
             xs = _ops.gather_rows(x, src[b:e].contiguous())
-            gs = _ops.gather_rows(g, dst[b:e].contiguous())
+            gs = g[b:e] if dst is None else _ops.gather_rows(g, dst[b:e].contiguous())
             gw[r] = torch.mm(xs.t(), gs)
     return gw
 
@@ -249,8 +249,9 @@ def _weight_grad(x, g, src, dst, seg, shape):
 # concatenated weights.  2 * n_src * R * K * N flops instead of 2 * E * K * N, no
 # atomics, deterministic; the aggregation is the plain SpMM over a combined index.
 # Chosen when the graph has at least half as many edges as (source, relation)
-# pairs and Y fits the memory budget; sparser inputs (sampled blocks with many
-# relations) use the fused gather-GEMM-scatter launch.
+# pairs and Y fits the memory budget -- on the pairs that own an edge only when those
+# are a minority (_pair_graph); sparser inputs (sampled blocks with many relations)
+# write one GEMM row per edge, or use the fused gather-GEMM-scatter launch.
 RGCN_DENSE_MAX_BYTES = 64 << 30
 RGCN_EDGE_ROWS_MAX_BYTES = 64 << 30        # per-edge rows of the sparse strategy; above: atomic scatter
 
@@ -290,6 +291,62 @@ def _rel_graph(ptr, idx, rel, n, n_src, R):
     return rg
 
 
+class _PairGraph:
+    """Index structures of the pair-compacted transform-first path for one (ptr, idx, rel).
+    Only the (source, relation) pairs that own an edge get a row of Y = x W, only the
+    (destination, relation) pairs that own one a row of Z = g W^T:
+      f_src [Uf], f_seg [R+1]  source of every forward pair, pairs sorted by (relation, source);
+      f_row [E]                pair row of every edge, in CSR edge order;
+      f_ptr [Uf+1], f_dst [E]  CSR over the forward pairs: destinations of a pair's edges;
+      b_dst [Ub], b_seg [R+1]  destination of every backward pair, sorted by (relation, destination);
+      ptr_src [n_src+1], b_row_rev [E]  reversed graph (rows = sources) and, per reversed edge,
+                               its backward pair row."""
+    __slots__ = ("n_edges", "f_src", "f_seg", "f_row", "f_ptr", "f_dst", "b_dst", "b_seg", "ptr_src", "b_row_rev",
+                 "_keep")
+
+
+_PAIR_CACHE = collections.OrderedDict()
+
+
+def _pair_graph(ptr, idx, rel, n, n_src, R):
+    key = (ptr.data_ptr(), idx.data_ptr(), rel.data_ptr(), ptr.shape[0], idx.shape[0], n, n_src, R,
+           ptr._version, idx._version, rel._version, ptr.device.index)
+    pg = _PAIR_CACHE.get(key)
+    if pg is not None:
+        _PAIR_CACHE.move_to_end(key)
+        return pg
+    pg = _PairGraph()
+    e = pg.n_edges = int(ptr[n].item())
+    dev = ptr.device
+    rel64 = rel[:e].to(torch.int64)
+    if e and (int(rel64.min()) < 0 or int(rel64.max()) >= R):
+        raise ValueError("relation ids must lie in [0, %d)" % R)
+    src = idx[:e]
+    dst = _ops.csr_row_ids(ptr, n, e)
+    bounds = torch.arange(R + 1, dtype=torch.int64, device=dev)
+    uf, pg.f_row = torch.unique(rel64 * n_src + src, sorted=True, return_inverse=True)
+    pg.f_src = (uf % n_src).contiguous()
+    pg.f_seg = torch.searchsorted(uf, bounds * n_src).contiguous()
+    pg.f_row = pg.f_row.contiguous()
+    pg.f_ptr, pg.f_dst, _ = _ops.coo_to_csr(dst, pg.f_row, uf.shape[0])
+    ub, b_row = torch.unique(rel64 * n + dst, sorted=True, return_inverse=True)
+    pg.b_dst = (ub % n).contiguous()
+    pg.b_seg = torch.searchsorted(ub, bounds * n).contiguous()
+    tg = _ops.transposed(ptr, idx, n, n_src)
+    pg.ptr_src = tg.ptr_t
+    pg.b_row_rev = b_row[tg.perm].contiguous()
+    pg._keep = (ptr, idx, rel)
+    _PAIR_CACHE[key] = pg
+    while len(_PAIR_CACHE) > _REL_CACHE_CAP:
+        _PAIR_CACHE.popitem(last=False)
+    return pg
+
+
+# The dense table is kept when nearly every (source, relation) pair owns an edge: its GEMM
+# reads and writes contiguous rows, the compacted one gathers its input rows.
+RGCN_PAIR_FILL_MAX = 0.8
+
+
 def _dense_seg(n_rows, device):
     return torch.tensor([0, n_rows], dtype=torch.int64, device=device)
 
@@ -318,6 +375,18 @@ class _RgcnFusedFunction(torch.autograd.Function):
         ctx.n, ctx.mean = n, mean
         n_edges = int(ptr[n].item())
         ctx.dense = force_dense or _use_dense(n_edges, n_src, R, N)
+        ctx.pairs = False
+        if ctx.dense:
+            # transform-first over the pairs that occur: Y and Z hold one row per (node, relation)
+            # pair that owns an edge instead of one per pair that could
+            pg = _pair_graph(ptr, idx, rel, n, n_src, R)
+            ctx.pairs = pg.f_src.shape[0] <= RGCN_PAIR_FILL_MAX * n_src * R
+        if ctx.pairs:
+            y = typed_gemm(x, weights, pg.f_seg, pg.f_src.shape[0], src_idx=pg.f_src)    # [Uf, N]
+            out = _ops.spmm(ptr, pg.f_row, y, n, mean=mean)
+            ctx.pg = pg
+            ctx.save_for_backward(x, weights, ptr)
+            return out
         if ctx.dense:
             rg = _rel_graph(ptr, idx, rel, n, n_src, R)
             wcat = weights.permute(1, 0, 2).reshape(1, K, R * N).contiguous()
@@ -353,6 +422,19 @@ class _RgcnFusedFunction(torch.autograd.Function):
         if ctx.mean:
             grad_out = grad_out * _inv_degree(ptr, n).unsqueeze(1)
         gx = gw = None
+        if ctx.pairs:
+            pg = ctx.pg
+            if ctx.needs_input_grad[0]:
+                # Z = g[d] @ W[r]^T for the (destination, relation) pairs that occur, then the
+                # plain SpMM over the reversed graph
+                z = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, pg.b_dst.shape[0],
+                               src_idx=pg.b_dst)
+                gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, z, n_src)
+            if ctx.needs_input_grad[3]:
+                # gY = sum of g over the edges of every (source, relation) pair; gW[r] = x[src]^T gY
+                gy = _ops.spmm(pg.f_ptr, pg.f_dst, grad_out, pg.f_src.shape[0])
+                gw = _weight_grad(x, gy, pg.f_src, None, pg.f_seg, weights.shape)
+            return gx, None, None, gw, None, None, None, None
         if ctx.dense:
             rg = ctx.rg
             if ctx.needs_input_grad[0]:

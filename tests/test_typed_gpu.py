@@ -165,19 +165,22 @@ def test_rgcn_fused_toy_all_ones():
     assert torch.all(out.cpu() == 3968.0)
 
 
-@pytest.mark.parametrize("strategy", ["transform_first", "per_edge_rows", "gather_gemm_scatter"])
+@pytest.mark.parametrize("strategy", ["transform_first", "pair_rows", "per_edge_rows", "gather_gemm_scatter"])
 @pytest.mark.parametrize("K,N,R", [(128, 128, 16), (64, 32, 3)])
 def test_rgcn_fused_forward_backward(K, N, R, strategy, monkeypatch):
-    """The three strategies of the fused relational layer: dense transform of every (source,
-    relation) pair, one GEMM row per edge summed per destination, atomic scatter."""
+    """The four strategies of the fused relational layer: dense transform of every (node,
+    relation) pair, transform of the pairs that own an edge, one GEMM row per edge summed per
+    destination, atomic scatter."""
     import cxgnncomp_backend as B
     from cxgnncomp import synthetic as S
     from cxgnncomp_backend import _typed
-    if strategy != "transform_first":
-        monkeypatch.setattr(_typed, "RGCN_DENSE_MAX_BYTES", 0)    # rules the dense path out
+    if strategy not in ("transform_first", "pair_rows"):
+        monkeypatch.setattr(_typed, "RGCN_DENSE_MAX_BYTES", 0)    # rules the transform-first paths out
     if strategy == "gather_gemm_scatter":
         monkeypatch.setattr(_typed, "RGCN_EDGE_ROWS_MAX_BYTES", 0)   # and the per-edge rows
-    assert _typed._use_dense(40000, 3000, R, N) == (strategy == "transform_first")
+    # the share of pairs that own an edge decides between the dense table and the compacted one
+    monkeypatch.setattr(_typed, "RGCN_PAIR_FILL_MAX", 2.0 if strategy == "pair_rows" else -1.0)
+    assert _typed._use_dense(40000, 3000, R, N) == (strategy in ("transform_first", "pair_rows"))
     ptr, idx, etype, _ = S.hetero_graph(3000, 40000, num_rel=R, seed=4)
     n = ptr.shape[0] - 1
     torch.manual_seed(14)
