@@ -401,7 +401,7 @@ def c4(iters):
            E * (4 * K + 8 * K + 12) + 4 * R * K * K, flops)
     del oe2
     on = torch.zeros(N, K, device="cuda")
-    report("c4", "typed_linear_s2d (out[dst[e]] += x[src[e]] W[type[e]]; per-row products summed per destination)",
+    report("c4", "typed_linear_s2d (out[dst[e]] += x[src[e]] W[type[e]]; products of the (source, type) pairs that occur, summed per destination)",
            timeit(lambda: B.typed_linear_s2d(x, w, on, idx, rows, rel32), max(2, iters // 2)),
            fused_bytes, flops)
     del on

@@ -142,20 +142,52 @@ def _typed_rows(vin, weights, output, types, src_id, dst_id, atomic):
     num = types.shape[0] if src_id is None else src_id.shape[0]
     if num == 0:
         return
-    perm, seg = rel_segment(types[:num].contiguous(), weights.shape[0])
-    src = perm if src_id is None else src_id[perm]
     if atomic and 4 * num * weights.shape[2] <= RGCN_EDGE_ROWS_MAX_BYTES:
         # several rows share a destination: instead of fp32 atomics, one product row per
-        # input row (written once, in input order), then every destination sums its own
-        # rows (positions grouped by destination once per dst_id array) and adds them
-        per_row = torch.empty((num, weights.shape[2]), dtype=torch.float32, device=vin.device)
-        typed_gemm(vin, weights, seg, num, src_idx=src, dst_idx=perm, out=per_row)
-        groups = _ops.dest_groups(dst_id[:num], output.shape[0])
-        output += _ops.spmm(groups.ptr, groups.perm, per_row, output.shape[0])
+        # (source, type) pair that occurs (rows that repeat a pair share it), then every
+        # destination sums the product rows of its input rows and adds them.  The pair
+        # list and the grouping by destination are built once per index arrays.
+        ptr_d, rows_d, pair_src, pair_seg = _scatter_pairs(src_id, types, dst_id, num, vin.shape[0],
+                                                           weights.shape[0], output.shape[0])
+        products = typed_gemm(vin, weights, pair_seg, pair_src.shape[0], src_idx=pair_src)
+        output += _ops.spmm(ptr_d, rows_d, products, output.shape[0])
         return
+    perm, seg = rel_segment(types[:num].contiguous(), weights.shape[0])
+    src = perm if src_id is None else src_id[perm]
     dst = perm if dst_id is None else dst_id[perm]
     typed_gemm(vin, weights, seg, num, src_idx=src, dst_idx=dst, out=output, accumulate=True,
                atomic=atomic)
+
+
+_SCATTER_PAIR_CACHE = collections.OrderedDict()
+
+
+def _scatter_pairs(src_id, types, dst_id, num, n_src, num_rel, n_out):
+    """For output[dst[i]] += vin[src[i]] @ W[type[i]], i < num: the (type, source) pairs that
+    occur, sorted (pair_src [U], pair_seg [R+1] relation segments), and the CSR over
+    destinations whose entries are the pair rows of the destination's input rows
+    (ptr_d [n_out+1], rows_d [num]).  Cached per (src_id, types, dst_id) arrays."""
+    key = (src_id.data_ptr(), src_id._version, types.data_ptr(), types._version, dst_id.data_ptr(),
+           dst_id._version, num, n_src, num_rel, n_out, types.device.index)
+    hit = _SCATTER_PAIR_CACHE.get(key)
+    if hit is not None:
+        _SCATTER_PAIR_CACHE.move_to_end(key)
+        return hit[:4]
+    types, dst_id = types[:num], dst_id[:num].contiguous()
+    if num and (int(types.min()) < 0 or int(types.max()) >= num_rel):
+        raise ValueError("type ids must lie in [0, %d)" % num_rel)
+    if num and (int(src_id[:num].min()) < 0 or int(src_id[:num].max()) >= n_src):
+        raise ValueError("source ids must lie in [0, %d)" % n_src)
+    uniq, pair_of_row = torch.unique(types.to(torch.int64) * n_src + src_id[:num], sorted=True, return_inverse=True)
+    pair_src = (uniq % n_src).contiguous()
+    bounds = torch.arange(num_rel + 1, dtype=torch.int64, device=types.device) * n_src
+    pair_seg = torch.searchsorted(uniq, bounds).contiguous()
+    groups = _ops.dest_groups(dst_id, n_out)
+    rows_d = pair_of_row[groups.perm].contiguous()
+    _SCATTER_PAIR_CACHE[key] = (groups.ptr, rows_d, pair_src, pair_seg, (src_id, types, dst_id))
+    while len(_SCATTER_PAIR_CACHE) > 4:
+        _SCATTER_PAIR_CACHE.popitem(last=False)
+    return groups.ptr, rows_d, pair_src, pair_seg
 
 
 def typed_linear(vin, weights, output, types, in_feat_tile=32):
