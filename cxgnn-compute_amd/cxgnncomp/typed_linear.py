@@ -171,8 +171,11 @@ class TypedLinearS2DMMAggrOP:
 class TypedLinearS2DAggrMMOP(torch.autograd.Function):
     """RGCN layer as "aggregate per relation, then transform the centers" (:224-258;
     upstream: one masked aggregation and one torch.mm per relation).  The R masked
-    aggregations are one SpMM into rows keyed by (destination, relation) and the R
-    transforms one GEMM [n, R*K] x [R*K, N]; the backward pass mirrors it."""
+    aggregations are one SpMM into one row per (destination, relation) pair that owns an
+    edge, the R transforms one typed GEMM over those rows (relation segments), and every
+    destination sums the product rows of its pairs; the backward pass mirrors it.  When
+    nearly every pair owns an edge the rows are the dense [n, R] table instead and the
+    transform one GEMM [n, R*K] x [R*K, N]."""
 
     @staticmethod
     def forward(ctx, x, weights, ptr, idx, rel, num_center):
@@ -180,19 +183,30 @@ class TypedLinearS2DAggrMMOP(torch.autograd.Function):
         x = x.contiguous()
         weights = weights.contiguous()
         R, K, N = weights.shape
+        pg = _typed._pair_graph(ptr, idx, rel, n, x.shape[0], R)
+        ctx.n, ctx.pairs = n, pg.b_dst.shape[0] <= _typed.RGCN_PAIR_FILL_MAX * n * R
+        if ctx.pairs:
+            out, z = _typed._pairs_aggregate_first(pg, x, weights, idx, n)
+            ctx.pg = pg
+            ctx.save_for_backward(x, weights, z)
+            return out
         ptr_dr, idx_dr = _typed.dst_rel_graph(ptr, idx, rel, n, R)
         z = _ops.spmm(ptr_dr, idx_dr, x, n * R)                     # [n*R, K]
         ctx.save_for_backward(x, weights, ptr_dr, idx_dr, z)
-        ctx.n = n
         return torch.mm(z.view(n, R * K), weights.view(R * K, N))
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, weights, ptr_dr, idx_dr, z = ctx.saved_tensors
         grad_out = grad_out.contiguous()
-        R, K, N = weights.shape
         n = ctx.n
         grad_x = grad_w = None
+        if ctx.pairs:
+            x, weights, z = ctx.saved_tensors
+            grad_x, grad_w = _typed._pairs_aggregate_first_bwd(ctx.pg, weights, z, grad_out, x.shape[0],
+                                                               ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+            return grad_x, grad_w, None, None, None, None
+        x, weights, ptr_dr, idx_dr, z = ctx.saved_tensors
+        R, K, N = weights.shape
         if ctx.needs_input_grad[0]:
             gz = torch.mm(grad_out, weights.view(R * K, N).t())         # [n, R*K]
             g = _ops.transposed(ptr_dr, idx_dr, n * R, x.shape[0])

@@ -332,9 +332,12 @@ class _PairGraph:
       f_ptr [Uf+1], f_dst [E]  CSR over the forward pairs: destinations of a pair's edges;
       b_dst [Ub], b_seg [R+1]  destination of every backward pair, sorted by (relation, destination);
       ptr_src [n_src+1], b_row_rev [E]  reversed graph (rows = sources) and, per reversed edge,
-                               its backward pair row."""
+                               its backward pair row.
+    For the aggregate-first order (built on first use, _pair_graph_aggregate):
+      bp_ptr [Ub+1], bp_src [E]  CSR over the backward pairs: sources of a pair's edges;
+      dp_ptr [n+1], dp_rows [Ub] CSR over the destinations: the pair rows of a destination."""
     __slots__ = ("n_edges", "f_src", "f_seg", "f_row", "f_ptr", "f_dst", "b_dst", "b_seg", "ptr_src", "b_row_rev",
-                 "_keep")
+                 "b_row", "bp_ptr", "bp_src", "dp_ptr", "dp_rows", "_keep")
 
 
 _PAIR_CACHE = collections.OrderedDict()
@@ -367,11 +370,47 @@ def _pair_graph(ptr, idx, rel, n, n_src, R):
     tg = _ops.transposed(ptr, idx, n, n_src)
     pg.ptr_src = tg.ptr_t
     pg.b_row_rev = b_row[tg.perm].contiguous()
+    pg.b_row = b_row.contiguous()
+    pg.bp_ptr = pg.bp_src = pg.dp_ptr = pg.dp_rows = None
     pg._keep = (ptr, idx, rel)
     _PAIR_CACHE[key] = pg
     while len(_PAIR_CACHE) > _REL_CACHE_CAP:
         _PAIR_CACHE.popitem(last=False)
     return pg
+
+
+def _pair_graph_aggregate(pg, idx, n):
+    """The two extra CSRs of the aggregate-first order, kept with the pair graph."""
+    if pg.bp_ptr is None:
+        n_pairs = pg.b_dst.shape[0]
+        pg.bp_ptr, pg.bp_src, _ = _ops.coo_to_csr(idx[:pg.n_edges].contiguous(), pg.b_row, n_pairs)
+        rows = torch.arange(n_pairs, dtype=torch.int64, device=idx.device)
+        pg.dp_ptr, pg.dp_rows, _ = _ops.coo_to_csr(rows, pg.b_dst, n)
+    return pg
+
+
+def _pairs_aggregate_first(pg, x, weights, idx, n):
+    """out[d] = sum_r (sum of x over d's edges of relation r) @ W[r] on the (destination,
+    relation) pairs that own an edge: one SpMM into the pair rows (gathering rows of x), one
+    typed GEMM over the relation segments of pair rows, one SpMM that gives every destination
+    the sum of its pairs' product rows.  Returns (out, z) with z the aggregated pair rows."""
+    _pair_graph_aggregate(pg, idx, n)
+    n_pairs = pg.b_dst.shape[0]
+    z = _ops.spmm(pg.bp_ptr, pg.bp_src, x, n_pairs)                       # [Ub, K]
+    t = typed_gemm(z, weights, pg.b_seg, n_pairs)                         # [Ub, N]
+    return _ops.spmm(pg.dp_ptr, pg.dp_rows, t, n), z
+
+
+def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w):
+    """Gradients of _pairs_aggregate_first for x and the weights."""
+    n_pairs = pg.b_dst.shape[0]
+    gx = gw = None
+    if need_x:
+        gz = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, n_pairs, src_idx=pg.b_dst)
+        gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, gz, n_src)
+    if need_w:
+        gw = _weight_grad(z, grad_out, _edge_positions(n_pairs, z.device), pg.b_dst, pg.b_seg, weights.shape)
+    return gx, gw
 
 
 # The dense table is kept when nearly every (source, relation) pair owns an edge: its GEMM
@@ -413,6 +452,14 @@ class _RgcnFusedFunction(torch.autograd.Function):
             # pair that owns an edge instead of one per pair that could
             pg = _pair_graph(ptr, idx, rel, n, n_src, R)
             ctx.pairs = pg.f_src.shape[0] <= RGCN_PAIR_FILL_MAX * n_src * R
+        ctx.aggregate_first = ctx.pairs and K <= N and not force_dense     # gather the narrower rows
+        if ctx.aggregate_first:
+            out, z = _pairs_aggregate_first(pg, x, weights, idx, n)
+            if mean:
+                out *= _inv_degree(ptr, n).unsqueeze(1)
+            ctx.pg = pg
+            ctx.save_for_backward(x, weights, ptr, z)
+            return out
         if ctx.pairs:
             y = typed_gemm(x, weights, pg.f_seg, pg.f_src.shape[0], src_idx=pg.f_src)    # [Uf, N]
             out = _ops.spmm(ptr, pg.f_row, y, n, mean=mean)
@@ -454,6 +501,10 @@ class _RgcnFusedFunction(torch.autograd.Function):
         if ctx.mean:
             grad_out = grad_out * _inv_degree(ptr, n).unsqueeze(1)
         gx = gw = None
+        if ctx.aggregate_first:
+            gx, gw = _pairs_aggregate_first_bwd(ctx.pg, weights, ctx.saved_tensors[3], grad_out, n_src,
+                                                ctx.needs_input_grad[0], ctx.needs_input_grad[3])
+            return gx, None, None, gw, None, None, None, None
         if ctx.pairs:
             pg = ctx.pg
             if ctx.needs_input_grad[0]:

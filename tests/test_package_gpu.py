@@ -157,11 +157,16 @@ def test_typed_linear_e2e_and_s2e_ops():
     assert_close(_np(wg2.grad) / sc, w64.grad.numpy() / sc, RTOL, 2 * ATOL, "s2e grad w")
 
 
+@pytest.mark.parametrize("tables", ["dense", "pairs"])
 @pytest.mark.parametrize("opname", ["RGCNOP", "RGCNOP2", "RGCNOP3", "SeastarRGCNOP",
                                     "TypedLinearS2DMMAggrOP", "TypedLinearS2DAggrMMOP"])
-def test_rgcn_op_variants(opname):
+def test_rgcn_op_variants(opname, tables, monkeypatch):
+    """Every RGCN operator name, with the intermediate tables holding a row for every (node,
+    relation) pair and with a row only for the pairs that own an edge."""
     import cxgnncomp
     from cxgnncomp import graph_conv
+    from cxgnncomp_backend import _typed
+    monkeypatch.setattr(_typed, "RGCN_PAIR_FILL_MAX", 2.0 if tables == "pairs" else -1.0)
     cxgnncomp.set_timers()
     ptr, idx, etype = _hetero()
     n = ptr.shape[0] - 1
@@ -339,8 +344,11 @@ def test_conv_layers_forward_backward():
     check(cxgnncomp.MyGATConv(32, 64, heads=1), gat_ref(1, 64, False), (pc, ic, n, n, E), "GAT 1 head, out>in")
 
 
-def test_rgcn_conv_layer():
+@pytest.mark.parametrize("tables", ["dense", "pairs"])
+def test_rgcn_conv_layer(tables, monkeypatch):
     import cxgnncomp
+    from cxgnncomp_backend import _typed
+    monkeypatch.setattr(_typed, "RGCN_PAIR_FILL_MAX", 2.0 if tables == "pairs" else -1.0)
     cxgnncomp.set_timers()
     ptr, idx, etype = _hetero(n=1500, e=20000, R=4, seed=8)
     n = ptr.shape[0] - 1
