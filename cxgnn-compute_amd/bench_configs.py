@@ -255,6 +255,11 @@ def c3(iters):
            spmm_bytes(N, E, H * C, H) + 8 * E, 2 * E * H * C)
     report("c3", "sddmm_csr (edge-value grad) H=4 C=64", timeit(lambda: _ops.sddmm_csr(ptr, idx, x, g, N), iters),
            E * (4 * H * C + 8) + 4 * N * H * C + 4 * E * H, 2 * E * H * C)
+    gev = torch.empty(E, H, device="cuda")
+    report("c3", "spmm_multihead_bwd + edge-value grad in one pass (spmm_dot) H=4 C=64",
+           timeit(lambda: _ops.spmm_dot(gt.ptr_t, gt.idx_t, g, N, ev, gt.perm, x, gev), iters),
+           spmm_bytes(N, E, H * C, H) + 8 * E + 4 * N * H * C + 4 * E * H, 4 * E * H * C)
+    del gev
     dst = _ops.csr_row_ids(ptr, N, E)
     out = torch.empty(E, H, device="cuda")
     report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),

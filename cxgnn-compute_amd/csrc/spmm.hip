@@ -83,6 +83,11 @@ struct SpmmArgs {
   int64_t rel_stride;
   const int64_t* src_map;  // source row = src_map[source row]
   const int64_t* targets;  // row r is added (atomically) into out[targets[r]]
+  // per-edge dot products beside the aggregation (DOTG kernels only):
+  // dot_out[vrow(e), h] = <x[idx[e], h, :], dot_b[r, h, :]> for every edge e of row r
+  const float* dot_b;
+  int64_t ld_dot_b;
+  float* dot_out;
 };
 
 __device__ __forceinline__ void atomic_add_vec(float* p, float v) { unsafeAtomicAdd(p, v); }
@@ -96,9 +101,24 @@ __device__ __forceinline__ void atomic_add_vec(float* p, float4 v) {
 
 // WMODE: 0 = unweighted, 1 = one weight per edge (heads == 1), 2 = one weight
 // per edge and head (each lane's V columns lie in one head).
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int U>
+// Sum over `G` consecutive lanes (power of two, aligned); the group's first lane holds it.
+template <int G> __device__ __forceinline__ float lane_group_sum(float v) {
+#pragma unroll
+  for (int m = G / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, CXG_WAVE);
+  return v;
+}
+__device__ __forceinline__ float vdot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
+
+// DOTG > 0 (V == 4, whole column tiles, DOTG = channels / 4 lanes per head): the wave also
+// multiplies every gathered row with the row of `dot_b` that belongs to the output row and
+// stores the per-head sums at the edge's weight row -- the edge-value gradient of the
+// attention layer from the gathers of its input gradient.  The rows of dot_b are loaded
+// three output rows ahead, so a row change costs no wait.
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int U, int DOTG = 0>
 __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   using vec_t = typename Vec<V>::type;
+  constexpr int kDotHeads = DOTG > 0 ? CXG_WAVE / DOTG : 1;       // heads of one 256-float column tile
+  __shared__ __attribute__((aligned(16))) float s_dot[DOTG > 0 ? kWavesPerBlock : 1][DOTG > 0 ? CXG_WAVE * kDotHeads : 1];
   const int lane = lane_id();
   const int wave = uniform_i32(threadIdx.x >> 6);
   const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -141,8 +161,18 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   int head_of_lane = 0;
   if (WMODE == 2) head_of_lane = col / a.channels;
 
+  vec_t xr0 = vzero<V>(), xr1 = vzero<V>(), xr2 = vzero<V>(), xr3 = vzero<V>();
+  auto load_dot_row = [&](int64_t row) -> vec_t {
+    const int64_t rc = row < n_rows ? row : n_rows - 1;
+    return *reinterpret_cast<const vec_t*>(a.dot_b + rc * a.ld_dot_b + col);
+  };
+  if (DOTG > 0) {
+    xr0 = load_dot_row(r); xr1 = load_dot_row(r + 1); xr2 = load_dot_row(r + 2); xr3 = load_dot_row(r + 3);
+  }
+
   auto next_row = [&]() {
     ++r;
+    if (DOTG > 0) { xr0 = xr1; xr1 = xr2; xr2 = xr3; xr3 = load_dot_row(r + 3); }
     if (r - rbase == CXG_WAVE) {
       rbase = r;
       row_ends = load_row_ends(rbase);
@@ -221,8 +251,34 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
           }
           if (WMODE == 0) vadd(acc, v[u]);
           else vfma(acc, v[u], w[u]);
+          if constexpr (DOTG > 0) {
+            const float p = lane_group_sum<DOTG>(vdot4(v[u], xr0));
+            if ((lane & (DOTG - 1)) == 0) s_dot[wave][jj * kDotHeads + lane / DOTG] = p;
+          }
         }
       }
+    }
+    if constexpr (DOTG > 0) {
+      // the chunk's products leave through LDS: one vector store per edge and chunk instead of
+      // one 4-byte store per (edge, head) between the gathers (stores and loads of a wave
+      // complete in order, so every scattered store held up the next gathers)
+      __builtin_amdgcn_wave_barrier();
+      if (lane < cn) {
+        const int64_t vrow = PERM ? my_vrow : (e0 + c0 + lane);
+        float* dst = a.dot_out + vrow * a.heads + blockIdx.y * kDotHeads;
+        const float* src = &s_dot[wave][lane * kDotHeads];
+        if constexpr (kDotHeads == 8) {
+          *reinterpret_cast<float4*>(dst) = *reinterpret_cast<const float4*>(src);
+          *reinterpret_cast<float4*>(dst + 4) = *reinterpret_cast<const float4*>(src + 4);
+        } else if constexpr (kDotHeads == 4) {
+          *reinterpret_cast<float4*>(dst) = *reinterpret_cast<const float4*>(src);
+        } else if constexpr (kDotHeads == 2) {
+          *reinterpret_cast<float2*>(dst) = *reinterpret_cast<const float2*>(src);
+        } else {
+          dst[0] = src[0];
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
   }
 
@@ -511,7 +567,7 @@ Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
   return p;
 }
 
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT>
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0>
 int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t stream) {
   // Gathers in flight per wave.  Measured on MI355X (61.9M-edge power-law graph):
   // with 32 waves per CU the memory system is already saturated, and issuing more
@@ -535,7 +591,7 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
       if (hipGetDeviceProperties(&prop, 0) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
       if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-              &blocks, spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U>, kBlock, 0) != hipSuccess || blocks < 1)
+              &blocks, spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U, DOTG>, kBlock, 0) != hipSuccess || blocks < 1)
         blocks = 4;
       return (int64_t)blocks * kWavesPerBlock * cus;
     }();
@@ -548,7 +604,7 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   }
   dim3 grid((unsigned)ceil_div(n_spans_cap, kWavesPerBlock), (unsigned)n_ct, 1);
   dim3 block(kBlock, 1, 1);
-  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U>), grid, block, 0, stream, a);
+  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U, DOTG>), grid, block, 0, stream, a);
   CXG_LAUNCH_CHECK("spmm_span_kernel");
   hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, V, GUARD>), grid, block, 0, stream, a);
   CXG_LAUNCH_CHECK("spmm_fixup_kernel");
@@ -633,11 +689,18 @@ struct SpmmExt {
   const int64_t* targets = nullptr;
 };
 
+struct SpmmDot {
+  const float* b = nullptr;     // [n_rows, heads, channels], row stride ld_b
+  int64_t ld_b = 0;
+  float* out = nullptr;         // [n_val_rows, heads]
+};
+
 template <typename IdxT>
 int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_t* perm,
                 const float* x, int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
                 int64_t n_edges_cap, int heads, int channels, unsigned flags, void* workspace,
-                size_t workspace_bytes, void* stream, const SpmmExt* ext = nullptr) {
+                size_t workspace_bytes, void* stream, const SpmmExt* ext = nullptr,
+                const SpmmDot* dot = nullptr) {
   CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
   CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
   CXG_REQUIRE((int64_t)heads * channels <= (1 << 20), CXG_ERR_UNSUPPORTED, "row too wide");
@@ -666,6 +729,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
   a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0;
   a.src_map = nullptr; a.targets = nullptr;
+  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (ext) {
     CXG_REQUIRE(!val, CXG_ERR_UNSUPPORTED, "extended gather takes no edge weights");
@@ -674,6 +738,29 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
     a.src_map = ext->src_map; a.targets = ext->targets;
     if constexpr (sizeof(IdxT) == 8) return dispatch_shape<IdxT, 0, false, true>(a, plan.n_spans_cap, st);
     return set_error(CXG_ERR_UNSUPPORTED, "extended gather needs int64 indices");
+  }
+  if (dot) {
+    if constexpr (sizeof(IdxT) == 8) {
+      CXG_REQUIRE(val && dot->b && dot->out, CXG_ERR_ARG, "null val/dot_b/dot_out");
+      CXG_REQUIRE(dot->ld_b >= F, CXG_ERR_ARG, "row stride of dot_b smaller than row");
+      const uintptr_t align_bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)a.carry | (uintptr_t)dot->b |
+                                   (uintptr_t)(ldx * 4) | (uintptr_t)(ldo * 4) | (uintptr_t)(dot->ld_b * 4);
+      CXG_REQUIRE(F % 256 == 0 && (align_bits & 15) == 0 &&
+                      (channels == 32 || channels == 64 || channels == 128 || channels == 256),
+                  CXG_ERR_UNSUPPORTED, "spmm with dot products needs heads*channels %% 256 == 0, channels in "
+                  "{32, 64, 128, 256} and 16-byte aligned rows");
+      a.dot_b = dot->b; a.ld_dot_b = dot->ld_b; a.dot_out = dot->out;
+#define CXG_DOT(WM, GG)                                                                          \
+  return perm ? launch_spmm<IdxT, 4, false, WM, true, false, GG>(a, plan.n_spans_cap, st)          \
+              : launch_spmm<IdxT, 4, false, WM, false, false, GG>(a, plan.n_spans_cap, st)
+      if (heads == 1) { CXG_DOT(1, 64); }
+      if (channels == 32) { CXG_DOT(2, 8); }
+      if (channels == 64) { CXG_DOT(2, 16); }
+      if (channels == 128) { CXG_DOT(2, 32); }
+      CXG_DOT(2, 64);
+#undef CXG_DOT
+    }
+    return set_error(CXG_ERR_UNSUPPORTED, "spmm with dot products needs int64 indices");
   }
   if (!val) return dispatch_shape<IdxT, 0, false>(a, plan.n_spans_cap, st);
   if constexpr (sizeof(IdxT) == 8) {
@@ -719,6 +806,18 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx, const float* v
   if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
   return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
                                    heads, channels, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_weighted_dot_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                              const int64_t* val_perm, const float* x, int64_t ldx, float* out,
+                              int64_t ldo, const float* dot_b, int64_t ld_dot_b, float* dot_out,
+                              int64_t n_rows, int64_t n_edges_cap, int heads, int channels,
+                              unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
+  cxg::SpmmDot dot;
+  dot.b = dot_b; dot.ld_b = ld_dot_b; dot.out = dot_out;
+  return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
+                                   heads, channels, flags, workspace, workspace_bytes, stream, nullptr, &dot);
 }
 
 int cxg_spmm_ext_f32(const int64_t* ptr, const int64_t* idx, const float* x, int64_t ldx, float* out,

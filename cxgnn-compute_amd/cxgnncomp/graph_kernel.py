@@ -3,7 +3,8 @@ node features and the edge values (cxgnncomp/graph_kernel.py:5-36).
 
 forward   out[r,h,:] = sum_e val[e,h] * x[idx[e],h,:]
 backward  grad_x over the cached transposed CSR (upstream: atomic scatter),
-          grad_val[e,h] = <grad_out[row(e),h,:], x[idx[e],h,:]> by the CSR SDDMM.
+          grad_val[e,h] = <grad_out[row(e),h,:], x[idx[e],h,:]> by the CSR SDDMM, or, for
+          rows of 256 floats, by the same pass that computes grad_x.
 Upstream feeds the [N,H,C] grad_out to an SDDMM kernel that indexes it as [N,C]
 (src/cpp/src/sddmm_kernel.cu:17), which is wrong for H > 1; the per-head product
 is what the chain rule requires and what is computed here.
@@ -32,6 +33,15 @@ class SpMMValOP(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         grad_x = grad_val = None
         g = _ops.transposed(ptr, idx, ctx.n, x.shape[0])       # cached with the graph
+        if (ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and x.dim() == 3 and val.dim() == 2
+                and _ops.spmm_dot_supported(x.shape[1], x.shape[2]) and val.shape[0] == idx.shape[0]):
+            # both gradients from one pass over the reversed graph: the rows of grad_out gathered
+            # for grad_x are also multiplied with the row of x they are added into
+            grad_val = torch.empty_like(val)
+            if g.n_edges < val.shape[0]:
+                grad_val[g.n_edges:].zero_()
+            grad_x, grad_val = _ops.spmm_dot(g.ptr_t, g.idx_t, grad_out, x.shape[0], val, g.perm, x, grad_val)
+            return grad_x, None, None, grad_val, None
         if ctx.needs_input_grad[0]:
             # spmm_multihead_bwd adds into a zeroed tensor; writing the rows of the transposed
             # graph directly saves the fill and the read-back of the accumulation

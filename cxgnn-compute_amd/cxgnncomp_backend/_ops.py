@@ -114,6 +114,53 @@ def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, 
     return out
 
 
+def spmm_dot_supported(heads, channels):
+    """Shapes ``spmm_dot`` takes (the others use spmm and sddmm_csr)."""
+    return (heads * channels) % 256 == 0 and channels in (32, 64, 128, 256)
+
+
+def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out):
+    """Weighted multi-head SpMM that also stores, for every edge e of output row r,
+    dot_out[vrow(e), h] = <x[idx[e], h, :], dot_b[r, h, :]> (vrow(e) = val_perm[e], or e):
+    (out [n_rows, H, C], dot_out).  x [n_src, H, C], val [*, H], dot_b [>= n_rows, H, C],
+    dot_out [*, H] (the entries of the edges of the first n_rows rows are written)."""
+    lib = _lib.load()
+    _check_graph(ptr, idx, n_rows)
+    _req(x, "x", torch.float32, 3)
+    _req(val, "val", torch.float32, 2)
+    _req(dot_b, "dot_b", torch.float32, 3)
+    _req(dot_out, "dot_out", torch.float32, 2)
+    heads, channels = x.shape[1], x.shape[2]
+    if val.shape[1] != heads or dot_out.shape[1] != heads or tuple(dot_b.shape[1:]) != (heads, channels):
+        raise ValueError("head / channel counts of x %s, val %s, dot_b %s, dot_out %s differ"
+                         % (tuple(x.shape), tuple(val.shape), tuple(dot_b.shape), tuple(dot_out.shape)))
+    if dot_b.shape[0] < n_rows:
+        raise ValueError("dot_b has %d rows, %d needed" % (dot_b.shape[0], n_rows))
+    if val_perm is not None:
+        _req(val_perm, "val_perm", torch.int64, 1)
+        if val_perm.shape[0] < idx.shape[0]:
+            raise ValueError("val_perm shorter than idx")
+        if dot_out.shape[0] != val.shape[0]:
+            raise ValueError("dot_out must have a row per row of val")
+    elif val.shape[0] < idx.shape[0] or dot_out.shape[0] < idx.shape[0]:
+        raise ValueError("val / dot_out shorter than idx")
+    if not spmm_dot_supported(heads, channels):
+        raise ValueError("spmm_dot needs heads*channels %% 256 == 0 and channels in (32, 64, 128, 256)")
+    row = heads * channels
+    out = torch.empty((n_rows, heads, channels), dtype=torch.float32, device=x.device)
+    if n_rows == 0:
+        return out, dot_out
+    ws = _workspace(lib.cxg_spmm_workspace_bytes(idx.shape[0], row), x.device)
+    flags = SPMM_HINT_EXACT_EDGES if n_rows == ptr.shape[0] - 1 else 0
+    with torch.cuda.device(x.device):
+        st = lib.cxg_spmm_weighted_dot_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(), _lib.ptr(val_perm),
+                                           _lib.ptr(x), row, out.data_ptr(), row, _lib.ptr(dot_b), row,
+                                           dot_out.data_ptr(), n_rows, idx.shape[0], heads, channels, flags,
+                                           ws.data_ptr(), ws.numel(), _lib.current_stream(x.device))
+    _lib.check(st)
+    return out, dot_out
+
+
 # --------------------------------------------------------------------------- #
 # transposed-graph cache
 # --------------------------------------------------------------------------- #

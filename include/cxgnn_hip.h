@@ -96,6 +96,26 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx,
                           size_t workspace_bytes, void* stream);
 
 /*
+ * cxg_spmm_weighted_f32 that also leaves, for every edge e of output row r,
+ *   dot_out[vrow(e), h] = sum_c x[idx[e], h, c] * dot_b[r, h, c]
+ * from the same gathered rows.  Called on the transposed CSR with x = the gradient of the
+ * aggregated features, val / val_perm = the edge values and the transposition's edge
+ * permutation, dot_b = the layer's input features, it yields the input gradient AND the
+ * edge-value gradient of the multi-head weighted aggregation in one pass: the pair
+ * spmm_multihead_bwd + run_sddmm of SpMMValOP.backward (cxgnncomp/graph_kernel.py:20-37,
+ * src/cpp/src/spmm_host.cu:198-214, src/cpp/src/sddmm_host.cu:4-14).  dot_b is
+ * [n_rows, heads, channels] with row stride ld_dot_b, dot_out [n_val_rows, heads].
+ * Shapes: heads*channels a multiple of 256, channels in {32, 64, 128, 256}, 16-byte
+ * aligned rows (CXG_ERR_UNSUPPORTED otherwise: use the two separate calls).
+ */
+int cxg_spmm_weighted_dot_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                              const int64_t* val_perm, const float* x, int64_t ldx, float* out,
+                              int64_t ldo, const float* dot_b, int64_t ld_dot_b, float* dot_out,
+                              int64_t n_rows, int64_t n_edges_cap, int heads, int channels,
+                              unsigned flags, void* workspace, size_t workspace_bytes,
+                              void* stream);
+
+/*
  * Sum aggregation with optional extras, each enabled by a non-NULL pointer:
  *   mask      [E] bytes: edges whose byte is 0 are skipped; the byte of edge
  *             position e is mask[mask_perm ? mask_perm[e] : e];

@@ -277,3 +277,36 @@ def test_attention_logits_op_autograd():
         assert g.shape == r.shape
         scale = max(1.0, float(r.abs().max()))
         assert_close(_np(g) / scale, _np(r) / scale, 1e-4, 2e-5, "autograd")
+
+
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
+@pytest.mark.parametrize("shape", [(4, 64), (8, 32), (2, 128), (1, 256), (8, 64)])
+def test_spmm_with_edge_dot_products(kind, shape):
+    """cxg_spmm_weighted_dot_f32 on the transposed graph: the aggregation equals the plain
+    weighted SpMM bit for bit, and the per-edge products equal the CSR SDDMM of the original
+    graph (the oracle's), written at the original edge positions."""
+    from cxgnncomp_backend import _ops
+    H, C = shape
+    ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    torch.manual_seed(11)
+    xs = torch.randn(n, H, C) / 8
+    g = torch.randn(n, H, C) / 8
+    ev = torch.rand(E, H)
+    pc, ic = ptr.cuda(), idx.cuda()
+    tg = _ops.transposed(pc, ic, n, n)
+    announce("spmm_dot kind=%s H=%d C=%d" % (kind, H, C))
+    dot = torch.full((E, H), float("nan"), device="cuda")
+    gx, dot = _ops.spmm_dot(tg.ptr_t, tg.idx_t, g.cuda(), n, ev.cuda(), tg.perm, xs.cuda(), dot)
+    want_gx = _ops.spmm(tg.ptr_t, tg.idx_t, g.cuda(), n, val=ev.cuda(), val_perm=tg.perm)
+    torch.cuda.synchronize()
+    assert torch.equal(gx, want_gx)
+    rows = np.repeat(np.arange(n), np.diff(ptr.numpy()))
+    ref = oracle.sddmm(idx.numpy(), rows, xs.numpy(), g.numpy())
+    assert_close(_np(dot), ref.reshape(E, H), RTOL, ATOL, "edge dot products")
+    # untransposed form (no permutation): products land at the edge's own position
+    dot2 = torch.empty(E, H, device="cuda")
+    out2, dot2 = _ops.spmm_dot(pc, ic, xs.cuda(), n, ev.cuda(), None, g.cuda(), dot2)
+    assert torch.equal(out2, _ops.spmm(pc, ic, xs.cuda(), n, val=ev.cuda()))
+    assert_close(_np(dot2), ref.reshape(E, H), RTOL, ATOL, "edge dot products, CSR order")
