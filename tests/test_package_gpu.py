@@ -530,3 +530,26 @@ def test_gat_layer_on_a_row_prefix(concat):
     for k, v in layer.named_parameters():
         sc = max(1.0, float(P[k].grad.abs().max()))
         assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "grad " + k)
+
+
+@pytest.mark.parametrize("opname", ["RGCNOP", "RGCNOP2", "TypedLinearS2DSort"])
+def test_rgcn_ops_on_a_graph_without_edges(opname):
+    """No edge at all: zeros out, zero gradients, no launch on empty pair tables."""
+    import cxgnncomp
+    from cxgnncomp import graph_conv
+    cxgnncomp.set_timers()
+    n, K, N, R = 70, 16, 8, 3
+    ptr = torch.zeros(n + 1, dtype=torch.int64).cuda()
+    idx = torch.zeros(0, dtype=torch.int64).cuda()
+    etype = torch.zeros(0, dtype=torch.int32).cuda()
+    x = torch.randn(n, K).cuda().requires_grad_(True)
+    w = torch.randn(R, K, N).cuda().requires_grad_(True)
+    announce("%s without edges" % opname)
+    if opname == "TypedLinearS2DSort":
+        out = cxgnncomp.TypedLinearS2DSort(x, w, ptr, idx, etype, n)
+    else:
+        out = getattr(graph_conv, opname).apply(x, w, ptr, idx, etype, n)
+    out.sum().backward()
+    torch.cuda.synchronize()
+    assert out.shape == (n, N) and float(out.detach().abs().max()) == 0.0
+    assert float(x.grad.abs().max()) == 0.0 and float(w.grad.abs().max()) == 0.0
