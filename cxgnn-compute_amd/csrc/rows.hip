@@ -40,6 +40,29 @@ __global__ __launch_bounds__(kBlock) void rows_kernel(const float* __restrict__ 
   }
 }
 
+// Rows of 1, 2, 4 or 8 floats: one row per thread as one (or two) vector accesses -- the
+// stores of a wave are contiguous, the loads are the random part.  A wave per row would
+// leave 60 of its 64 lanes idle on such rows.
+template <int W>
+__global__ __launch_bounds__(kBlock) void narrow_rows_gather_kernel(const float* __restrict__ in,
+                                                                    const int64_t* __restrict__ sel,
+                                                                    float* __restrict__ out, int64_t n) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= n) return;
+  const int64_t t = sel[e];
+  if constexpr (W == 1) {
+    out[e] = in[t];
+  } else if constexpr (W == 2) {
+    reinterpret_cast<float2*>(out)[e] = reinterpret_cast<const float2*>(in)[t];
+  } else if constexpr (W == 4) {
+    reinterpret_cast<float4*>(out)[e] = reinterpret_cast<const float4*>(in)[t];
+  } else {
+    const float4 a = reinterpret_cast<const float4*>(in)[2 * t], b = reinterpret_cast<const float4*>(in)[2 * t + 1];
+    reinterpret_cast<float4*>(out)[2 * e] = a;
+    reinterpret_cast<float4*>(out)[2 * e + 1] = b;
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void head_sum_kernel(const float* __restrict__ in,
                                                           float* __restrict__ out, int64_t n,
                                                           int heads, int channels) {
@@ -76,6 +99,17 @@ int cxg_gather_rows_f32(const float* in, const int64_t* sel, float* out, int64_t
   CXG_REQUIRE(n_rows_out >= 0 && feat >= 1, CXG_ERR_ARG, "bad n_rows/feat");
   if (n_rows_out == 0) return CXG_OK;
   CXG_REQUIRE(in && sel && out, CXG_ERR_ARG, "null pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const bool aligned = (((uintptr_t)in | (uintptr_t)out) & (uintptr_t)(feat >= 4 ? 15 : 4 * feat - 1)) == 0;
+  if ((feat == 1 || feat == 2 || feat == 4 || feat == 8) && aligned) {
+    const dim3 grid((unsigned)cxg::ceil_div(n_rows_out, cxg::kBlock)), block(cxg::kBlock);
+    if (feat == 1) hipLaunchKernelGGL(cxg::narrow_rows_gather_kernel<1>, grid, block, 0, st, in, sel, out, n_rows_out);
+    else if (feat == 2) hipLaunchKernelGGL(cxg::narrow_rows_gather_kernel<2>, grid, block, 0, st, in, sel, out, n_rows_out);
+    else if (feat == 4) hipLaunchKernelGGL(cxg::narrow_rows_gather_kernel<4>, grid, block, 0, st, in, sel, out, n_rows_out);
+    else hipLaunchKernelGGL(cxg::narrow_rows_gather_kernel<8>, grid, block, 0, st, in, sel, out, n_rows_out);
+    CXG_LAUNCH_CHECK("narrow_rows_gather_kernel");
+    return CXG_OK;
+  }
   const int64_t waves = cxg::ceil_div(n_rows_out, cxg::kRowsPerWave);
   hipLaunchKernelGGL(cxg::rows_kernel<false>, dim3((unsigned)cxg::ceil_div(waves * CXG_WAVE, cxg::kBlock)),
                      dim3(cxg::kBlock), 0, reinterpret_cast<hipStream_t>(stream), in, sel, out,

@@ -310,3 +310,17 @@ def test_spmm_with_edge_dot_products(kind, shape):
     out2, dot2 = _ops.spmm_dot(pc, ic, xs.cuda(), n, ev.cuda(), None, g.cuda(), dot2)
     assert torch.equal(out2, _ops.spmm(pc, ic, xs.cuda(), n, val=ev.cuda()))
     assert_close(_np(dot2), ref.reshape(E, H), RTOL, ATOL, "edge dot products, CSR order")
+
+
+@pytest.mark.parametrize("feat", [1, 2, 4, 8, 3, 16, 100])
+def test_gather_rows_all_widths(feat):
+    """out[e] = in[sel[e]]: the one-thread-per-row path for rows of 1, 2, 4, 8 floats and the
+    wave-per-row path for the others, bit-exact."""
+    from cxgnncomp_backend import _ops
+    g0 = torch.Generator().manual_seed(feat)
+    inp = torch.randn(5000, feat, generator=g0)
+    sel = torch.randint(0, 5000, (70001,), generator=g0)
+    announce("gather_rows feat=%d" % feat)
+    out = _ops.gather_rows(inp.cuda(), sel.cuda())
+    assert torch.equal(out.cpu(), inp[sel])
+    assert _ops.gather_rows(inp.cuda(), sel[:0].cuda()).shape == (0, feat)
