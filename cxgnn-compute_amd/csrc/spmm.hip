@@ -574,7 +574,9 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   // than one row gather per wave at a time only lengthens the queues and lowers
   // the L2 hit rate (F=128: 16 in flight 5.56 ms, 8: 4.94, 4: 4.51, 1: 4.31 ms).
   // 16-byte-per-lane gathers (V == 4) are flat from 1 to 8 and best at 8.
-  constexpr int U = (V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U;
+  // With the per-edge dot products four in flight are best: 62 registers instead of 80 keep eight
+  // waves per SIMD resident (12.7 -> 11.5 ms on the GAT graph; 16 in flight: 14.5 ms).
+  constexpr int U = DOTG > 0 ? 4 : ((V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U);
   const int tile = CXG_WAVE * V;
   const int64_t n_ct = ceil_div(a_in.F, tile);
   SpmmArgs<IdxT> a = a_in;
