@@ -487,15 +487,17 @@ def test_sage_layer_on_a_row_prefix(widths):
         assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "frozen input, grad " + k)
 
 
+@pytest.mark.parametrize("heads_channels", [(4, 8), (4, 64)])
 @pytest.mark.parametrize("concat", [True, False])
-def test_gat_layer_on_a_row_prefix(concat):
+def test_gat_layer_on_a_row_prefix(concat, heads_channels):
     """MyGATConv (several heads, one autograd node on CUDA) on a sampled-batch layer: num_dst
     destination rows over num_src source rows of a longer x; output and every gradient against
     the float64 composition of the upstream expressions."""
     import cxgnncomp
     cxgnncomp.set_timers()               # MyGATConv brackets its phases with TimerOP, as upstream
     torch.manual_seed(6)
-    n_all, n_src, n_dst, fin, H, C = 700, 600, 200, 24, 4, 8
+    n_all, n_src, n_dst, fin = 700, 600, 200, 24
+    H, C = heads_channels       # 4 x 64 = 256 floats per row: the backward pass with the fused edge products
     deg = torch.randint(0, 12, (n_dst,))
     deg[3] = 0
     ptr = torch.zeros(n_dst + 1, dtype=torch.int64)
