@@ -88,6 +88,7 @@ struct SpmmArgs {
   const float* dot_b;
   int64_t ld_dot_b;
   float* dot_out;
+  const float* bias;       // [F] added to every output row, or null
 };
 
 __device__ __forceinline__ void atomic_add_vec(float* p, float v) { unsafeAtomicAdd(p, v); }
@@ -195,6 +196,9 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
       if (a.mean) {
         const int deg = cur_end - cur_start;
         if (deg > 0) vscale(acc, 1.0f / (float)deg);
+      }
+      if (a.bias) {
+        if (col_ok) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
       }
       if (a.accumulate) {
         if (col_ok) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
@@ -402,6 +406,9 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
         const int deg = cur_end - cur_start;
         if (deg > 0) vscale(acc, 1.0f / (float)deg);
       }
+      if (a.bias) {
+        if (writer) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
+      }
       if (a.accumulate) {
         if (writer) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
       }
@@ -537,6 +544,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   }
   if (a.mean) vscale(acc, 1.0f / (float)(row_end - row_begin));
   float* dst = a.out + t * a.ldo;
+  if (a.bias) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
   if (a.accumulate) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
   *reinterpret_cast<vec_t*>(dst + col) = acc;
 }
@@ -617,7 +625,7 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
 // Returns 1 if it launched, 0 if the shape is not narrow, < 0 on a launch error.
 template <typename IdxT, int WMODE, bool PERM>
 int launch_group(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t stream) {
-  const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry |
+  const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry | (uintptr_t)a.bias |
                                (uintptr_t)(a.ldx * 4) | (uintptr_t)(a.ldo * 4) | (uintptr_t)(a.F * 4);
   const int unit = (WMODE == 2) ? a.channels : a.F;
   int v = 1;
@@ -661,7 +669,7 @@ int dispatch_shape(const SpmmArgs<IdxT>& a, int64_t n_spans_cap, hipStream_t str
   // widest vector that divides the row (and the head, for per-head weights) and
   // keeps every access aligned; among those the one needing the fewest column
   // tiles, ties to the narrower vector (more lanes busy).
-  const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry |
+  const uintptr_t align_bits = (uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.carry | (uintptr_t)a.bias |
                                (uintptr_t)(a.ldx * 4) | (uintptr_t)(a.ldo * 4) | (uintptr_t)(a.F * 4);
   int unit = (WMODE == 2) ? a.channels : a.F;
   int best_v = 1;
@@ -702,7 +710,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
                 const float* x, int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
                 int64_t n_edges_cap, int heads, int channels, unsigned flags, void* workspace,
                 size_t workspace_bytes, void* stream, const SpmmExt* ext = nullptr,
-                const SpmmDot* dot = nullptr) {
+                const SpmmDot* dot = nullptr, const float* bias = nullptr) {
   CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
   CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
   CXG_REQUIRE((int64_t)heads * channels <= (1 << 20), CXG_ERR_UNSUPPORTED, "row too wide");
@@ -732,6 +740,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0;
   a.src_map = nullptr; a.targets = nullptr;
   a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr;
+  a.bias = bias;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (ext) {
     CXG_REQUIRE(!val, CXG_ERR_UNSUPPORTED, "extended gather takes no edge weights");
@@ -746,6 +755,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
       CXG_REQUIRE(val && dot->b && dot->out, CXG_ERR_ARG, "null val/dot_b/dot_out");
       CXG_REQUIRE(dot->ld_b >= F, CXG_ERR_ARG, "row stride of dot_b smaller than row");
       const uintptr_t align_bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)a.carry | (uintptr_t)dot->b |
+                                   (uintptr_t)a.bias |
                                    (uintptr_t)(ldx * 4) | (uintptr_t)(ldo * 4) | (uintptr_t)(dot->ld_b * 4);
       CXG_REQUIRE(F % 256 == 0 && (align_bits & 15) == 0 &&
                       (channels == 32 || channels == 64 || channels == 128 || channels == 256),
@@ -808,6 +818,18 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx, const float* v
   if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
   return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
                                    heads, channels, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_weighted_bias_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                               const int64_t* val_perm, const float* x, int64_t ldx, const float* bias,
+                               float* out, int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int heads,
+                               int channels, unsigned flags, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
+  CXG_REQUIRE(!(bias && (flags & CXG_SPMM_MEAN)), CXG_ERR_ARG, "bias cannot be combined with mean");
+  return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
+                                   heads, channels, flags, workspace, workspace_bytes, stream, nullptr, nullptr,
+                                   bias);
 }
 
 int cxg_spmm_weighted_dot_f32(const int64_t* ptr, const int64_t* idx, const float* val,

@@ -454,10 +454,13 @@ class GatLayerOP(torch.autograd.Function):
         xs = F.linear(x[:num_src], w).view(-1, H, C)
         a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
         ev, mask = _ops.edge_softmax_fwd(ptr, idx, a_dst, a_src, num_edge, slope)
-        out = _ops.spmm(ptr, idx, xs, num_dst, val=ev)
-        out = out.view(-1, H * C) if concat else out.mean(dim=1)
-        if bias is not None:
-            out.add_(bias)
+        if concat:
+            # the bias goes into the aggregation's row stores
+            out = _ops.spmm(ptr, idx, xs, num_dst, val=ev, bias=bias).view(-1, H * C)
+        else:
+            out = _ops.spmm(ptr, idx, xs, num_dst, val=ev).mean(dim=1)
+            if bias is not None:
+                out.add_(bias)
         ctx.save_for_backward(x, w, att_src, att_dst, xs, ev, mask, ptr, idx)
         ctx.dims = (num_dst, num_src, H, C, concat, float(slope), bias is not None)
         return out

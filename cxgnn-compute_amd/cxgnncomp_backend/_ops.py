@@ -49,11 +49,12 @@ def _check_graph(ptr, idx, n_rows, dtype=torch.int64):
         raise ValueError("ptr and idx are on different devices")
 
 
-def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, accumulate=False):
+def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, accumulate=False, bias=None):
     """out[r] = sum_{e in row r} (val[vrow(e)] *) x[idx[e]] for r < n_rows.
 
     x is [n_src, F] or [n_src, H, C]; val (optional) is [E] or [E, H].  Returns
-    a new [n_rows, ...] tensor unless ``out`` is given.
+    a new [n_rows, ...] tensor unless ``out`` is given.  ``bias`` (with val, without mean:
+    one float per column of a row) is added to every output row as it is stored.
     """
     lib = _lib.load()
     int32 = ptr.dtype == torch.int32
@@ -91,6 +92,8 @@ def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, 
             raise ValueError("out has shape %s, expected %s" % (tuple(out.shape), out_shape))
     if n_rows == 0:
         return out
+    if bias is not None and val is None:
+        raise ValueError("bias needs edge values")
     n_cap = idx.shape[0]
     ws_bytes = lib.cxg_spmm_workspace_bytes(n_cap, row)
     ws = _workspace(ws_bytes, x.device)
@@ -106,10 +109,19 @@ def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, 
         else:
             if int32:
                 raise ValueError("weighted SpMM needs int64 ptr/idx")
-            st = lib.cxg_spmm_weighted_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(),
-                                           _lib.ptr(val_perm), _lib.ptr(x), row, out.data_ptr(), row,
-                                           n_rows, n_cap, heads, channels, flags, ws.data_ptr(),
-                                           ws.numel(), stream)
+            if bias is not None:
+                _req(bias, "bias", torch.float32, 1)
+                if bias.shape[0] != row or mean:
+                    raise ValueError("bias needs %d floats and no mean" % row)
+                st = lib.cxg_spmm_weighted_bias_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(),
+                                                    _lib.ptr(val_perm), _lib.ptr(x), row, bias.data_ptr(),
+                                                    out.data_ptr(), row, n_rows, n_cap, heads, channels, flags,
+                                                    ws.data_ptr(), ws.numel(), stream)
+            else:
+                st = lib.cxg_spmm_weighted_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(),
+                                               _lib.ptr(val_perm), _lib.ptr(x), row, out.data_ptr(), row,
+                                               n_rows, n_cap, heads, channels, flags, ws.data_ptr(),
+                                               ws.numel(), stream)
     _lib.check(st)
     return out
 

@@ -96,6 +96,18 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx,
                           size_t workspace_bytes, void* stream);
 
 /*
+ * cxg_spmm_weighted_f32 with bias[heads*channels] added to every output row as it is
+ * stored (NULL: none; not with CXG_SPMM_MEAN): the `out + self.bias` that follows the
+ * aggregation in MyGATConv.forward_many (cxgnncomp/graph_conv.py:488-494) without a second
+ * pass over the output.
+ */
+int cxg_spmm_weighted_bias_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                               const int64_t* val_perm, const float* x, int64_t ldx,
+                               const float* bias, float* out, int64_t ldo, int64_t n_rows,
+                               int64_t n_edges_cap, int heads, int channels, unsigned flags,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * cxg_spmm_weighted_f32 that also leaves, for every edge e of output row r,
  *   dot_out[vrow(e), h] = sum_c x[idx[e], h, c] * dot_b[r, h, c]
  * from the same gathered rows.  Called on the transposed CSR with x = the gradient of the

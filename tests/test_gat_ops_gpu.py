@@ -324,3 +324,25 @@ def test_gather_rows_all_widths(feat):
     out = _ops.gather_rows(inp.cuda(), sel.cuda())
     assert torch.equal(out.cpu(), inp[sel])
     assert _ops.gather_rows(inp.cuda(), sel[:0].cuda()).shape == (0, feat)
+
+
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
+@pytest.mark.parametrize("shape", [(4, 64), (2, 32), (1, 40), (8, 64)])
+def test_weighted_spmm_with_bias(kind, shape):
+    """cxg_spmm_weighted_bias_f32: the bias reaches every row exactly once -- rows that end
+    inside a span, rows completed by the fix-up kernel (one_hub) and empty rows -- so the result
+    equals the plain weighted SpMM plus the bias bit for bit."""
+    from cxgnncomp_backend import _ops
+    H, C = shape
+    ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    torch.manual_seed(13)
+    x = (torch.randn(n, H, C) / 8).cuda()
+    ev = torch.rand(E, H).cuda()
+    bias = torch.randn(H * C).cuda()
+    announce("spmm weighted + bias kind=%s H=%d C=%d" % (kind, H, C))
+    got = _ops.spmm(ptr.cuda(), idx.cuda(), x, n, val=ev, bias=bias)
+    want = _ops.spmm(ptr.cuda(), idx.cuda(), x, n, val=ev) + bias.view(1, H, C)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
