@@ -60,7 +60,8 @@ SIGNATURES = {
     "cxg_csr_row_ids_i32": (_I32, [_P, _I64, _I64, _P, _P]),
     "cxg_segment_gather_sum_workspace_bytes": (_SZ, [_I64, _I32]),
     "cxg_segment_gather_sum_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _P, _SZ, _P]),
-    "cxg_gspmm_i32_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "cxg_gspmm_workspace_bytes": (_SZ, [_I64, _I32]),
+    "cxg_gspmm_i32_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _I32, _P, _SZ, _P]),
     "cxg_topo_sort_host_i64": (_I64, [_P, _P, _P, _I64, _P]),
     "cxg_scan_workspace_bytes": (_SZ, [_I64]),
     "cxg_neighbor_group_plan_i64": (_I32, [_P, _I64, _I64, _P, _P, _SZ, _P]),

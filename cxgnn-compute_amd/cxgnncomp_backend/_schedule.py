@@ -180,9 +180,12 @@ def _gspmm(rowptr, colind, val, b, red, comp):
         if val.shape[0] < colind.shape[0]:
             raise ValueError("A_csrVal shorter than A_colind")
     out = torch.empty((n, b.shape[1]), dtype=torch.float32, device=b.device)
+    ws_bytes = lib.cxg_gspmm_workspace_bytes(colind.shape[0], b.shape[1])
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=b.device) if ws_bytes else None
     with torch.cuda.device(b.device):
         st = lib.cxg_gspmm_i32_f32(rowptr.data_ptr(), _lib.ptr(colind), _lib.ptr(val), _lib.ptr(b), _lib.ptr(out),
-                                   n, b.shape[1], int(red), int(comp), _lib.current_stream(b.device))
+                                   n, colind.shape[0], b.shape[1], int(red), int(comp), _lib.ptr(ws), ws_bytes,
+                                   _lib.current_stream(b.device))
     _lib.check(st)
     return out
 

@@ -438,12 +438,19 @@ int cxg_pad_rel_i64(int64_t* rel, int64_t* idx, const int64_t* count, int thres,
  * 3 b/val (the enum values of src/cpp/include/dgsparse.h:13-14); val == NULL: the
  * operand is b itself and compute_op is ignored.  A non-empty row's accumulator
  * starts at 0 / (float)INT_MIN / (float)INT_MAX / 0, empty rows give 0, mean
- * divides by the row length.  Replaces GSpMM_u / GSpMM_u_e
- * (src/cpp/python_bindings/binding.cpp:87-107, src/cpp/src/dgsparse.cu:444-474).
+ * divides by the row length.  n_edges is the length of colind (at least
+ * rowptr[n_rows]); workspace holds cxg_gspmm_workspace_bytes(n_edges, feat) bytes:
+ * rows of more than 512 edges are cut at the multiples of 512 in the edge array,
+ * one wave per piece leaves a partial row there, and the row's own wave folds
+ * them in edge order (results do not depend on the schedule).  Replaces
+ * GSpMM_u / GSpMM_u_e (src/cpp/python_bindings/binding.cpp:87-107,
+ * src/cpp/src/dgsparse.cu:444-474).
  */
+size_t cxg_gspmm_workspace_bytes(int64_t n_edges, int feat);
 int cxg_gspmm_i32_f32(const int32_t* rowptr, const int32_t* colind, const float* val,
-                      const float* b, float* out, int64_t n_rows, int feat, int reduce_op,
-                      int compute_op, void* stream);
+                      const float* b, float* out, int64_t n_rows, int64_t n_edges, int feat,
+                      int reduce_op, int compute_op, void* workspace, size_t workspace_bytes,
+                      void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Scheduling helpers as device index work (bit-exact)                          */

@@ -73,6 +73,53 @@ def test_gspmm_u_e(n_dst, n_src, e, feat, hub, red, comp):
         assert_close(_np(got) / sc, want / sc, RTOL, ATOL, "GSpMM_u_e %s %s" % (red, comp))
 
 
+def _long_row_graph(n_src, lead, rng):
+    """Rows of more than 512 edges next to each other, at both ends of the edge array, with
+    lengths at and around the piece size, short and empty rows in between; `lead` unused
+    column ids in front of the first row (rowptr[0] = lead)."""
+    degs = [1300, 513, 512, 0, 0, 2049, 3, 511, 1024, 1025, 0, 7, 700]
+    ptr = (np.concatenate([[0], np.cumsum(degs)]) + lead).astype(np.int32)
+    idx = rng.integers(0, n_src, int(ptr[-1])).astype(np.int32)
+    return ptr, idx
+
+
+@pytest.mark.parametrize("feat", [4, 7, 100, 300])
+@pytest.mark.parametrize("lead", [0, 37])
+@pytest.mark.parametrize("red,comp", [("MAX", None), ("MIN", "SUB"), ("SUM", "ADD"), ("MEAN", "DIV"), ("SUM", "MUL")])
+def test_gspmm_rows_cut_into_pieces(feat, lead, red, comp):
+    """Rows above 512 edges go through per-piece partial rows: same answers as the oracle,
+    max / min exactly, and the same bits on a second call."""
+    import cxgnncomp_backend as B
+    rng = np.random.default_rng(feat + lead)
+    n_src = 500
+    ptr, idx = _long_row_graph(n_src, lead, rng)
+    scale = 1.0 / np.sqrt(2049.0) if red == "SUM" else 1.0
+    b = (rng.standard_normal((n_src, feat)) * scale).astype(np.float32)
+    val = None
+    if comp is not None:
+        val = ((rng.random(idx.shape[0]) + 0.5) * rng.choice([-1.0, 1.0], idx.shape[0])).astype(np.float32)
+        if red == "SUM" and comp == "ADD":
+            val = (val * scale).astype(np.float32)
+    rop = getattr(B.REDUCEOP, red)
+    announce("GSpMM long rows %s %s F=%d lead=%d" % (red, comp, feat, lead))
+    tp, ti, tb = torch.from_numpy(ptr).cuda(), torch.from_numpy(idx).cuda(), torch.from_numpy(b).cuda()
+    if comp is None:
+        run = lambda: B.GSpMM_u(tp, ti, tb, rop)
+        want = oracle.gspmm(ptr, idx, b, int(rop))
+    else:
+        cop = getattr(B.COMPUTEOP, comp)
+        tv = torch.from_numpy(val).cuda()
+        run = lambda: B.GSpMM_u_e(tp, ti, tv, tb, rop, cop)
+        want = oracle.gspmm(ptr, idx, b, int(rop), int(cop), val=val)
+    got = run()
+    if red in ("MAX", "MIN"):
+        assert np.array_equal(_np(got), want)
+    else:
+        sc = max(1.0, float(np.abs(want).max()))
+        assert_close(_np(got) / sc, want / sc, RTOL, ATOL, "GSpMM long rows %s %s" % (red, comp))
+    assert torch.equal(run(), got)
+
+
 def test_gspmm_enum_values_and_errors():
     import cxgnncomp_backend as B
     assert [int(B.REDUCEOP.SUM), int(B.REDUCEOP.MAX), int(B.REDUCEOP.MIN), int(B.REDUCEOP.MEAN)] == [0, 1, 2, 3]
