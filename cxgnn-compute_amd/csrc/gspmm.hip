@@ -131,9 +131,9 @@ __global__ __launch_bounds__(kBlock) void gspmm_long_rows_kernel(
   const int64_t piece = (int64_t)blockIdx.x * (kBlock / CXG_WAVE) + uniform_i32(threadIdx.x >> 6);
   if (piece >= n_pieces) return;
   const int first = rowptr[0], last = rowptr[n_rows];
-  int a = (int)(piece * kLongRow), z = a + kLongRow;
-  a = a < first ? first : a;
-  z = z > last ? last : z;
+  const int64_t a64 = piece * kLongRow, z64 = a64 + kLongRow;     // z64 may pass 2^31 in the last piece
+  const int a = a64 < first ? first : (int)a64;
+  const int z = z64 > last ? last : (int)z64;
   if (a >= z) return;
   const int col = (blockIdx.y * L + lane % L) * V;
   const bool col_ok = col < feat;

@@ -113,7 +113,7 @@ def main():
         "out": [[6.0, 2.0], [3.0, 4.0], [18.0, 10.0]],
     }
 
-    # --- byte/flop arithmetic held in the reference's notebooks / survey -------------
+    # --- byte/flop arithmetic held in the reference's notebooks ----------------------
     fx["arithmetic"] = {"mm_flops_test_dup": [128, 256, 2332486, 128 * 256 * 2332486],
                         "expected_mm_flops": 76430901248}
 
