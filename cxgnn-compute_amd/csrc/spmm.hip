@@ -75,7 +75,8 @@ struct SpmmArgs {
   int64_t exact_edges;     // > 0: the caller vouches for this edge count (span-length hint)
   int mean, accumulate;
   float* carry;            // [n_spans_cap][2][F]: head partial, tail partial
-  int64_t* tail_row;       // [n_spans_cap]: row whose tail partial the span holds, or -1
+  int64_t* tail_row;       // [n_spans_cap][3]: row whose tail partial the span holds, or -1; then the
+                           // run [begin, end) of rows without edges the span leaves to the fix-up kernel
   // extended gather (EXT kernels only); every pointer may be null
   const uint8_t* mask;     // skip edges whose mask byte is 0
   const int64_t* mask_perm;// mask index of edge position (null: the position itself)
@@ -171,19 +172,48 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     xr0 = load_dot_row(r); xr1 = load_dot_row(r + 1);
   }
 
-  auto next_row = [&]() {
+  auto store_vec = [&](float* dst, vec_t v) {
+    if (col_ok) *reinterpret_cast<vec_t*>(dst + col) = v;
+  };
+  // What finish_row leaves in a row without edges.
+  auto store_empty_row = [&](int64_t row) {
+    if ((EXT && a.targets) || (a.accumulate && !a.bias) || !col_ok) return;
+    float* dst = a.out + row * a.ldo;
+    vec_t z = vzero<V>();
+    if (a.bias) vadd(z, *reinterpret_cast<const vec_t*>(a.bias + col));
+    if (a.accumulate) vadd(z, *reinterpret_cast<const vec_t*>(dst + col));
+    *reinterpret_cast<vec_t*>(dst + col) = z;
+  };
+  int64_t run_begin = 0, run_end = 0;
+  // `own`: the rows without edges that follow the finished row belong to this span.
+  auto next_row = [&](bool own) {
     ++r;
     if (DOTG > 0) { xr0 = xr1; xr1 = load_dot_row(r + 1); }
     if (r - rbase == CXG_WAVE) {
       rbase = r;
       row_ends = load_row_ends(rbase);
+      if constexpr (DOTG == 0) {
+        // A long run of rows without edges (the seed rows of a sampled batch in the reversed
+        // graph): walked row by row, every 64 rows cost a load of the next row ends that first
+        // waits for the 64 stores before it (1024 such rows: 125 us), and one wave keeps at most
+        // 64 stores in flight.  When the whole window is empty, find the end of the run with one
+        // search and leave its rows to the fix-up kernel, where 64 waves share them.
+        if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) {
+          const int64_t q = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + cur_end + 1);
+          if (run_end == run_begin) {         // the first such run: the fix-up waves share it
+            run_begin = r;
+            run_end = q;
+          } else {
+            for (int64_t row = r; row < q; ++row) store_empty_row(row);
+          }
+          r = rbase = q;
+          row_ends = load_row_ends(rbase);
+        }
+      }
     }
     cur_start = cur_end;
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
     is_head = false;
-  };
-  auto store_vec = [&](float* dst, vec_t v) {
-    if (col_ok) *reinterpret_cast<vec_t*>(dst + col) = v;
   };
   // Row r is complete inside this span: write it (or its head partial).
   auto finish_row = [&]() {
@@ -251,7 +281,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
           const int j = c0 + jj;
           while (j >= cur_end) {
             finish_row();
-            next_row();
+            next_row(true);
           }
           if (WMODE == 0) vadd(acc, v[u]);
           else vfma(acc, v[u], w[u]);
@@ -299,10 +329,15 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
       break;
     }
     if (!(is_head || cur_start < n || last)) break;
+    const bool own = last || cur_end < n;
     finish_row();
-    next_row();
+    next_row(own);
   }
-  if (lane == 0 && blockIdx.y == 0) a.tail_row[s] = tail;
+  if (lane == 0 && blockIdx.y == 0) {
+    a.tail_row[3 * s] = tail;
+    a.tail_row[3 * s + 1] = run_begin;
+    a.tail_row[3 * s + 2] = run_end;
+  }
 }
 
 // ----------------------------------------------------------------------------
@@ -377,11 +412,36 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   float* const carry_head = a.carry + (size_t)(2 * s) * F;
   float* const carry_tail = carry_head + F;
 
-  auto next_row = [&]() {
+  // What finish_row leaves in a row without edges.
+  auto store_empty_row = [&](int64_t row) {
+    if ((a.accumulate && !a.bias) || !col_ok) return;
+    float* dst = a.out + row * a.ldo;
+    vec_t z = vzero<V>();
+    if (a.bias) vadd(z, *reinterpret_cast<const vec_t*>(a.bias + col));
+    if (a.accumulate) vadd(z, *reinterpret_cast<const vec_t*>(dst + col));
+    *reinterpret_cast<vec_t*>(dst + col) = z;
+  };
+  // `own`: the rows without edges that follow the finished row belong to this span.  A whole
+  // window of them is not walked row by row (see spmm_span_kernel): one search finds the end of
+  // the run; the first run of a span is left to the fix-up kernel, later ones the groups store,
+  // G rows at a time.
+  int64_t run_begin = 0, run_end = 0;
+  auto next_row = [&](bool own) {
     ++r;
     if (r - rbase == CXG_WAVE) {
       rbase = r;
       row_ends = load_row_ends(rbase);
+      if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) {
+        const int64_t q = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + cur_end + 1);
+        if (run_end == run_begin) {
+          run_begin = r;
+          run_end = q;
+        } else {
+          for (int64_t row = r + g; row < q; row += G) store_empty_row(row);
+        }
+        r = rbase = q;
+        row_ends = load_row_ends(rbase);
+      }
     }
     cur_start = cur_end;
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
@@ -447,7 +507,7 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     while (j < cn) {
       while (c0 + j >= cur_end) {
         finish_row();
-        next_row();
+        next_row(true);
       }
       const int left = (cur_end - (c0 + j)) < (cn - j) ? (cur_end - (c0 + j)) : (cn - j);
       if (left >= UF * G) {                   // long row: UF steps of G edges, loads first
@@ -488,10 +548,15 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
       break;
     }
     if (!(is_head || cur_start < n || last)) break;
+    const bool own = last || cur_end < n;
     finish_row();
-    next_row();
+    next_row(own);
   }
-  if (lane == 0) a.tail_row[s] = tail;
+  if (lane == 0) {
+    a.tail_row[3 * s] = tail;
+    a.tail_row[3 * s + 1] = run_begin;
+    a.tail_row[3 * s + 2] = run_end;
+  }
 }
 
 // One wave per span: if the span holds the tail partial of row t, add the head
@@ -508,10 +573,35 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   const int T = a.T;
   const int64_t n_spans = total > 0 ? (total + T - 1) / T : 1;
   if (s >= n_spans) return;
-  const int64_t t = uniform_i64(a.tail_row[s]);
-  if (t < 0) return;
   const int col = blockIdx.y * (CXG_WAVE * V) + lane * V;
   const bool col_ok = GUARD ? (col < a.F) : true;
+  // Runs of rows without edges that the spans left behind: the run of span q is shared by the
+  // waves q, q + 1, ..., q + J - 1 (modulo the span count), row by row in turn.
+  if (!a.targets && !(a.accumulate && !a.bias)) {
+    const int64_t J = n_spans < CXG_WAVE ? n_spans : CXG_WAVE;
+    int64_t rb = 0, re = 0;
+    if (lane < J) {
+      const int64_t q = (s - lane + n_spans) % n_spans;
+      rb = a.tail_row[3 * q + 1];
+      re = a.tail_row[3 * q + 2];
+    }
+    unsigned long long pending = __ballot(re > rb);
+    while (pending) {
+      const int j = __ffsll((long long)pending) - 1;
+      pending &= pending - 1;
+      const int64_t row_b = shfl_i64(rb, j), row_e = shfl_i64(re, j);
+      for (int64_t row = row_b + j; row < row_e; row += J) {
+        if (!col_ok) continue;
+        float* dst = a.out + row * a.ldo;
+        vec_t z = vzero<V>();
+        if (a.bias) vadd(z, *reinterpret_cast<const vec_t*>(a.bias + col));
+        if (a.accumulate) vadd(z, *reinterpret_cast<const vec_t*>(dst + col));
+        *reinterpret_cast<vec_t*>(dst + col) = z;
+      }
+    }
+  }
+  const int64_t t = uniform_i64(a.tail_row[3 * s]);
+  if (t < 0) return;
   if (!col_ok) return;
   const int F = a.F;
   const int64_t row_begin = (int64_t)a.ptr[t];
@@ -549,6 +639,10 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   *reinterpret_cast<vec_t*>(dst + col) = acc;
 }
 
+// Waves (spans x column tiles) up to which a launch counts as latency-bound: twice what the
+// chip holds at eight waves per SIMD.
+constexpr int64_t kSmallLaunchWaves = 2 * 256 * 4 * 8;
+
 // Span length: 512 edges for large graphs, shorter for small ones so that the
 // launch still has a few thousand waves.
 int choose_span(int64_t n_edges_cap) {
@@ -570,12 +664,12 @@ Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
   Plan p;
   p.T = choose_span(n_edges_cap);
   p.n_spans_cap = n_edges_cap > 0 ? ceil_div(n_edges_cap, p.T) : 1;
-  p.tail_bytes = (size_t)((p.n_spans_cap * sizeof(int64_t) + 255) / 256 * 256);
+  p.tail_bytes = (size_t)((p.n_spans_cap * 3 * sizeof(int64_t) + 255) / 256 * 256);
   p.carry_bytes = (size_t)p.n_spans_cap * 2 * (size_t)row_floats * sizeof(float);
   return p;
 }
 
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0>
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0, bool SMALL = false>
 int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t stream) {
   // Gathers in flight per wave.  Measured on MI355X (61.9M-edge power-law graph):
   // with 32 waves per CU the memory system is already saturated, and issuing more
@@ -584,9 +678,16 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   // 16-byte-per-lane gathers (V == 4) are flat from 1 to 8 and best at 8.
   // With the per-edge dot products four in flight are best: 62 registers instead of 80 keep eight
   // waves per SIMD resident (12.7 -> 11.5 ms on the GAT graph; 16 in flight: 14.5 ms).
-  constexpr int U = DOTG > 0 ? 4 : ((V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U);
+  // A launch too small to fill the chip (a sampled batch's upper layers) is bound by the
+  // latency of its gathers instead, and there the narrow kernels want them overlapped too:
+  // 15 k edges of 47 floats over the transposed graph, 154 -> __ us.
+  constexpr int U = DOTG > 0 ? 4 : ((V == 4) ? CXG_SPMM_U_V4 : (SMALL ? 8 : CXG_SPMM_U));
   const int tile = CXG_WAVE * V;
   const int64_t n_ct = ceil_div(a_in.F, tile);
+  if constexpr (V < 4 && DOTG == 0 && !SMALL) {
+    if (n_spans_cap * n_ct <= kSmallLaunchWaves)
+      return launch_spmm<IdxT, V, GUARD, WMODE, PERM, EXT, DOTG, true>(a_in, n_spans_cap, stream);
+  }
   SpmmArgs<IdxT> a = a_in;
   if (a.exact_edges > 0 && V <= 2) {
     // The edge count is known: lengthen the spans (never shorten: the workspace was sized for

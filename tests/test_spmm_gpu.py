@@ -119,3 +119,67 @@ def test_spmm_width_sweep(feat):
     inv[perm] = torch.arange(idx.shape[0])
     got2 = _ops.spmm(pc, ic, xc, n, val=val[perm].cuda(), val_perm=inv.cuda())
     assert torch.equal(got, got2)
+
+
+def _graph_with_empty_runs(seed):
+    """Long runs of rows without edges at the start, in the middle (two of them inside one
+    64-edge span, one across a span boundary) and at the end, between rows of 1-3 edges and
+    one row long enough to cross spans."""
+    rng = np.random.default_rng(seed)
+    blocks = [np.zeros(1000), rng.integers(1, 4, 20), np.zeros(70), rng.integers(1, 3, 5), np.zeros(300),
+              rng.integers(1, 4, 15), [400], np.zeros(129), rng.integers(0, 3, 2000), np.zeros(64),
+              rng.integers(1, 4, 30), np.zeros(2500)]
+    deg = np.concatenate(blocks).astype(np.int64)
+    ptr = np.concatenate([[0], np.cumsum(deg)])
+    n = deg.shape[0]
+    idx = rng.integers(0, n, int(ptr[-1]))
+    return torch.from_numpy(ptr), torch.from_numpy(idx), n
+
+
+@pytest.mark.parametrize("feat", [8, 47, 128, 256, 330])
+def test_spmm_runs_of_rows_without_edges(feat):
+    """Runs of empty rows are not walked row by row: every variant of the row store (plain,
+    mean, bias, accumulate, int32 indices, a row prefix) still leaves the right values in
+    them and around them."""
+    import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
+    ptr, idx, n = _graph_with_empty_runs(feat)
+    torch.manual_seed(feat)
+    x = torch.randn(n, feat) / 20
+    pc, ic, xc = ptr.cuda(), idx.cuda(), x.cuda()
+    pn, in_, xn = ptr.numpy(), idx.numpy(), x.numpy()
+    announce("spmm empty runs F=%d n=%d E=%d" % (feat, n, idx.shape[0]))
+    want = oracle.spmm(pn, in_, xn, n)
+    got = _ops.spmm(pc, ic, xc, n, out=torch.full((n, feat), 7.0, device="cuda"))
+    assert_close(got.cpu().numpy(), want, RTOL, ATOL, "sum")
+    got = _ops.spmm(pc, ic, xc, n, mean=True, out=torch.full((n, feat), 7.0, device="cuda"))
+    assert_close(got.cpu().numpy(), oracle.spmm(pn, in_, xn, n, mean=True), RTOL, ATOL, "mean")
+    got = B.run_spmm_configurable_int32(pc.int(), ic.int(), xc, n, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+    assert_close(got.cpu().numpy(), want, RTOL, ATOL, "int32")
+    base = torch.randn(n, feat)
+    out = base.clone().cuda()
+    _ops.spmm(pc, ic, xc, n, out=out, accumulate=True)
+    assert_close(out.cpu().numpy(), want + base.numpy(), RTOL, ATOL, "accumulate")
+    val = torch.rand(idx.shape[0]) + 0.5
+    bias = torch.randn(feat)
+    wantw = oracle.spmm(pn, in_, xn, n, val=val.numpy())
+    got = _ops.spmm(pc, ic, xc, n, val=val.cuda(), bias=bias.cuda(), out=torch.full((n, feat), 7.0, device="cuda"))
+    assert_close(got.cpu().numpy(), wantw + bias.numpy(), RTOL, ATOL, "weighted + bias")
+    out = base.clone().cuda()
+    _ops.spmm(pc, ic, xc, n, val=val.cuda(), bias=bias.cuda(), out=out, accumulate=True)
+    assert_close(out.cpu().numpy(), wantw + bias.numpy() + base.numpy(), RTOL, ATOL, "weighted + bias + accumulate")
+    for rows in (1500, 3700, n - 2400):      # prefixes that end inside runs of empty rows
+        got = _ops.spmm(pc, ic, xc, rows, out=torch.full((rows, feat), 7.0, device="cuda"))
+        assert_close(got.cpu().numpy(), want[:rows], RTOL, ATOL, "prefix %d" % rows)
+
+
+def test_spmm_multihead_runs_of_rows_without_edges():
+    from cxgnncomp_backend import _ops
+    ptr, idx, n = _graph_with_empty_runs(5)
+    torch.manual_seed(5)
+    x = torch.randn(n, 4, 64) / 20
+    val = torch.rand(idx.shape[0], 4) + 0.5
+    announce("spmm multihead empty runs")
+    got = _ops.spmm(ptr.cuda(), idx.cuda(), x.cuda(), n, val=val.cuda(), out=torch.full((n, 4, 64), 7.0, device="cuda"))
+    want = oracle.spmm(ptr.numpy(), idx.numpy(), x.numpy(), n, val=val.numpy())
+    assert_close(got.cpu().numpy(), want, RTOL, ATOL, "multihead")
