@@ -215,6 +215,16 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
     is_head = false;
   };
+  if constexpr (DOTG == 0) {
+    // the same for a span that starts with a window of rows without edges
+    if (!is_head && r < n_rows && __ballot(row_ends != 0) == 0) {
+      run_begin = r;
+      run_end = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + 1);
+      r = rbase = run_end;
+      row_ends = load_row_ends(rbase);
+      cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
+    }
+  }
   // Row r is complete inside this span: write it (or its head partial).
   auto finish_row = [&]() {
     if (is_head) {
@@ -447,6 +457,14 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
     is_head = false;
   };
+  // the same for a span that starts with a window of rows without edges
+  if (!is_head && r < n_rows && __ballot(row_ends != 0) == 0) {
+    run_begin = r;
+    run_end = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + 1);
+    r = rbase = run_end;
+    row_ends = load_row_ends(rbase);
+    cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
+  }
   // sum of the groups' partials, valid in group 0 afterwards
   auto reduce_groups = [&]() {
 #pragma unroll
@@ -639,10 +657,6 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   *reinterpret_cast<vec_t*>(dst + col) = acc;
 }
 
-// Waves (spans x column tiles) up to which a launch counts as latency-bound: twice what the
-// chip holds at eight waves per SIMD.
-constexpr int64_t kSmallLaunchWaves = 2 * 256 * 4 * 8;
-
 // Span length: 512 edges for large graphs, shorter for small ones so that the
 // launch still has a few thousand waves.
 int choose_span(int64_t n_edges_cap) {
@@ -669,7 +683,7 @@ Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
   return p;
 }
 
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0, bool SMALL = false>
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0>
 int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t stream) {
   // Gathers in flight per wave.  Measured on MI355X (61.9M-edge power-law graph):
   // with 32 waves per CU the memory system is already saturated, and issuing more
@@ -678,16 +692,11 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   // 16-byte-per-lane gathers (V == 4) are flat from 1 to 8 and best at 8.
   // With the per-edge dot products four in flight are best: 62 registers instead of 80 keep eight
   // waves per SIMD resident (12.7 -> 11.5 ms on the GAT graph; 16 in flight: 14.5 ms).
-  // A launch too small to fill the chip (a sampled batch's upper layers) is bound by the
-  // latency of its gathers instead, and there the narrow kernels want them overlapped too:
-  // 15 k edges of 47 floats over the transposed graph, 154 -> __ us.
-  constexpr int U = DOTG > 0 ? 4 : ((V == 4) ? CXG_SPMM_U_V4 : (SMALL ? 8 : CXG_SPMM_U));
+  // (More gathers in flight for the narrow kernels on launches too small to fill the chip were
+  // measured too: 15 k - 936 k edges of 47 floats, no gain or a loss.)
+  constexpr int U = DOTG > 0 ? 4 : ((V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U);
   const int tile = CXG_WAVE * V;
   const int64_t n_ct = ceil_div(a_in.F, tile);
-  if constexpr (V < 4 && DOTG == 0 && !SMALL) {
-    if (n_spans_cap * n_ct <= kSmallLaunchWaves)
-      return launch_spmm<IdxT, V, GUARD, WMODE, PERM, EXT, DOTG, true>(a_in, n_spans_cap, stream);
-  }
   SpmmArgs<IdxT> a = a_in;
   if (a.exact_edges > 0 && V <= 2) {
     // The edge count is known: lengthen the spans (never shorten: the workspace was sized for
