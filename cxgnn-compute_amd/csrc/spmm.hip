@@ -197,7 +197,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
         // graph): walked row by row, every 64 rows cost a load of the next row ends that first
         // waits for the 64 stores before it (1024 such rows: 125 us), and one wave keeps at most
         // 64 stores in flight.  When the whole window is empty, find the end of the run with one
-        // search and leave its rows to the fix-up kernel, where 64 waves share them.
+        // search and leave its rows to the fix-up kernel, where sixteen waves share them.
         if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) {
           const int64_t q = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + cur_end + 1);
           if (run_end == run_begin) {         // the first such run: the fix-up waves share it
@@ -577,6 +577,8 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   }
 }
 
+constexpr int kRunHelpers = 16;   // fix-up waves that share one span's run of rows without edges
+
 // One wave per span: if the span holds the tail partial of row t, add the head
 // partials of the following spans that row t runs through, in span order.
 template <typename IdxT, int V, bool GUARD>
@@ -594,9 +596,10 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   const int col = blockIdx.y * (CXG_WAVE * V) + lane * V;
   const bool col_ok = GUARD ? (col < a.F) : true;
   // Runs of rows without edges that the spans left behind: the run of span q is shared by the
-  // waves q, q + 1, ..., q + J - 1 (modulo the span count), row by row in turn.
+  // waves q, q + 1, ..., q + J - 1 (modulo the span count), row by row in turn.  (Sixteen
+  // helpers: with 64 the slot reads alone cost the headline launch 13 us.)
   if (!a.targets && !(a.accumulate && !a.bias)) {
-    const int64_t J = n_spans < CXG_WAVE ? n_spans : CXG_WAVE;
+    const int64_t J = n_spans < kRunHelpers ? n_spans : kRunHelpers;
     int64_t rb = 0, re = 0;
     if (lane < J) {
       const int64_t q = (s - lane + n_spans) % n_spans;
