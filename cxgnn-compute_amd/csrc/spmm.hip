@@ -36,6 +36,11 @@ namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
+// Windows of 64 rows without edges after which the end of a run of them is found with a search
+// and the run left to the fix-up kernel (for a shorter run the search costs more than a look
+// at the next windows: with the search from the first window on, an RGCN layer whose pair
+// tables hold many runs of 64-200 such rows lost 2 %).
+constexpr int kRunWindows = 4;
 
 template <int V> struct Vec;
 template <> struct Vec<1> { using type = float; };
@@ -185,6 +190,43 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     *reinterpret_cast<vec_t*>(dst + col) = z;
   };
   int64_t run_begin = 0, run_end = 0;
+  // A long run of rows without edges (the seed rows of a sampled batch in the reversed graph):
+  // walked row by row, every 64 rows cost a load of the next row ends that first waits for the
+  // 64 stores before it (1024 such rows: 125 us), and one wave keeps at most 64 stores in
+  // flight.  Called with rbase == r and a window whose rows all end at `end_rel`, i.e. have no
+  // edges: looks on window by window, and after kRunWindows of them finds the end of the run
+  // with one search.  A run of kRunWindows windows or more is left to the fix-up kernel, where
+  // sixteen waves share it (the first one of a span; its workspace slot holds one run), a
+  // shorter one is stored here, now without loads between the stores.
+  auto skip_rows_without_edges = [&](int end_rel) {
+    const int64_t first = r;
+    int64_t q = r;
+    for (int hop = 1;; ++hop) {
+      q += CXG_WAVE;
+      if (q >= n_rows) { q = rbase = n_rows; break; }
+      if (hop == kRunWindows) {
+        q += wave_lower_bound(a.ptr + q + 1, n_rows - q, e0 + end_rel + 1);
+        rbase = q;
+        if (q < n_rows) row_ends = load_row_ends(rbase);
+        break;
+      }
+      const int w = load_row_ends(q);
+      const unsigned long long busy = __ballot(w != end_rel);
+      if (busy) {
+        rbase = q;
+        row_ends = w;
+        q += __ffsll((long long)busy) - 1;
+        break;
+      }
+    }
+    r = q;
+    if (r - first >= kRunWindows * CXG_WAVE && run_end == run_begin) {
+      run_begin = first;
+      run_end = r;
+    } else {
+      for (int64_t row = first; row < r; ++row) store_empty_row(row);
+    }
+  };
   // `own`: the rows without edges that follow the finished row belong to this span.
   auto next_row = [&](bool own) {
     ++r;
@@ -193,22 +235,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
       rbase = r;
       row_ends = load_row_ends(rbase);
       if constexpr (DOTG == 0) {
-        // A long run of rows without edges (the seed rows of a sampled batch in the reversed
-        // graph): walked row by row, every 64 rows cost a load of the next row ends that first
-        // waits for the 64 stores before it (1024 such rows: 125 us), and one wave keeps at most
-        // 64 stores in flight.  When the whole window is empty, find the end of the run with one
-        // search and leave its rows to the fix-up kernel, where sixteen waves share them.
-        if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) {
-          const int64_t q = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + cur_end + 1);
-          if (run_end == run_begin) {         // the first such run: the fix-up waves share it
-            run_begin = r;
-            run_end = q;
-          } else {
-            for (int64_t row = r; row < q; ++row) store_empty_row(row);
-          }
-          r = rbase = q;
-          row_ends = load_row_ends(rbase);
-        }
+        if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) skip_rows_without_edges(cur_end);
       }
     }
     cur_start = cur_end;
@@ -218,11 +245,8 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   if constexpr (DOTG == 0) {
     // the same for a span that starts with a window of rows without edges
     if (!is_head && r < n_rows && __ballot(row_ends != 0) == 0) {
-      run_begin = r;
-      run_end = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + 1);
-      r = rbase = run_end;
-      row_ends = load_row_ends(rbase);
-      cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
+      skip_rows_without_edges(0);
+      cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
     }
   }
   // Row r is complete inside this span: write it (or its head partial).
@@ -436,22 +460,41 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   // the run; the first run of a span is left to the fix-up kernel, later ones the groups store,
   // G rows at a time.
   int64_t run_begin = 0, run_end = 0;
+  auto skip_rows_without_edges = [&](int end_rel) {     // see spmm_span_kernel
+    const int64_t first = r;
+    int64_t q = r;
+    for (int hop = 1;; ++hop) {
+      q += CXG_WAVE;
+      if (q >= n_rows) { q = rbase = n_rows; break; }
+      if (hop == kRunWindows) {
+        q += wave_lower_bound(a.ptr + q + 1, n_rows - q, e0 + end_rel + 1);
+        rbase = q;
+        if (q < n_rows) row_ends = load_row_ends(rbase);
+        break;
+      }
+      const int w = load_row_ends(q);
+      const unsigned long long busy = __ballot(w != end_rel);
+      if (busy) {
+        rbase = q;
+        row_ends = w;
+        q += __ffsll((long long)busy) - 1;
+        break;
+      }
+    }
+    r = q;
+    if (r - first >= kRunWindows * CXG_WAVE && run_end == run_begin) {
+      run_begin = first;
+      run_end = r;
+    } else {
+      for (int64_t row = first + g; row < r; row += G) store_empty_row(row);
+    }
+  };
   auto next_row = [&](bool own) {
     ++r;
     if (r - rbase == CXG_WAVE) {
       rbase = r;
       row_ends = load_row_ends(rbase);
-      if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) {
-        const int64_t q = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + cur_end + 1);
-        if (run_end == run_begin) {
-          run_begin = r;
-          run_end = q;
-        } else {
-          for (int64_t row = r + g; row < q; row += G) store_empty_row(row);
-        }
-        r = rbase = q;
-        row_ends = load_row_ends(rbase);
-      }
+      if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) skip_rows_without_edges(cur_end);
     }
     cur_start = cur_end;
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
@@ -459,11 +502,8 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   };
   // the same for a span that starts with a window of rows without edges
   if (!is_head && r < n_rows && __ballot(row_ends != 0) == 0) {
-    run_begin = r;
-    run_end = r + wave_lower_bound(a.ptr + r + 1, n_rows - r, e0 + 1);
-    r = rbase = run_end;
-    row_ends = load_row_ends(rbase);
-    cur_end = (r < n_rows) ? bcast_i32(row_ends, 0) : 0x7fffffff;
+    skip_rows_without_edges(0);
+    cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
   }
   // sum of the groups' partials, valid in group 0 afterwards
   auto reduce_groups = [&]() {
@@ -598,6 +638,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
   // Runs of rows without edges that the spans left behind: the run of span q is shared by the
   // waves q, q + 1, ..., q + J - 1 (modulo the span count), row by row in turn.  (Sixteen
   // helpers: with 64 the slot reads alone cost the headline launch 13 us.)
+  const int64_t t_slot = a.tail_row[3 * s];       // issued with the slot reads below: one wait for both
   if (!a.targets && !(a.accumulate && !a.bias)) {
     const int64_t J = n_spans < kRunHelpers ? n_spans : kRunHelpers;
     int64_t rb = 0, re = 0;
@@ -621,7 +662,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
       }
     }
   }
-  const int64_t t = uniform_i64(a.tail_row[3 * s]);
+  const int64_t t = uniform_i64(t_slot);
   if (t < 0) return;
   if (!col_ok) return;
   const int F = a.F;
