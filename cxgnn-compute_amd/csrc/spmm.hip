@@ -189,7 +189,11 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     if (a.accumulate) vadd(z, *reinterpret_cast<const vec_t*>(dst + col));
     *reinterpret_cast<vec_t*>(dst + col) = z;
   };
-  int64_t run_begin = 0, run_end = 0;
+  // (not in the per-head kernels: there the extra live registers cost a wave of occupancy, and
+  // the fused dot-product form prefetches rows of dot_b in step with the walk)
+  constexpr bool kSkipRuns = DOTG == 0 && WMODE != 2;
+  bool run_left = false;                       // this span's slot holds a run
+  if (lane == 0 && blockIdx.y == 0) { a.tail_row[3 * s + 1] = 0; a.tail_row[3 * s + 2] = 0; }
   // A long run of rows without edges (the seed rows of a sampled batch in the reversed graph):
   // walked row by row, every 64 rows cost a load of the next row ends that first waits for the
   // 64 stores before it (1024 such rows: 125 us), and one wave keeps at most 64 stores in
@@ -220,9 +224,9 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
       }
     }
     r = q;
-    if (r - first >= kRunWindows * CXG_WAVE && run_end == run_begin) {
-      run_begin = first;
-      run_end = r;
+    if (r - first >= kRunWindows * CXG_WAVE && !run_left) {
+      run_left = true;
+      if (lane == 0 && blockIdx.y == 0) { a.tail_row[3 * s + 1] = first; a.tail_row[3 * s + 2] = r; }
     } else {
       for (int64_t row = first; row < r; ++row) store_empty_row(row);
     }
@@ -234,7 +238,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     if (r - rbase == CXG_WAVE) {
       rbase = r;
       row_ends = load_row_ends(rbase);
-      if constexpr (DOTG == 0) {
+      if constexpr (kSkipRuns) {
         if (own && r < n_rows && __ballot(row_ends != cur_end) == 0) skip_rows_without_edges(cur_end);
       }
     }
@@ -242,7 +246,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
     is_head = false;
   };
-  if constexpr (DOTG == 0) {
+  if constexpr (kSkipRuns) {
     // the same for a span that starts with a window of rows without edges
     if (!is_head && r < n_rows && __ballot(row_ends != 0) == 0) {
       skip_rows_without_edges(0);
@@ -367,11 +371,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     finish_row();
     next_row(own);
   }
-  if (lane == 0 && blockIdx.y == 0) {
-    a.tail_row[3 * s] = tail;
-    a.tail_row[3 * s + 1] = run_begin;
-    a.tail_row[3 * s + 2] = run_end;
-  }
+  if (lane == 0 && blockIdx.y == 0) a.tail_row[3 * s] = tail;
 }
 
 // ----------------------------------------------------------------------------
@@ -459,7 +459,8 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   // window of them is not walked row by row (see spmm_span_kernel): one search finds the end of
   // the run; the first run of a span is left to the fix-up kernel, later ones the groups store,
   // G rows at a time.
-  int64_t run_begin = 0, run_end = 0;
+  bool run_left = false;                       // this span's slot holds a run
+  if (lane == 0) { a.tail_row[3 * s + 1] = 0; a.tail_row[3 * s + 2] = 0; }
   auto skip_rows_without_edges = [&](int end_rel) {     // see spmm_span_kernel
     const int64_t first = r;
     int64_t q = r;
@@ -482,9 +483,9 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
       }
     }
     r = q;
-    if (r - first >= kRunWindows * CXG_WAVE && run_end == run_begin) {
-      run_begin = first;
-      run_end = r;
+    if (r - first >= kRunWindows * CXG_WAVE && !run_left) {
+      run_left = true;
+      if (lane == 0) { a.tail_row[3 * s + 1] = first; a.tail_row[3 * s + 2] = r; }
     } else {
       for (int64_t row = first + g; row < r; row += G) store_empty_row(row);
     }
@@ -610,11 +611,7 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     finish_row();
     next_row(own);
   }
-  if (lane == 0) {
-    a.tail_row[3 * s] = tail;
-    a.tail_row[3 * s + 1] = run_begin;
-    a.tail_row[3 * s + 2] = run_end;
-  }
+  if (lane == 0) a.tail_row[3 * s] = tail;
 }
 
 constexpr int kRunHelpers = 16;   // fix-up waves that share one span's run of rows without edges
