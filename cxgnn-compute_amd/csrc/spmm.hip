@@ -18,6 +18,13 @@
 // run_spmm_sharedmem* (src/cpp/src/spmm_kernel.cu:231-512).
 #include "cxg_common.hpp"
 
+#include <atomic>
+
+// Carry buffer and span table of cxg_spmm_sum_f32_noalloc: one copy per GPU, part of the
+// code object, held until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress; the device address is looked up once per device (static_scratch()).
+static __device__ __align__(256) unsigned char scratch[CXG_SPMM_NOALLOC_SCRATCH_BYTES];
+
 namespace cxg {
 namespace {
 
@@ -937,6 +944,24 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   return set_error(CXG_ERR_UNSUPPORTED, "weighted SpMM needs int64 indices");
 }
 
+// Device address of `scratch` on the current device, looked up on the first call there.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_scratch(void** out) {
+  int dev = -1;
+  CXG_HIP_CHECK(hipGetDevice(&dev));
+  CXG_REQUIRE(dev >= 0 && dev < kMaxDevices, CXG_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    CXG_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    CXG_REQUIRE(p != nullptr, CXG_ERR_HIP, "hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return CXG_OK;
+}
+
 }  // namespace
 }  // namespace cxg
 
@@ -953,6 +978,23 @@ int cxg_spmm_sum_f32(const int64_t* ptr, const int64_t* idx, const float* x, int
                      unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
   return cxg::spmm_common<int64_t>(ptr, idx, nullptr, nullptr, x, ldx, out, ldo, n_rows,
                                    n_edges_cap, 1, feat, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_sum_f32_noalloc(const int64_t* ptr, const int64_t* idx, const float* x, int64_t ldx,
+                             float* out, int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int feat,
+                             unsigned flags, void* stream) {
+  CXG_REQUIRE(n_edges_cap >= 0 && feat >= 1, CXG_ERR_ARG, "negative size");
+  const cxg::Plan p = cxg::make_plan(n_edges_cap, feat);
+  const size_t need = p.tail_bytes + p.carry_bytes;
+  CXG_REQUIRE(need <= (size_t)CXG_SPMM_NOALLOC_SCRATCH_BYTES, CXG_ERR_WORKSPACE,
+              "cxg_spmm_sum_f32_noalloc: %lld edges of %d floats need %zu bytes of scratch, the built-in "
+              "buffer holds %zu; use cxg_spmm_sum_f32 with a workspace",
+              (long long)n_edges_cap, feat, need, (size_t)CXG_SPMM_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  const int rc = cxg::static_scratch(&ws);
+  if (rc != CXG_OK) return rc;
+  return cxg::spmm_common<int64_t>(ptr, idx, nullptr, nullptr, x, ldx, out, ldo, n_rows, n_edges_cap,
+                                   1, feat, flags, ws, (size_t)CXG_SPMM_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int cxg_spmm_sum_f32_i32(const int32_t* ptr, const int32_t* idx, const float* x, int64_t ldx,

@@ -26,6 +26,7 @@ SIGNATURES = {
     "cxg_last_error": (_c.c_char_p, []),
     "cxg_spmm_workspace_bytes": (_SZ, [_I64, _I64]),
     "cxg_spmm_sum_f32": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
+    "cxg_spmm_sum_f32_noalloc": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P]),
     "cxg_spmm_sum_f32_i32": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
     "cxg_spmm_weighted_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32,
                                      _U32, _P, _SZ, _P]),

@@ -69,6 +69,27 @@ int cxg_spmm_sum_f32(const int64_t* ptr, const int64_t* idx, const float* x,
                      int64_t n_edges_cap, int feat, unsigned flags,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * cxg_spmm_sum_f32 for callers that can neither allocate device memory nor hand over a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference.  Same kernels and results as
+ * cxg_spmm_sum_f32; the carry buffer and span table live in a device array of
+ * CXG_SPMM_NOALLOC_SCRATCH_BYTES that is part of the library's code object (every GPU the
+ * library runs on holds its own copy until the process ends).  The call allocates and frees
+ * nothing.  Shapes whose cxg_spmm_workspace_bytes(n_edges_cap, feat) exceeds that size are
+ * rejected with CXG_ERR_WORKSPACE (the limit is 32 million edges at feat = 128, 16 million
+ * at feat = 256).  Every call on one GPU uses that GPU's
+ * one array: calls that overlap in time on the same GPU (two streams, two threads) race;
+ * calls on one stream are ordered and safe.  Nothing in the array needs clearing between
+ * calls: each launch writes every slot it later reads.  The first call on a device looks up
+ * the array's address (hipGetSymbolAddress) and must therefore happen outside a graph
+ * capture; later calls only launch kernels.
+ */
+#define CXG_SPMM_NOALLOC_SCRATCH_BYTES (64u << 20)
+int cxg_spmm_sum_f32_noalloc(const int64_t* ptr, const int64_t* idx, const float* x,
+                             int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
+                             int64_t n_edges_cap, int feat, unsigned flags, void* stream);
+
 /* Same with int32 ptr/idx.  Replaces run_spmm_configurable_int32
  * (src/cpp/src/spmm_host.cu:99-156). */
 int cxg_spmm_sum_f32_i32(const int32_t* ptr, const int32_t* idx, const float* x,
