@@ -121,6 +121,11 @@ def _pad_rel(rel, idx, count, thres, num_rel, base):
         st = lib.cxg_pad_rel_i64(rel.data_ptr(), _lib.ptr(idx), count.data_ptr(), thres, num_rel, base,
                                  _lib.current_stream(rel.device))
     _lib.check(st)
+    # the library wrote through raw pointers: bump the tensors' version counters, which key
+    # the caches of structures derived from index arrays (transposed graphs, pair tables)
+    torch.autograd.graph.increment_version(rel)
+    if idx is not None:
+        torch.autograd.graph.increment_version(idx)
 
 
 def pad_rel(rel, count, thres, num_rel, base):
