@@ -215,12 +215,16 @@ class MyGINConv(torch.nn.Module):
 
 class MyRGCNConv(torch.nn.Module):
 
-    def __init__(self, in_channels, hidden_channels, num_rel):
+    def __init__(self, in_channels, hidden_channels, num_rel, precision=None):
+        """``precision`` (not upstream): how the typed GEMMs of the layer multiply --
+        None / "split6" (fp32-accurate), "split3", "fp32", or "bf16" (operands rounded to
+        bf16 on the bf16 matrix cores, fp32 accumulation and fp32 aggregation)."""
         super().__init__()
         assert num_rel > 0
         self.in_channels = in_channels
         self.hidden_channels = hidden_channels
         self.num_rel = num_rel
+        self.precision = precision
         self.linear = torch.nn.Parameter(torch.randn(num_rel, in_channels, hidden_channels))
         self.register_parameter("rel_weight", self.linear)
         self.single_linear = torch.nn.Linear(in_channels, hidden_channels)
@@ -238,7 +242,7 @@ class MyRGCNConv(torch.nn.Module):
         # rows of every destination (run_rgcn4, :309-326, :352-378); the same layer as
         # one op that never materialises per-edge rows.  Rows without edges give 0
         # (upstream divides 0 by 0 there).
-        return cxgnncomp_backend.aggr_rgcn_mean(x, ptr, idx, self.linear, edge_types, num_node)
+        return cxgnncomp_backend.aggr_rgcn_mean(x, ptr, idx, self.linear, edge_types, num_node, self.precision)
 
 
 _ARANGE = {}

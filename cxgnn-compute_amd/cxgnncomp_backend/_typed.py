@@ -16,7 +16,9 @@ GEMM_SPLIT_BF16X3 = 8
 
 # How fp32 typed GEMMs multiply: "split6" (six bf16 partial products per fp32
 # product: fp32-accurate and HBM bound for K <= 128), "split3" (three partial
-# products, relative error below 2^-16 per product) or "fp32" (v_mfma_f32_32x32x2_f32).
+# products, relative error below 2^-16 per product), "fp32" (v_mfma_f32_32x32x2_f32) or
+# "bf16" (operands rounded to bf16, one bf16 MFMA product, fp32 accumulation; weight
+# gradients then use "split3").
 GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split6")
 _PRECISION_FLAGS = {"fp32": 0, "split6": GEMM_SPLIT_BF16X6, "split3": GEMM_SPLIT_BF16X3}
 
@@ -48,9 +50,11 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
     a [*, K] fp32, w [R, K, N] fp32.  precision "split6" (the default, see
     GEMM_PRECISION) forms every fp32 product from six bf16 partial products
     (fp32-accurate), "split3" from three (relative error per product < 2^-16, the
-    reference's tl.dot is TF32); "fp32" forces v_mfma_f32_32x32x2_f32.  With bf16=True the operands are rounded
-    to bf16 (W transposed to [R, N, K]) and multiplied on the bf16 matrix cores."""
+    reference's tl.dot is TF32); "fp32" forces v_mfma_f32_32x32x2_f32.  With bf16=True or
+    precision "bf16" the operands are rounded to bf16 (W transposed to [R, N, K]) and multiplied
+    on the bf16 matrix cores with fp32 accumulation."""
     lib = _lib.load()
+    bf16 = bf16 or (precision or GEMM_PRECISION) == "bf16"
     _req(a, "a", torch.float32 if not (bf16 and a.dtype == torch.bfloat16) else torch.bfloat16, 2)
     if w.dim() != 3:
         raise ValueError("weights must be [num_rel, K, N]")
@@ -79,9 +83,12 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
         raise ValueError("output has fewer rows than M")
     flags = (GEMM_ACCUMULATE if accumulate else 0) | (GEMM_ATOMIC if atomic else 0)
     precision = precision or GEMM_PRECISION
-    if precision not in _PRECISION_FLAGS:
-        raise ValueError("precision must be one of %s" % sorted(_PRECISION_FLAGS))
-    flags |= _PRECISION_FLAGS[precision]
+    if precision == "bf16":
+        bf16 = True
+    elif precision not in _PRECISION_FLAGS:
+        raise ValueError("precision must be one of %s" % sorted(list(_PRECISION_FLAGS) + ["bf16"]))
+    else:
+        flags |= _PRECISION_FLAGS[precision]
     stream = _lib.current_stream(a.device)
     with torch.cuda.device(a.device):
         if bf16:
@@ -248,7 +255,7 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     if K % 4 or N % 4 or (K > 128 and num_rel != 1):
         return None
     precision = precision or GEMM_PRECISION
-    flags = GEMM_SPLIT_BF16X3 if precision == "split3" else GEMM_SPLIT_BF16X6
+    flags = GEMM_SPLIT_BF16X3 if precision in ("split3", "bf16") else GEMM_SPLIT_BF16X6
     gw = torch.empty((num_rel, K, N), dtype=torch.float32, device=a.device)
     with torch.cuda.device(a.device):
         for k0 in range(0, K, 128):
@@ -262,12 +269,12 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     return gw
 
 
-def _weight_grad(x, g, src, dst, seg, shape):
+def _weight_grad(x, g, src, dst, seg, shape, precision=None):
     """grad_W[r] = sum over the rows of segment r of x[src]^T g[dst]: one launch of the
     typed weight-gradient kernel; shapes it does not take use a row gather plus one
     library GEMM per relation."""
     x, g = x.contiguous(), g.contiguous()
-    gw = typed_gemm_wgrad(x, g, seg, src.shape[0], shape[0], src_idx=src, dst_idx=dst)
+    gw = typed_gemm_wgrad(x, g, seg, src.shape[0], shape[0], src_idx=src, dst_idx=dst, precision=precision)
     if gw is not None:
         return gw
     gw = torch.zeros(shape, dtype=torch.float32, device=x.device)
@@ -394,7 +401,7 @@ def _pair_graph_aggregate(pg, idx, n):
     return pg
 
 
-def _pairs_aggregate_first(pg, x, weights, idx, n):
+def _pairs_aggregate_first(pg, x, weights, idx, n, precision=None):
     """out[d] = sum_r (sum of x over d's edges of relation r) @ W[r] on the (destination,
     relation) pairs that own an edge: one SpMM into the pair rows (gathering rows of x), one
     typed GEMM over the relation segments of pair rows, one SpMM that gives every destination
@@ -402,19 +409,21 @@ def _pairs_aggregate_first(pg, x, weights, idx, n):
     _pair_graph_aggregate(pg, idx, n)
     n_pairs = pg.b_dst.shape[0]
     z = _ops.spmm(pg.bp_ptr, pg.bp_src, x, n_pairs)                       # [Ub, K]
-    t = typed_gemm(z, weights, pg.b_seg, n_pairs)                         # [Ub, N]
+    t = typed_gemm(z, weights, pg.b_seg, n_pairs, precision=precision)                         # [Ub, N]
     return _ops.spmm(pg.dp_ptr, pg.dp_rows, t, n), z
 
 
-def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w):
+def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w, precision=None):
     """Gradients of _pairs_aggregate_first for x and the weights."""
     n_pairs = pg.b_dst.shape[0]
     gx = gw = None
     if need_x:
-        gz = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, n_pairs, src_idx=pg.b_dst)
+        gz = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, n_pairs, src_idx=pg.b_dst,
+                        precision=precision)
         gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, gz, n_src)
     if need_w:
-        gw = _weight_grad(z, grad_out, _edge_positions(n_pairs, z.device), pg.b_dst, pg.b_seg, weights.shape)
+        gw = _weight_grad(z, grad_out, _edge_positions(n_pairs, z.device), pg.b_dst, pg.b_seg, weights.shape,
+                          precision)
     return gx, gw
 
 
@@ -438,7 +447,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
     gradients are computed here."""
 
     @staticmethod
-    def forward(ctx, x, ptr, idx, weights, rel, num_node, mean=False, force_dense=False):
+    def forward(ctx, x, ptr, idx, weights, rel, num_node, mean=False, force_dense=False, precision=None):
         n = as_int(num_node)
         if n == 0:
             n = ptr.shape[0] - 1
@@ -449,6 +458,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
         R, K, N = weights.shape
         n_src = x.shape[0]
         ctx.n, ctx.mean = n, mean
+        ctx.precision = precision
         n_edges = int(ptr[n].item())
         ctx.dense = force_dense or _use_dense(n_edges, n_src, R, N)
         ctx.pairs = False
@@ -459,14 +469,14 @@ class _RgcnFusedFunction(torch.autograd.Function):
             ctx.pairs = pg.f_src.shape[0] <= RGCN_PAIR_FILL_MAX * n_src * R
         ctx.aggregate_first = ctx.pairs and K <= N and not force_dense     # gather the narrower rows
         if ctx.aggregate_first:
-            out, z = _pairs_aggregate_first(pg, x, weights, idx, n)
+            out, z = _pairs_aggregate_first(pg, x, weights, idx, n, precision)
             if mean:
                 out *= _inv_degree(ptr, n).unsqueeze(1)
             ctx.pg = pg
             ctx.save_for_backward(x, weights, ptr, z)
             return out
         if ctx.pairs:
-            y = typed_gemm(x, weights, pg.f_seg, pg.f_src.shape[0], src_idx=pg.f_src)    # [Uf, N]
+            y = typed_gemm(x, weights, pg.f_seg, pg.f_src.shape[0], src_idx=pg.f_src, precision=precision)    # [Uf, N]
             out = _ops.spmm(ptr, pg.f_row, y, n, mean=mean)
             ctx.pg = pg
             ctx.save_for_backward(x, weights, ptr)
@@ -474,7 +484,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
         if ctx.dense:
             rg = _rel_graph(ptr, idx, rel, n, n_src, R)
             wcat = weights.permute(1, 0, 2).reshape(1, K, R * N).contiguous()
-            y = typed_gemm(x, wcat, _dense_seg(n_src, x.device), n_src)          # [n_src, R*N]
+            y = typed_gemm(x, wcat, _dense_seg(n_src, x.device), n_src, precision=precision)          # [n_src, R*N]
             out = _ops.spmm(ptr, rg.key_fwd, y.view(n_src * R, N), n, mean=mean)
             ctx.rg = rg
             ctx.save_for_backward(x, weights, ptr)
@@ -486,12 +496,12 @@ class _RgcnFusedFunction(torch.autograd.Function):
             # one output row per edge, written once in CSR order, then the plain sum over
             # each destination's (consecutive) rows: no atomics, reproducible
             tmp = torch.empty((n_edges, N), dtype=torch.float32, device=x.device)
-            typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=perm, out=tmp)
+            typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=perm, out=tmp, precision=precision)
             out = _ops.spmm(ptr, _edge_positions(n_edges, x.device), tmp, n, mean=mean)
             ctx.save_for_backward(x, weights, ptr, src, dst, seg, perm, idx)
             return out
         out = torch.zeros((n, N), dtype=torch.float32, device=x.device)
-        typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=dst, out=out, atomic=True)
+        typed_gemm(x, weights, seg, n_edges, src_idx=src, dst_idx=dst, out=out, atomic=True, precision=precision)
         if mean:
             out *= _inv_degree(ptr, n).unsqueeze(1)
         ctx.save_for_backward(x, weights, ptr, src, dst, seg)
@@ -503,42 +513,44 @@ class _RgcnFusedFunction(torch.autograd.Function):
         x, weights, ptr = ctx.saved_tensors[:3]
         R, K, N = weights.shape
         n, n_src = ctx.n, x.shape[0]
+        precision = ctx.precision
         if ctx.mean:
             grad_out = grad_out * _inv_degree(ptr, n).unsqueeze(1)
         gx = gw = None
         if ctx.aggregate_first:
             gx, gw = _pairs_aggregate_first_bwd(ctx.pg, weights, ctx.saved_tensors[3], grad_out, n_src,
-                                                ctx.needs_input_grad[0], ctx.needs_input_grad[3])
-            return gx, None, None, gw, None, None, None, None
+                                                ctx.needs_input_grad[0], ctx.needs_input_grad[3], precision)
+            return gx, None, None, gw, None, None, None, None, None
         if ctx.pairs:
             pg = ctx.pg
             if ctx.needs_input_grad[0]:
                 # Z = g[d] @ W[r]^T for the (destination, relation) pairs that occur, then the
                 # plain SpMM over the reversed graph
                 z = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, pg.b_dst.shape[0],
-                               src_idx=pg.b_dst)
+                               src_idx=pg.b_dst, precision=precision)
                 gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, z, n_src)
             if ctx.needs_input_grad[3]:
                 # gY = sum of g over the edges of every (source, relation) pair; gW[r] = x[src]^T gY
                 gy = _ops.spmm(pg.f_ptr, pg.f_dst, grad_out, pg.f_src.shape[0])
-                gw = _weight_grad(x, gy, pg.f_src, None, pg.f_seg, weights.shape)
-            return gx, None, None, gw, None, None, None, None
+                gw = _weight_grad(x, gy, pg.f_src, None, pg.f_seg, weights.shape, precision)
+            return gx, None, None, gw, None, None, None, None, None
         if ctx.dense:
             rg = ctx.rg
             if ctx.needs_input_grad[0]:
                 # Z[d, r] = g[d] @ W[r]^T for every (destination, relation), then the
                 # plain SpMM over the reversed graph
                 wcat_t = weights.permute(2, 0, 1).reshape(1, N, R * K).contiguous()
-                z = typed_gemm(grad_out, wcat_t, _dense_seg(n, x.device), n)      # [n, R*K]
+                z = typed_gemm(grad_out, wcat_t, _dense_seg(n, x.device), n, precision=precision)      # [n, R*K]
                 gx = _ops.spmm(rg.ptr_src, rg.key_bwd, z.view(n * R, K), n_src)
             if ctx.needs_input_grad[3]:
                 # gY[s, r] = sum of g over the edges (s -> d) of relation r; gW[r] = x^T gY[:, r]
                 gy = _ops.spmm(rg.ptr_key, rg.idx_key, grad_out, n_src * R)      # [n_src*R, N]
-                gw = typed_gemm_wgrad(x, gy.view(n_src, R * N), _dense_seg(n_src, x.device), n_src, 1)
+                gw = typed_gemm_wgrad(x, gy.view(n_src, R * N), _dense_seg(n_src, x.device), n_src, 1,
+                                      precision=precision)
                 if gw is None:
                     gw = torch.mm(x.t(), gy.view(n_src, R * N))
                 gw = gw.view(K, R, N).permute(1, 0, 2).contiguous()
-            return gx, None, None, gw, None, None, None, None
+            return gx, None, None, gw, None, None, None, None, None
         src, dst, seg = ctx.saved_tensors[3:6]
         if ctx.needs_input_grad[0] and ctx.per_edge:
             # per-edge rows g[dst(e)] @ W[rel(e)]^T in CSR order, summed per source over the
@@ -546,16 +558,16 @@ class _RgcnFusedFunction(torch.autograd.Function):
             perm, idx = ctx.saved_tensors[6:8]
             tmp = torch.empty((ctx.n_edges, K), dtype=torch.float32, device=x.device)
             typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), seg, ctx.n_edges, src_idx=dst,
-                       dst_idx=perm, out=tmp)
+                       dst_idx=perm, out=tmp, precision=precision)
             gt = _ops.transposed(ptr, idx, n, n_src)
             gx = _ops.spmm(gt.ptr_t, gt.perm, tmp, n_src)
         elif ctx.needs_input_grad[0]:
             gx = torch.zeros_like(x)
             typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), seg, ctx.n_edges, src_idx=dst,
-                       dst_idx=src, out=gx, atomic=True)
+                       dst_idx=src, out=gx, atomic=True, precision=precision)
         if ctx.needs_input_grad[3]:
-            gw = _weight_grad(x, grad_out, src, dst, seg, weights.shape)
-        return gx, None, None, gw, None, None, None, None
+            gw = _weight_grad(x, grad_out, src, dst, seg, weights.shape, precision)
+        return gx, None, None, gw, None, None, None, None, None
 
 
 _DST_REL_CACHE = collections.OrderedDict()
@@ -592,11 +604,12 @@ def aggr_rgcn_direct_func(input, ptr, idx, weights, rel, num_node):
     return _RgcnFusedFunction.apply(input, ptr, idx, weights, rel, num_node)
 
 
-def aggr_rgcn_mean(input, ptr, idx, weights, rel, num_node):
+def aggr_rgcn_mean(input, ptr, idx, weights, rel, num_node, precision=None):
     """aggr_rgcn_direct_func divided by each row's edge count (rows without edges
     give 0): the whole relational layer of MyRGCNConv
-    (cxgnncomp/graph_conv.py:352-378) in one differentiable op."""
-    return _RgcnFusedFunction.apply(input, ptr, idx, weights, rel, num_node, True)
+    (cxgnncomp/graph_conv.py:352-378) in one differentiable op.  ``precision`` selects how
+    the typed GEMMs multiply (see typed_gemm; None = GEMM_PRECISION)."""
+    return _RgcnFusedFunction.apply(input, ptr, idx, weights, rel, num_node, True, False, precision)
 
 
 def aggr_rel_direct(input, ptr, idx, weights, etype, num_node, num_rel):

@@ -165,3 +165,308 @@ def test_gspmm_full_size(big):
     ref = oracle.gspmm(sp.astype(np.int32), si.astype(np.int32), x.cpu().numpy(), 2, 0,
                        val=val[torch.from_numpy(pos).cuda()].cpu().numpy())
     assert np.array_equal(got2[torch.from_numpy(rows).cuda()].cpu().numpy(), ref)
+
+
+# --------------------------------------------------------------------------- #
+# RGCN configuration at its stated size: 1,000,000 nodes / 20,000,000 edges / 16 relations
+# --------------------------------------------------------------------------- #
+C4_N, C4_E, C4_R, C4_K = 1000000, 20000000, 16, 128
+
+
+@pytest.fixture(scope="module")
+def hetero():
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    announce("generate the 1M-node / 20M-edge / 16-relation graph on the GPU")
+    ptr, idx, etype, _ = S.hetero_graph(C4_N, C4_E, num_rel=C4_R, seed=0, device="cuda")
+    rows = _ops.csr_row_ids(ptr, C4_N, C4_E)
+    torch.manual_seed(4)
+    x = torch.randn(C4_N, C4_K, device="cuda") / 8
+    w = torch.randn(C4_R, C4_K, C4_K, device="cuda") * 0.02
+    g = torch.randn(C4_N, C4_K, device="cuda") / 16
+    torch.cuda.synchronize()
+    return ptr, idx, etype, rows, x, w, g
+
+
+def _rgcn_float64(ptr, idx, etype, rows, x, w, g):
+    """out[d] = sum_e x[idx[e]] W[rel[e]] and both gradients for the output gradient g, in float64
+    with plain torch ops on the device, one relation at a time (index_select, mm, index_add_)."""
+    x64, w64, g64 = x.double(), w.double(), g.double()
+    out = torch.zeros(x.shape[0], w.shape[2], dtype=torch.float64, device=x.device)
+    gx = torch.zeros_like(x64)
+    gw = torch.zeros_like(w64)
+    for r in range(w.shape[0]):
+        e = torch.nonzero(etype == r).squeeze(1)
+        for chunk in torch.split(e, 1 << 21):
+            s, d = idx[chunk], rows[chunk]
+            xs, gd = x64[s], g64[d]
+            out.index_add_(0, d, xs @ w64[r])
+            gx.index_add_(0, s, gd @ w64[r].t())
+            gw[r] += xs.t() @ gd
+    return out, gx, gw
+
+
+@pytest.fixture(scope="module")
+def hetero_ref(hetero):
+    announce("float64 torch reference of the relational layer at full size")
+    ref = _rgcn_float64(*hetero)
+    torch.cuda.synchronize()
+    return ref
+
+
+def _close_scaled(got, want, rtol, atol, what, floor=1.0):
+    """|got - want| <= atol * scale + rtol * |want| with scale = max(floor, max |want|), on the device."""
+    scale = max(floor, float(want.abs().max()))
+    err = (got.double() - want).abs()
+    tol = atol * scale + rtol * want.abs()
+    bad = err > tol
+    if bool(bad.any()):
+        i = int(torch.argmax(err - tol))
+        raise AssertionError("%s: %d of %d off; worst got %r want %r (err %.3e, tol %.3e)"
+                             % (what, int(bad.sum()), bad.numel(), float(got.flatten()[i]), float(want.flatten()[i]),
+                                float(err.flatten()[i]), float(tol.flatten()[i])))
+
+
+def test_c4_graph_shape(hetero):
+    ptr, idx, etype, rows, x, w, g = hetero
+    assert idx.shape[0] == C4_E and int(ptr[-1]) == C4_E and ptr.shape[0] == C4_N + 1
+    deg = ptr[1:] - ptr[:-1]
+    assert int(deg.min()) >= 1                       # the layer divides by the in-degree
+    cnt = torch.bincount(etype, minlength=C4_R)
+    assert int(cnt.min()) > 0 and bool((cnt[:-1] >= cnt[1:]).all())       # Zipf over the 16 relations
+    assert 0.2 < float(cnt[0]) / C4_E < 0.4
+
+
+def test_c4_aggr_rel_direct_full_size(hetero, hetero_ref):
+    """The fused relational aggregation, forward and both gradients, on every row against the
+    float64 reference; sampled rows against the CPU oracle; the identical-weights closed form
+    A (X W); run-to-run determinism."""
+    import cxgnncomp_backend as B
+    ptr, idx, etype, rows, x, w, g = hetero
+    want, want_gx, want_gw = hetero_ref
+    rel = etype.int()
+    xg = x.clone().requires_grad_(True)
+    wg = w.clone().requires_grad_(True)
+    announce("aggr_rel_direct fwd+bwd at 1M / 20M / 16")
+    out = B.aggr_rel_direct(xg, ptr, idx, wg, rel, C4_N, C4_R)
+    out.backward(g)
+    torch.cuda.synchronize()
+    _close_scaled(out.detach(), want, 1e-4, 1e-5, "rgcn fused forward, every row")
+    _close_scaled(xg.grad, want_gx, 1e-4, 1e-5, "rgcn fused grad x")
+    _close_scaled(wg.grad, want_gw, 1e-4, 1e-5, "rgcn fused grad W")
+    # sampled rows against the CPU oracle
+    rng = np.random.default_rng(2)
+    sel = np.unique(rng.integers(0, C4_N, 400))
+    sp, si, pos = _sub_csr(ptr, idx, sel)
+    ref = oracle.rgcn_fused(x.cpu().numpy(), sp, si, w.cpu().numpy(), rel[torch.from_numpy(pos).cuda()].cpu().numpy(),
+                            len(sel))
+    assert_close(out.detach()[torch.from_numpy(sel).cuda()].cpu().numpy(), ref, 1e-4, 1e-5, "sampled rows vs oracle")
+    # identical weights: sum_e x[idx[e]] W0 == A (x W0), the plain aggregation of transformed rows
+    w_same = w[:1].expand(C4_R, -1, -1).contiguous()
+    announce("aggr_rel_direct with identical weights == A (X W)")
+    got = B.aggr_rel_direct(x, ptr, idx, w_same, rel, C4_N, C4_R)
+    xw = (x.double() @ w[0].double())
+    axw = torch.zeros(C4_N, C4_K, dtype=torch.float64, device="cuda")
+    for chunk in torch.split(torch.arange(C4_E, device="cuda"), 1 << 22):
+        axw.index_add_(0, rows[chunk], xw[idx[chunk]])
+    _close_scaled(got, axw, 1e-4, 1e-5, "identical weights")
+    # no atomics on this path: bit-identical on a second run
+    again = B.aggr_rel_direct(x, ptr, idx, w, rel, C4_N, C4_R)
+    assert torch.equal(again, out.detach())
+
+
+@pytest.mark.parametrize("precision", [None, "bf16"])
+def test_c4_rgcn_layer_full_size(hetero, hetero_ref, precision):
+    """MyRGCNConv (typed transform, relational aggregate, division by the in-degree), forward
+    and backward, with fp32-accurate products and with bf16 operands.  bf16 tolerance: each
+    operand carries a relative rounding error of 2^-9, so a row of K = 128 products is compared
+    to 2e-2 of the output scale (the largest |value| of the reference)."""
+    import cxgnncomp
+    ptr, idx, etype, rows, x, w, g = hetero
+    want, want_gx, want_gw = hetero_ref          # of the sum; the layer divides by the degree
+    inv = 1.0 / (ptr[1:] - ptr[:-1]).double()
+    layer = cxgnncomp.MyRGCNConv(C4_K, C4_K, C4_R, precision=precision).cuda()
+    with torch.no_grad():
+        layer.linear.copy_(w)
+    xg = x.clone().requires_grad_(True)
+    announce("MyRGCNConv fwd+bwd at 1M / 20M / 16, precision=%s" % precision)
+    out = layer(xg, ptr, idx, etype, C4_N)
+    # feeding g * deg makes the gradient that reaches the aggregation equal g, so the float64
+    # gradients of the sum apply unchanged
+    out.backward(g * (ptr[1:] - ptr[:-1]).float()[:, None])
+    torch.cuda.synchronize()
+    rtol, atol, floor = (1e-4, 1e-5, 1.0) if precision is None else (2e-2, 2e-2, 0.0)
+    _close_scaled(out.detach(), want * inv[:, None], rtol, atol, "layer forward", floor)
+    _close_scaled(xg.grad, want_gx, rtol, atol, "layer grad x", floor)
+    _close_scaled(layer.linear.grad, want_gw, rtol, atol, "layer grad W", floor)
+    if precision == "bf16":
+        # the variant really multiplies rounded operands: it differs from the fp32-accurate result
+        exact = cxgnncomp.MyRGCNConv(C4_K, C4_K, C4_R).cuda()
+        with torch.no_grad():
+            exact.linear.copy_(w)
+            ref = exact(x, ptr, idx, etype, C4_N)
+        assert float((out.detach() - ref).abs().max()) > 0
+
+
+def test_c4_typed_linear_s2d_full_size(hetero, hetero_ref):
+    """typed_linear_s2d accumulates out[dst[e]] += x[src[e]] W[type[e]] into the caller's buffer:
+    with the CSR's (source, row, relation) triples that is the fused aggregation again."""
+    import cxgnncomp_backend as B
+    ptr, idx, etype, rows, x, w, g = hetero
+    want = hetero_ref[0]
+    out = torch.full((C4_N, C4_K), 0.5, device="cuda")          # accumulates onto what is there
+    announce("typed_linear_s2d at 20M rows")
+    B.typed_linear_s2d(x, w, out, idx, rows, etype.int())
+    torch.cuda.synchronize()
+    _close_scaled(out, want + 0.5, 1e-4, 1e-5, "typed_linear_s2d")
+
+
+def test_c4_rel_schedule_full_size(hetero):
+    """The 16 per-relation sub-graphs of the 20M-edge graph, bit for bit against the CPU oracle."""
+    import cxgnncomp_backend as B
+    ptr, idx, etype, rows, x, w, g = hetero
+    rel = etype.int()
+    layers = [C4_N // 100, C4_N // 10, C4_N, C4_N]
+    announce("rel_schedule at 20M edges")
+    got = B.rel_schedule(ptr, idx, rel, torch.tensor(layers), C4_R)
+    torch.cuda.synchronize()
+    want = oracle.rel_schedule(ptr.cpu().numpy(), idx.cpu().numpy(), rel.cpu().numpy(), layers, C4_R)
+    assert len(got) == len(want) == 3 * C4_R + 1
+    for k, (a, b) in enumerate(zip(got, want)):
+        assert a.dtype == torch.int64 and np.array_equal(a.cpu().numpy(), b), "output %d differs" % k
+    assert sum(int(got[3 * r + 1].shape[0]) for r in range(C4_R)) == C4_E
+
+
+# --------------------------------------------------------------------------- #
+# Sampled mini-batch at its stated size: 1,024 seeds, fanouts 15 / 10 / 5, 111M-id space
+# --------------------------------------------------------------------------- #
+@pytest.fixture(scope="module")
+def sampled():
+    from cxgnncomp import synthetic as S
+    announce("generate the 1,024-seed sampled batch")
+    ptr, idx, nn, ne = S.sampled_batch(seed=0)              # defaults are the stated configuration
+    torch.manual_seed(5)
+    x = torch.randn(nn[-1], 128)
+    return ptr, idx, nn, ne, x
+
+
+def test_c5_batch_shape(sampled):
+    ptr, idx, nn, ne, x = sampled
+    # every node first reached at hop h - 1 draws fanout[h] neighbours; collisions in a 111M-id
+    # space are rare, so the realised sizes sit just below 1,024 x (1, 16, 166, 916)
+    assert nn[0] == 1024 and ne[0] == 15360
+    assert ne[1] == ne[0] + 10 * (nn[1] - nn[0]) and ne[2] == ne[1] + 5 * (nn[2] - nn[1])
+    assert 16300 <= nn[1] <= 16384 and 169000 <= nn[2] <= 169984 and 930000 <= nn[3] <= 937984
+    assert int(ptr[nn[2]]) == ne[2] and idx.shape[0] == ne[2] and int(idx.max()) == nn[3] - 1
+
+
+def test_c5_sage_mean_prefix_layers_full_size(sampled):
+    """The three sage_mean_forward calls of a batch (rows 169,984 / 16,384 / 1,024 over edge
+    prefixes of one nested CSR), forward and backward, every row against the oracle."""
+    import cxgnncomp_backend as B
+    ptr, idx, nn, ne, x = sampled
+    ptr_d, idx_d = ptr.cuda(), idx.cuda()
+    for layer in (2, 1, 0):
+        rows, n_src = nn[layer], nn[layer + 1]
+        xs = x[:n_src].contiguous()
+        xg = xs.cuda().requires_grad_(True)
+        announce("sage_mean_forward rows=%d edges=%d" % (rows, ne[layer]))
+        out = B.sage_mean_forward(xg, ptr_d, idx_d, rows)
+        torch.manual_seed(layer)
+        g = torch.randn(rows, 128)
+        out.backward(g.cuda())
+        torch.cuda.synchronize()
+        ref = oracle.spmm(ptr.numpy(), idx.numpy(), xs.numpy(), rows, mean=True)
+        assert out.shape == (rows, 128)
+        assert_close(out.detach().cpu().numpy(), ref, 1e-4, 1e-5, "mean forward, layer %d" % layer)
+        ref_g = oracle.spmm_bwd(ptr.numpy(), idx.numpy(), g.numpy(), rows, n_src, mean=True)
+        assert_close(xg.grad.cpu().numpy(), ref_g, 1e-4, 1e-5, "mean backward, layer %d" % layer)
+
+
+def test_c5_sage_model_full_size(sampled):
+    """3-layer SAGE 128 -> 256 -> 256 -> 47 on the full batch, logits, input gradient and the first
+    layer's weight gradient against a float64 restatement of the stack on the host.
+
+    The forward pass is continuous, the gradient is not: a ReLU input that the float64
+    reference puts within fp32 rounding of zero (a handful of the 48 million) may fall on the other
+    side in fp32, which switches that unit's whole gradient path.  The input rows such a unit
+    reaches (its own row and its neighbours, one or two hops down) are left out of the
+    gradient comparison; they must be a negligible share of the rows."""
+    import copy
+
+    import torch.nn.functional as F
+
+    import cxgnncomp
+    from oracle import pyref
+    ptr, idx, nn, ne, x = sampled
+    b = cxgnncomp.Batch(x, ptr, idx, torch.tensor(nn), torch.tensor(ne))
+    torch.manual_seed(7)
+    model = cxgnncomp.SAGE(128, 256, 47, 3, 0.0, "CSR_Layer")
+    ref = copy.deepcopy(model).double()
+    x64 = x.double().requires_grad_(True)
+
+    def mean64(h, rows):
+        s = pyref.spmm_torch(h, ptr, idx, rows, torch.ones(idx.shape[0], dtype=h.dtype))
+        deg = (ptr[1:rows + 1] - ptr[:rows]).double().unsqueeze(1)
+        return torch.where(deg > 0, s / deg.clamp(min=1), torch.zeros_like(s))
+
+    p_np, i_np = ptr.numpy(), idx.numpy()
+
+    def with_sources(rows_set):
+        """The rows and the sources of their edges."""
+        if len(rows_set) == 0:
+            return rows_set
+        src = np.concatenate([i_np[p_np[r]:p_np[r + 1]] for r in rows_set])
+        return np.unique(np.concatenate([rows_set, src]))
+
+    h = x64
+    skip = np.zeros(0, dtype=np.int64)                    # input rows behind an ambiguous ReLU
+    for i, conv in enumerate(ref.convs):
+        rows = nn[2 - i]
+        if conv.in_channels > conv.hidden_channels:
+            out = mean64(conv.lin_l(h), rows)
+        else:
+            out = conv.lin_l(mean64(h, rows))
+        h = out + conv.lin_r(h[:rows])
+        if i < 2:
+            bn = ref.bns[i]
+            h = F.batch_norm(h, None, None, bn.weight, bn.bias, True, 0.0, bn.eps)
+            near = np.nonzero((h.detach().abs() < 3e-6).any(1).numpy())[0]
+            for _ in range(i + 1):                        # down to the rows of x
+                near = with_sources(near)
+            skip = np.union1d(skip, near)
+            h = F.relu(h)
+    assert len(skip) < 5e-3 * nn[3]
+    keep = np.setdiff1d(np.arange(nn[3]), skip)
+    want = h.log_softmax(-1)
+    g = torch.randn(nn[0], 47, dtype=torch.float64) / 8
+    want.backward(g)
+    announce("SAGE 128-256-256-47 on the full sampled batch")
+    model = model.cuda()
+    gb = copy.copy(b).to("cuda")
+    gb.x = x.cuda().requires_grad_(True)
+    got = model(gb)
+    got.backward(g.float().cuda())
+    torch.cuda.synchronize()
+    assert got.shape == (1024, 47)
+    assert_close(got.detach().cpu().numpy(), want.detach().numpy(), 2e-4, 2e-5, "SAGE logits")
+    # the gradient shrinks by orders of magnitude from hop to hop: every hop's rows are compared at
+    # that hop's own scale
+    gx_got, gx_want = gb.x.grad.cpu().numpy(), x64.grad.numpy()
+    for lo, hi in zip([0] + nn[:-1], nn):
+        rows = keep[(keep >= lo) & (keep < hi)]
+        sc = float(np.abs(gx_want[lo:hi]).max())
+        assert_close(gx_got[rows] / sc, gx_want[rows] / sc, 2e-4, 2e-5, "SAGE grad x, rows %d..%d" % (lo, hi))
+    # A weight gradient sums over all 170 k rows, the ambiguous ones included: each of them moves a
+    # whole row of the gradient by about 1e-3 of its size, so the matrices are compared in norm
+    # (a dropped term, a wrong scale or a transposed operand is an O(1) error there).
+    for name, got_p, want_p in (("lin_l", model.convs[0].lin_l.weight.grad, ref.convs[0].lin_l.weight.grad),
+                                ("lin_r", model.convs[0].lin_r.weight.grad, ref.convs[0].lin_r.weight.grad),
+                                ("last lin_l", model.convs[2].lin_l.weight.grad, ref.convs[2].lin_l.weight.grad)):
+        wg, wr = got_p.cpu().numpy().astype(np.float64), want_p.numpy()
+        rel = np.linalg.norm(wg - wr) / np.linalg.norm(wr)
+        assert rel < 1e-3, "SAGE grad %s: relative error in norm %.3e" % (name, rel)
+    # the last layer sits above every ReLU: its weight gradient is compared element by element
+    wg, wr = model.convs[2].lin_r.weight.grad.cpu().numpy(), ref.convs[2].lin_r.weight.grad.numpy()
+    scw = float(np.abs(wr).max())
+    assert_close(wg / scw, wr / scw, 2e-4, 2e-5, "SAGE grad lin_r of the last layer")
