@@ -21,5 +21,6 @@ from .batch import Batch, PyGBatch
 from .util import global_tuner
 from .graph_kernel import SpMMValOP
 from .batchnorm import BatchNorm1d
-from .model import GNN, SAGE, GCN, GIN, GAT, RGCN
+from .model import (GNN, SAGE, GCN, GIN, GAT, RGCN, get_model, get_conv_from_str, get_model_from_str,
+                    graph_type_dict, model_dict)
 from . import synthetic  # noqa: F401

@@ -153,3 +153,88 @@ class RGCN(GNN):
         if self.graph_type == "CSR_Layer":
             et = et[:int(batch.num_edge_in_layer[self.num_layer - 1 - i])]
         return conv(x, batch.ptr, batch.idx, et, self._rows(batch, i))
+
+
+# --------------------------------------------------------------------------- #
+# Factories (cxgnncomp/model.py:345-467)
+# --------------------------------------------------------------------------- #
+graph_type_dict = {
+    "cxg": "CSR_Layer",
+    "dgl": "DGL",
+    "pyg": "PyG",
+}
+
+model_dict = {
+    "gcn": GCN,
+    "gat": GAT,
+    "gin": GIN,
+    "rgcn": RGCN,
+    "sage": SAGE,
+}
+
+
+def _item(node, key, default=None):
+    """``node[key]`` / ``node.key`` of a config node (omegaconf, dict or plain namespace)."""
+    if isinstance(node, dict):
+        return node.get(key, default)
+    getter = getattr(node, "get", None)
+    if callable(getter):
+        try:
+            return getter(key, default)
+        except TypeError:
+            pass
+    return getattr(node, key, default)
+
+
+def get_model(config):
+    """Model from a training configuration (cxgnncomp/model.py:362-399): reads
+    ``dl.dataset.{feature_dim, num_classes, name}``, ``dl.sampler.train.num_layer``,
+    ``train.type`` (cxg / dgl / pyg) and ``train.model.{type, hidden_dim, dropout, heads, concat,
+    num_rel}``.  The dgl / pyg graph types raise NotImplementedError."""
+    dataset = config.dl.dataset
+    spec = config.train.model
+    kind = str(_item(spec, "type")).lower()
+    graph_type = graph_type_dict[str(config.train.type).lower()]
+    args = (_item(dataset, "feature_dim"), _item(spec, "hidden_dim"), _item(dataset, "num_classes"),
+            config.dl.sampler.train.num_layer, _item(spec, "dropout"), graph_type, config)
+    if "gat" in kind:
+        return model_dict[kind](*args, heads=_item(spec, "heads", 1), concat=_item(spec, "concat", False))
+    if "rgcn" in kind:
+        return model_dict[kind](*args, num_rel=int(_item(spec, "num_rel")),
+                                dataset_name=str(_item(dataset, "name")).lower())
+    return model_dict[kind](*args)
+
+
+def get_conv_from_str(model_str, infeat, outfeat, num_head=-1, num_rel=-1):
+    """One convolution layer by name (cxgnncomp/model.py:402-414)."""
+    model_str = model_str.lower()
+    if model_str == "gat":
+        return MyGATConv(infeat, outfeat, heads=num_head)
+    if model_str == "gcn":
+        return MyGCNConv(infeat, outfeat)
+    if model_str == "sage":
+        return MySageConv(infeat, outfeat)
+    if model_str == "rgcn":
+        return MyRGCNConv(infeat, outfeat, num_rel=num_rel)
+    assert False, f"unknown model {model_str}"
+
+
+def get_model_from_str(mtype, infeat, hiddenfeat, outfeat, graph_type, num_layer, num_head=-1, num_rel=-1,
+                       dataset=None, dropout=0.5):
+    """One layer stack by name (cxgnncomp/model.py:417-467).  ``LSTM`` (the neighbour-LSTM
+    aggregator) is outside this package."""
+    mtype = mtype.upper()
+    common = dict(dropout=dropout, graph_type=graph_type, config=None)
+    if mtype == "GCN":
+        return GCN(infeat, hiddenfeat, outfeat, num_layer, **common)
+    if mtype == "GAT":
+        return GAT(infeat, hiddenfeat, outfeat, num_layer, heads=num_head, **common)
+    if mtype == "SAGE":
+        return SAGE(infeat, hiddenfeat, outfeat, num_layer, **common)
+    if mtype == "RGCN":
+        return RGCN(infeat, hiddenfeat, outfeat, num_layer, num_rel=num_rel, dataset_name=dataset, **common)
+    if mtype == "GIN":
+        return GIN(infeat, hiddenfeat, outfeat, num_layer, **common)
+    if mtype == "LSTM":
+        raise NotImplementedError("the neighbour-LSTM model (cxgnncomp/neighbor_lstm.py) is not part of this package")
+    assert False, f"unknown model {mtype}"

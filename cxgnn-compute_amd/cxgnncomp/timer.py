@@ -1,6 +1,13 @@
-"""Named wall-clock timers and the autograd marker op the conv layers call
-(cxgnncomp/timer.py:7-164).  Timers are created skipped (no-ops) exactly as
-upstream; ``get_timers()`` needs ``set_timers()`` first."""
+"""Named stage timers behind the reference's names (cxgnncomp/timer.py): ``set_timers()`` installs
+a process-wide ``Timers`` registry, ``get_timers()`` returns it (and asserts that it was installed),
+``TimerOP`` is an identity autograd function that opens / closes the stage ``<name>_fwd`` in the
+forward pass and ``<name>_bwd`` in the backward pass, ``TimerModule`` wraps a module in such a pair.
+
+Every stopwatch starts out with ``skip = True`` and then costs nothing: no device synchronisation,
+no clock read.  Clearing ``skip`` on a stopwatch makes it measure wall-clock seconds between
+``start()`` and ``stop()``, each taken after the device has drained.  The report lines keep the
+reference's layout, ``time (ms) | <name>: <milliseconds per call>``.
+"""
 import time
 
 import torch
@@ -8,84 +15,99 @@ import torch
 _GLOBAL_TIMERS = None
 
 
-class _Timer:
+def _drain_device():
+    if torch.cuda.is_available() and torch.cuda.is_initialized():
+        torch.cuda.synchronize()
+
+
+class _Stopwatch:
+    """Accumulated wall time and number of completed start/stop pairs of one named stage."""
 
     def __init__(self, name):
-        self.name_ = name
-        self.elapsed_ = 0.0
+        self.name = name
+        self.skip = True
+        self.total_s = 0.0
         self.num_call = 0
-        self.started_ = False
-        self.start_time = time.time()
+        self.opened_at = None          # perf_counter() of the pending start(), None when closed
         self.input_shape = None
         self.output_shape = None
-        self.skip = True
+
+    @property
+    def running(self):
+        return self.opened_at is not None
 
     def start(self):
         if self.skip:
             return
-        assert not self.started_, "timer" + self.name_ + "has already been started"
-        torch.cuda.synchronize()
-        self.start_time = time.time()
-        self.started_ = True
+        assert not self.running, "timer %s was started twice" % self.name
+        _drain_device()
+        self.opened_at = time.perf_counter()
 
     def stop(self):
         if self.skip:
             return
-        assert self.started_, "timer" + self.name_ + " is not started"
-        torch.cuda.synchronize()
-        self.elapsed_ += time.time() - self.start_time
+        assert self.running, "timer %s was stopped without a start" % self.name
+        _drain_device()
+        self.total_s += time.perf_counter() - self.opened_at
         self.num_call += 1
-        self.started_ = False
+        self.opened_at = None
 
     def reset(self):
         if self.skip:
             return
-        self.elapsed_ = 0.0
-        self.started_ = False
-        self.num_call = 0
+        self.total_s, self.num_call, self.opened_at = 0.0, 0, None
 
     def elapsed(self, reset=True):
+        """(seconds, calls) accumulated so far, or None while the stopwatch is skipping."""
         if self.skip:
-            return
-        assert not self.started_, "timer" + self.name_ + "is still started"
-        out = (self.elapsed_, self.num_call)
+            return None
+        assert not self.running, "timer %s is still running" % self.name
+        result = (self.total_s, self.num_call)
         if reset:
             self.reset()
-        return out
+        return result
 
 
 class Timers:
+    """Registry of stopwatches; calling it with a name returns (and on first use creates) one."""
 
     def __init__(self):
         self.timers = {}
 
     def __call__(self, name):
-        if name not in self.timers:
-            self.timers[name] = _Timer(name)
-        return self.timers[name]
+        watch = self.timers.get(name)
+        if watch is None:
+            watch = self.timers[name] = _Stopwatch(name)
+        return watch
+
+    @staticmethod
+    def _ms_per(watch, divisor, reset):
+        got = watch.elapsed(reset=reset) if watch is not None else None
+        if got is None:
+            return 0.0
+        seconds, calls = got
+        d = calls if divisor is None else divisor
+        return seconds * 1000.0 / d if d else 0.0
 
     def log(self, log_fn, names, normalizer=1.0, reset=True):
+        """One line with the given stages, milliseconds divided by ``normalizer``."""
         assert normalizer > 0.0
         parts = ["time (ms)"]
         for name in names:
-            ms = 0
-            if name in self.timers:
-                got = self.timers[name].elapsed(reset=reset)
-                ms = got[0] * 1000.0 / normalizer if got else 0
-            parts.append("{}: {:.2f}".format(name, ms))
+            parts.append("%s: %.2f" % (name, self._ms_per(self.timers.get(name), normalizer, reset)))
         log_fn(" | ".join(parts))
 
     def log_all(self, log_fn, normalizer=1.0, reset=True):
+        """One line with every stage in name order, milliseconds per completed call; stages that
+        recorded shapes (TimerModule(report_shape=True)) append them."""
         assert normalizer > 0.0
         parts = ["time (ms)"]
         for name in sorted(self.timers):
-            t = self.timers[name]
-            got = t.elapsed(reset=reset)
-            ms = got[0] * 1000.0 / got[1] if got and got[1] else 0.0
-            text = "{}: {:.2f}".format(name, ms)
-            if t.input_shape is not None:
-                text += "| {}: in:{} out:{}".format(name, t.input_shape, t.output_shape)
-            parts.append(text)
+            watch = self.timers[name]
+            item = "%s: %.2f" % (name, self._ms_per(watch, None, reset))
+            if watch.input_shape is not None:
+                item += "| %s: in:%s out:%s" % (name, watch.input_shape, watch.output_shape)
+            parts.append(item)
         log_fn(" | ".join(parts))
 
 
@@ -95,37 +117,39 @@ def set_timers():
 
 
 def get_timers():
-    assert _GLOBAL_TIMERS is not None
+    assert _GLOBAL_TIMERS is not None, "call set_timers() first"
     return _GLOBAL_TIMERS
 
 
 class TimerOP(torch.autograd.Function):
-    """Identity in value; starts/stops ``<name>_fwd`` in forward and ``<name>_bwd``
-    (in the opposite order) in backward."""
+    """``TimerOP.apply(tensor, name, is_front)`` returns ``tensor``.  The front marker opens
+    ``<name>_fwd`` and the back marker closes it; in the backward pass, which meets the markers in
+    the opposite order, the back marker opens ``<name>_bwd`` and the front marker closes it."""
 
     @staticmethod
     def forward(ctx, input, timer_name, is_front):
-        timers = get_timers()
+        watch = get_timers()(timer_name + "_fwd")
         if is_front:
-            timers(timer_name + "_fwd").start()
+            watch.start()
         else:
-            timers(timer_name + "_fwd").stop()
-        ctx.timer_name = timer_name
-        ctx.is_front = is_front
+            watch.stop()
+        ctx.stage = (timer_name, is_front)
         return input
 
     @staticmethod
-    def backward(ctx, grad_in):
-        timers = get_timers()
-        name = ctx.timer_name + "_bwd"
-        if ctx.is_front:
-            timers(name).stop()
+    def backward(ctx, grad):
+        name, is_front = ctx.stage
+        watch = get_timers()(name + "_bwd")
+        if is_front:
+            watch.stop()
         else:
-            timers(name).start()
-        return grad_in, None, None
+            watch.start()
+        return grad, None, None
 
 
 class TimerModule(torch.nn.Module):
+    """``model`` bracketed by a TimerOP pair named ``timer_name``; with ``report_shape`` the input
+    and output shapes are kept on the stage ``<timer_name>_shape``."""
 
     def __init__(self, model, timer_name, report_shape=False):
         super().__init__()
@@ -135,10 +159,8 @@ class TimerModule(torch.nn.Module):
 
     def forward(self, input):
         input = TimerOP.apply(input, self.timer_name, True)
-        output = self.model(input)
-        output = TimerOP.apply(output, self.timer_name, False)
+        output = TimerOP.apply(self.model(input), self.timer_name, False)
         if self.report_shape:
-            t = get_timers()(self.timer_name + "_shape")
-            t.input_shape = input.shape
-            t.output_shape = output.shape
+            watch = get_timers()(self.timer_name + "_shape")
+            watch.input_shape, watch.output_shape = input.shape, output.shape
         return output

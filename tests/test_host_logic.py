@@ -303,17 +303,94 @@ def test_synthetic_graphs_have_the_configured_shapes():
 
 
 def test_batch_round_trip(tmp_path):
+    """The reference's container (cxgnncomp/batch.py:7-90): target as the sixth argument,
+    x.dat / ptr.dat / idx.dat / target.dat as flat numpy images, an instance fromfile that leaves
+    every tensor flat, totype, and the two-argument PyGBatch."""
     import cxgnncomp
     from cxgnncomp import synthetic as S
     ptr, idx, nn, ne = S.sampled_batch(num_seeds=16, fanouts=(3, 2), id_space=5000, seed=2)
     x = torch.randn(nn[-1], 8)
-    b = cxgnncomp.Batch(x, ptr, idx, nn, ne)
+    target = torch.arange(ptr.shape[0] - 1) * 3
+    b = cxgnncomp.Batch(x, ptr, idx, nn, ne, target)
+    assert b.target is target and b.block is None and b.edge_index is None
     b.tofile(str(tmp_path))
-    raw = np.fromfile(str(tmp_path / "ptr.dat"), dtype="<i8")
-    assert np.array_equal(raw, ptr.numpy())
-    b2 = cxgnncomp.Batch.fromfile(str(tmp_path), 8)
-    assert torch.equal(b2.x, x) and torch.equal(b2.ptr, ptr) and torch.equal(b2.idx, idx)
-    assert b2.num_node_in_layer.tolist() == nn and b2.num_edge_in_layer.tolist() == ne
+    assert np.array_equal(np.fromfile(str(tmp_path / "ptr.dat"), dtype="<i8"), ptr.numpy())
+    assert np.array_equal(np.fromfile(str(tmp_path / "target.dat"), dtype="<i8"), target.numpy())
+    assert np.array_equal(np.fromfile(str(tmp_path / "x.dat"), dtype="<f4"), x.numpy().ravel())
+    # instance method, as upstream: fills the object, x stays flat
+    b2 = cxgnncomp.Batch(None, None, None)
+    assert b2.fromfile(str(tmp_path)) is None
+    assert torch.equal(b2.x, x.flatten()) and torch.equal(b2.ptr, ptr) and torch.equal(b2.idx, idx)
+    assert torch.equal(b2.target, target)
+    # the ready-to-use loader
+    b3 = cxgnncomp.Batch.load(str(tmp_path), 8)
+    assert torch.equal(b3.x, x) and torch.equal(b3.target, target)
+    assert b3.num_node_in_layer.tolist() == nn and b3.num_edge_in_layer.tolist() == ne
+    b3.totype(torch.int32)
+    assert b3.ptr.dtype == b3.idx.dtype == b3.target.dtype == torch.int32
+    assert torch.equal(b3.ptr.long(), ptr)
+    assert b3.to("cpu") is b3
+    with pytest.raises(NotImplementedError):
+        b3.todgl(4, 2)
+    # a batch without target writes no target.dat, and fromfile leaves target alone
+    d2 = tmp_path / "no_target"
+    cxgnncomp.Batch(x, ptr, idx).tofile(str(d2))
+    assert not (d2 / "target.dat").exists()
+    pg = cxgnncomp.PyGBatch(x, torch.stack([idx, idx]))
+    assert pg.x is x and pg.edge_index.shape[0] == 2
+    with pytest.raises(TypeError):
+        cxgnncomp.PyGBatch(x, ptr, idx)
+
+
+def test_model_factories_build_the_reference_layouts():
+    """get_conv_from_str / get_model_from_str / get_model (cxgnncomp/model.py:362-467) for the CSR
+    graph types: classes, layer widths and state-dict keys of the reference's modules."""
+    import types
+
+    import cxgnncomp
+    from cxgnncomp import get_conv_from_str, get_model, get_model_from_str
+    for name, cls in (("gat", cxgnncomp.MyGATConv), ("GCN", cxgnncomp.MyGCNConv), ("sage", cxgnncomp.MySageConv),
+                      ("rgcn", cxgnncomp.MyRGCNConv)):
+        conv = get_conv_from_str(name, 8, 16, num_head=2, num_rel=3)
+        assert type(conv) is cls
+    with pytest.raises(AssertionError):
+        get_conv_from_str("hgt", 8, 16)
+    bn = {"bns.0." + k for k in ("weight", "bias", "running_mean", "running_var", "num_batches_tracked")}
+    conv_keys = {
+        "GCN": {"bias", "lin.weight"},
+        "SAGE": {"lin_l.weight", "lin_l.bias", "lin_r.weight"},
+        "GAT": {"att_src", "att_dst", "bias", "lin_src"},
+        "RGCN": {"linear", "rel_weight", "single_linear.weight", "single_linear.bias"},
+    }
+    for mtype, keys in conv_keys.items():
+        m = get_model_from_str(mtype, 8, 16, 4, "CSR_Layer", 2, num_head=2, num_rel=3, dataset="x")
+        assert type(m) is getattr(cxgnncomp, mtype) and m.dropout == 0.5 and len(m.convs) == 2
+        want = bn | {"convs.%d.%s" % (i, k) for i in range(2) for k in keys}
+        assert set(m.state_dict()) == want, mtype
+    assert get_model_from_str("sage", 8, 16, 4, "CSR", 3).convs[2].lin_l.weight.shape == (4, 16)
+    with pytest.raises(NotImplementedError):
+        get_model_from_str("GCN", 8, 16, 4, "DGL", 2)
+    with pytest.raises(NotImplementedError):
+        get_model_from_str("LSTM", 8, 16, 4, "CSR_Layer", 2)
+    with pytest.raises(AssertionError):
+        get_model_from_str("MLP", 8, 16, 4, "CSR_Layer", 2)
+
+    def config(model, train_type="cxg"):
+        ns = types.SimpleNamespace
+        return ns(dl=ns(dataset=ns(feature_dim=8, num_classes=4, name="Arxiv"),
+                        sampler=ns(train=ns(num_layer=3))),
+                  train=ns(type=train_type, model=model))
+    m = get_model(config({"type": "SAGE", "hidden_dim": 16, "dropout": 0.25}))
+    assert type(m) is cxgnncomp.SAGE and m.graph_type == "CSR_Layer" and m.num_layer == 3 and m.dropout == 0.25
+    assert m.convs[0].lin_l.weight.shape == (16, 8) and m.convs[2].lin_l.weight.shape == (4, 16)
+    m = get_model(config({"type": "gat", "hidden_dim": 16, "dropout": 0.0, "heads": 4, "concat": True}))
+    assert type(m) is cxgnncomp.GAT and m.convs[0].heads == 4 and m.convs[0].att_src.shape == (1, 4, 4)
+    m = get_model(config({"type": "rgcn", "hidden_dim": 16, "dropout": 0.0, "num_rel": "7"}))
+    assert type(m) is cxgnncomp.RGCN and m.convs[0].linear.shape == (7, 8, 16) and m.dataset_name == "arxiv"
+    m = get_model(config(types.SimpleNamespace(type="gin", hidden_dim=16, dropout=0.0)))
+    assert type(m) is cxgnncomp.GIN
+    with pytest.raises(NotImplementedError):
+        get_model(config({"type": "gcn", "hidden_dim": 16, "dropout": 0.0}, train_type="dgl"))
 
 
 def test_topo_sort_matches_restatement(capsys):

@@ -503,3 +503,27 @@ def test_batchnorm_restatement_matches_torch_and_autograd(relu, affine):
     if not relu and not affine:
         assert np.allclose(y.mean(axis=0), 0, atol=1e-12)
         assert np.allclose(y.var(axis=0), var / (var + eps), rtol=1e-12)
+
+
+def test_gcn_norm_is_one_over_the_row_degree():
+    """pyref.gcn_norm (MyGCNConv.gcn_norm, cxgnncomp/graph_conv.py:587-596): every edge of row r
+    carries 1 / deg(r).  Pinned by a hand case with an empty row, by the closed form on a random
+    graph, by the C restatement of edge_value_degree, and by what it is for: with these weights
+    the weighted aggregation of all-ones features is 1 in every non-empty row (a row mean)."""
+    ptr = torch.tensor([0, 2, 2, 3, 7])
+    idx = torch.tensor([1, 3, 0, 0, 1, 2, 3])
+    assert pyref.gcn_norm(ptr, idx).tolist() == [0.5, 0.5, 1.0, 0.25, 0.25, 0.25, 0.25]
+    rng = np.random.default_rng(8)
+    deg = rng.integers(0, 9, 300)
+    deg[::7] = 0
+    p = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    E = int(p[-1])
+    i = rng.integers(0, 300, E)
+    ev = pyref.gcn_norm(torch.from_numpy(p), torch.from_numpy(i)).numpy()
+    rows = np.repeat(np.arange(300), deg)
+    assert ev.dtype == np.float32 and ev.shape == (E,)
+    assert np.array_equal(ev, (1.0 / deg[rows]).astype(np.float32))
+    assert np.array_equal(ev, oracle.edge_value_degree(p, 300, E))
+    a = sp.csr_matrix((ev.astype(np.float64), i, p), shape=(300, 300))
+    sums = np.asarray(a @ np.ones(300))
+    assert np.allclose(sums[deg > 0], 1.0, atol=1e-6) and np.all(sums[deg == 0] == 0)
