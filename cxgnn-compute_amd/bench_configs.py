@@ -479,11 +479,22 @@ def c5(iters):
                timeit(lambda: B.sage_mean_forward(x, ptr, idx, rows), iters), spmm_bytes(rows, edges, 128), edges * 128)
     from cxgnncomp_backend import _ops
 
+    def prepare_sorts():
+        # the reversed graph of each layer by its own stable sort
+        for li, rows in enumerate(nn[2::-1]):
+            _ops.csr_transpose(ptr, idx, rows, nn[3 - li])
+
     def prepare():
-        # what a NEW batch pays once before its first backward: the reversed graph of each layer
-        for rows in nn[2::-1]:
-            _ops.csr_transpose(ptr, idx, rows, n_src)
-    report("c5", "per-batch preparation: reversed CSR of the 3 layers (stable sort + fills)", timeit(prepare, iters))
+        # what a NEW batch pays once before its first backward: the reversed graph of the largest
+        # layer by a stable sort, the two smaller ones cut out of it (they are edge prefixes)
+        _ops.clear_graph_cache()
+        for li, rows in enumerate(nn[2::-1]):
+            _ops.note_layer(ptr, idx, rows, nn[3 - li])
+        for li, rows in enumerate(nn[:3]):
+            _ops.transposed(ptr, idx, rows, nn[li + 1])
+    report("c5", "per-batch preparation, three stable sorts: reversed CSR of the 3 layers", timeit(prepare_sorts, iters))
+    report("c5", "per-batch preparation: reversed CSR of the largest layer (stable sort + fills), the two smaller "
+                 "ones compacted out of it", timeit(prepare, iters))
     xg = x.clone().requires_grad_(True)
 
     def batch_step():
@@ -494,9 +505,15 @@ def c5(iters):
             if li < 2:
                 h = torch.relu(h)
         h.sum().backward()
-    report("c5", "3-layer SAGE fwd+bwd per batch (%s nodes per layer)" % nn, timeit(batch_step, iters),
-           note="60 kernel launches per batch, 12 of them this library's (6 aggregations x span + fix-up); "
-                "counted with a rocprofv3 kernel trace of 10 vs 20 steps")
+    launches = "kernel launches per batch counted with rocprofv3 kernel traces of 10 and 20 steps"
+    report("c5", "3-layer SAGE fwd+bwd per batch, reversed graphs cached (%s nodes per layer)" % nn,
+           timeit(batch_step, iters), note=launches)
+
+    def new_batch_step():
+        _ops.clear_graph_cache()                 # a new sampled batch: nothing of the graph is cached
+        batch_step()
+    report("c5", "3-layer SAGE fwd+bwd per NEW batch, preparation of the reversed graphs included",
+           timeit(new_batch_step, iters), note=launches)
     if CPU_BASELINE:
         cpu_spmm("c5", ptr, idx, n_src, 128, nn[2])
 

@@ -79,18 +79,6 @@ __device__ __forceinline__ void stream_store(float* p, float4 v) {
   f4_t t = {v.x, v.y, v.z, v.w};
   __builtin_nontemporal_store(t, reinterpret_cast<f4_t*>(p));
 }
-__device__ __forceinline__ float stream_load_vec(const float* p, float) { return __builtin_nontemporal_load(p); }
-__device__ __forceinline__ float2 stream_load_vec(const float* p, float2) {
-  typedef float f2_t __attribute__((ext_vector_type(2)));
-  const f2_t t = __builtin_nontemporal_load(reinterpret_cast<const f2_t*>(p));
-  return make_float2(t.x, t.y);
-}
-__device__ __forceinline__ float4 stream_load_vec(const float* p, float4) {
-  typedef float f4_t __attribute__((ext_vector_type(4)));
-  const f4_t t = __builtin_nontemporal_load(reinterpret_cast<const f4_t*>(p));
-  return make_float4(t.x, t.y, t.z, t.w);
-}
-
 // First index i in [0, n) with a[i] >= key (n if none); `a` is non-decreasing.
 // All 64 lanes cooperate: each round probes 64 evenly spaced elements, so the
 // search finishes in ceil(log64(n)) dependent memory round trips.

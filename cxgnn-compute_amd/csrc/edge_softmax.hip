@@ -238,6 +238,21 @@ template <int N> __device__ __forceinline__ void store_f(float* __restrict__ p, 
     for (int i = 0; i < N; ++i) p[i] = v[i];
   }
 }
+// The same for data that is written once and not read again by this launch (non-temporal:
+// it should not displace the gathered logits from the L2).
+template <int N> __device__ __forceinline__ void store_f_stream(float* __restrict__ p, const float (&v)[N]) {
+  if constexpr (N == 4) {
+    stream_store(p, make_float4(v[0], v[1], v[2], v[3]));
+  } else if constexpr (N == 2) {
+    stream_store(p, make_float2(v[0], v[1]));
+  } else if constexpr (N == 8) {
+    stream_store(p, make_float4(v[0], v[1], v[2], v[3]));
+    stream_store(p + 4, make_float4(v[4], v[5], v[6], v[7]));
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; ++i) stream_store(p + i, v[i]);
+  }
+}
 template <int N> __device__ __forceinline__ void load_b(const uint8_t* __restrict__ p, bool (&v)[N]) {
   if constexpr (N == 4 || N == 8) {
 #pragma unroll
@@ -258,7 +273,7 @@ template <int N> __device__ __forceinline__ void store_b(uint8_t* __restrict__ p
       uint32_t t = 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) t |= (v[4 * w + i] ? 1u : 0u) << (8 * i);
-      reinterpret_cast<uint32_t*>(p)[w] = t;
+      __builtin_nontemporal_store(t, reinterpret_cast<uint32_t*>(p) + w);
     }
   } else {
 #pragma unroll
@@ -504,7 +519,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_walk_kernel(
     const int64_t k = w.eb + (rel < w.total ? rel : w.total - 1);
     const int64_t r = first_row + row;
     float a[H], d[H], t[H], mx[H], p[H];
-    load_f<H>(att_src + idx[k] * H, a);
+    load_f<H>(att_src + stream_load(idx + k) * H, a);
     load_f<H>(att_dst + (r < n_rows ? r : n_rows - 1) * H, d);
 #pragma unroll
     for (int h = 0; h < H; ++h) mx[h] = t[h] = leaky(d[h] + a[h], slope);
@@ -544,7 +559,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_walk_kernel(
       mk[h] = t[h] > 0.f;
     }
     if (act) {
-      store_f<H>(out + k * H, o);
+      store_f_stream<H>(out + k * H, o);
       store_b<H>(mask + k * H, mk);
     }
   }
@@ -561,7 +576,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_walk_kernel(
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
         kk[u] = k + u * sc.nl;
-        src[u] = idx[kk[u] < e ? kk[u] : e - 1];
+        src[u] = stream_load(idx + (kk[u] < e ? kk[u] : e - 1));
       }
 #pragma unroll
       for (int u = 0; u < kU; ++u) load_f<H>(att_src + src[u] * H, a[u]);
@@ -598,7 +613,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_walk_kernel(
             o[h] = __expf(t[u][h] - bm[h]) * bsum[h];
             mk[h] = t[u][h] > 0.f;
           }
-          store_f<H>(out + kk[u] * H, o);
+          store_f_stream<H>(out + kk[u] * H, o);
           store_b<H>(mask + kk[u] * H, mk);
         }
     }

@@ -5,6 +5,7 @@
 
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
 #include <rocprim/iterator/transform_iterator.hpp>
 
@@ -131,6 +132,34 @@ __global__ void pad_rel_kernel(int64_t* __restrict__ rel, int64_t* __restrict__ 
   if (idx) idx[base + t] = -1;
 }
 
+// Transposed graph of an edge prefix from the transposed graph of the whole edge array.
+// A stable sort by source keeps every source's edges in position order, so the entries of
+// the prefix [0, limit) are, per source, the leading ones: the prefix graph is the stable
+// compaction of the entries with perm < limit -- one scan and one scatter instead of a sort.
+struct EntryInPrefix {
+  const int64_t* perm;
+  int64_t n_entries, limit;
+  __device__ int64_t operator()(int64_t k) const { return (k < n_entries && perm[k] < limit) ? 1 : 0; }
+};
+
+__global__ void transpose_prefix_fill_kernel(const int64_t* __restrict__ ptr_t_all,
+                                             const int64_t* __restrict__ idx_t_all,
+                                             const int64_t* __restrict__ perm_all, int64_t n_entries,
+                                             int64_t limit, int64_t n_cols, const int64_t* __restrict__ pos,
+                                             int64_t* __restrict__ ptr_t, int64_t* __restrict__ idx_t,
+                                             int64_t* __restrict__ perm) {
+  const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (k < n_entries) {
+    const int64_t p = perm_all[k];
+    if (p < limit) {
+      const int64_t o = pos[k];
+      idx_t[o] = idx_t_all[k];
+      perm[o] = p;
+    }
+  }
+  if (k <= n_cols) ptr_t[k] = pos[ptr_t_all[k]];
+}
+
 int bits_for(int64_t n) {
   int b = 1;
   while (b < 63 && ((int64_t)1 << b) < n) ++b;
@@ -219,6 +248,48 @@ int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows
                      dim3(cxg::kBlock), 0, st, ptr, n_rows, sorted_src, perm, n_edges, n_cols, ptr_t,
                      idx_t);
   CXG_LAUNCH_CHECK("transpose_fill_kernel");
+  return CXG_OK;
+}
+
+size_t cxg_csr_transpose_prefix_workspace_bytes(int64_t n_edges_all) {
+  if (n_edges_all < 0) return 0;
+  size_t temp = 0;
+  cxg::EntryInPrefix f{nullptr, 0, 0};
+  auto in = rocprim::make_transform_iterator(rocprim::counting_iterator<int64_t>(0), f);
+  if (rocprim::exclusive_scan(nullptr, temp, in, (int64_t*)nullptr, (int64_t)0, (size_t)(n_edges_all + 1),
+                              rocprim::plus<int64_t>(), (hipStream_t)0) != hipSuccess)
+    return 0;
+  return cxg::align256((size_t)(n_edges_all + 1) * sizeof(int64_t)) + cxg::align256(temp) + 256;
+}
+
+int cxg_csr_transpose_prefix_i64(const int64_t* ptr_t_all, const int64_t* idx_t_all, const int64_t* perm_all,
+                                 int64_t n_edges_all, int64_t edge_limit, int64_t n_cols, int64_t* ptr_t,
+                                 int64_t* idx_t, int64_t* perm, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  CXG_REQUIRE(n_edges_all >= 0 && edge_limit >= 0 && n_cols >= 0, CXG_ERR_ARG, "negative size");
+  CXG_REQUIRE(edge_limit <= n_edges_all, CXG_ERR_ARG, "edge_limit %lld exceeds the %lld edges of the whole graph",
+              (long long)edge_limit, (long long)n_edges_all);
+  CXG_REQUIRE(ptr_t_all && ptr_t, CXG_ERR_ARG, "null ptr_t");
+  CXG_REQUIRE(n_edges_all == 0 || (idx_t_all && perm_all), CXG_ERR_ARG, "null idx_t_all/perm_all");
+  CXG_REQUIRE(edge_limit == 0 || (idx_t && perm), CXG_ERR_ARG, "null idx_t/perm");
+  const size_t need = cxg_csr_transpose_prefix_workspace_bytes(n_edges_all);
+  CXG_REQUIRE(workspace && workspace_bytes >= need, CXG_ERR_WORKSPACE,
+              "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  CXG_REQUIRE(((uintptr_t)workspace & 255) == 0, CXG_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  int64_t* pos = reinterpret_cast<int64_t*>(workspace);
+  const size_t off = cxg::align256((size_t)(n_edges_all + 1) * sizeof(int64_t));
+  void* temp = reinterpret_cast<char*>(workspace) + off;
+  size_t temp_bytes = workspace_bytes - off;
+  cxg::EntryInPrefix f{perm_all, n_edges_all, edge_limit};
+  auto in = rocprim::make_transform_iterator(rocprim::counting_iterator<int64_t>(0), f);
+  CXG_HIP_CHECK(rocprim::exclusive_scan(temp, temp_bytes, in, pos, (int64_t)0, (size_t)(n_edges_all + 1),
+                                        rocprim::plus<int64_t>(), st));
+  const int64_t work = (n_edges_all > n_cols + 1) ? n_edges_all : n_cols + 1;
+  hipLaunchKernelGGL(cxg::transpose_prefix_fill_kernel, dim3((unsigned)cxg::ceil_div(work, cxg::kBlock)),
+                     dim3(cxg::kBlock), 0, st, ptr_t_all, idx_t_all, perm_all, n_edges_all, edge_limit, n_cols,
+                     pos, ptr_t, idx_t, perm);
+  CXG_LAUNCH_CHECK("transpose_prefix_fill_kernel");
   return CXG_OK;
 }
 

@@ -37,15 +37,6 @@ namespace {
 #ifndef CXG_SPMM_U
 #define CXG_SPMM_U 1
 #endif
-#ifndef CXG_NT_IDX
-#define CXG_NT_IDX 1
-#endif
-#ifndef CXG_NT_OUT
-#define CXG_NT_OUT 1
-#endif
-#ifndef CXG_NT_GATHER
-#define CXG_NT_GATHER 0
-#endif
 #ifndef CXG_SPMM_U_V4
 #define CXG_SPMM_U_V4 8
 #endif
@@ -194,11 +185,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   }
 
   auto store_vec = [&](float* dst, vec_t v) {
-#if CXG_NT_OUT
     if (col_ok) stream_store(dst + col, v);
-#else
-    if (col_ok) *reinterpret_cast<vec_t*>(dst + col) = v;
-#endif
   };
   // What finish_row leaves in a row without edges.
   auto store_empty_row = [&](int64_t row) {
@@ -303,23 +290,14 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
     float my_w = 0.f;
     if (lane < cn) {
       const int64_t pos = e0 + c0 + lane;
-#if CXG_NT_IDX
       my_src = (int64_t)stream_load(a.idx + pos);
-#else
-      my_src = (int64_t)a.idx[pos];
-#endif
       if (EXT) {
         if (a.rel) my_src += (int64_t)a.rel[pos] * a.rel_stride;
         if (a.src_map) my_src = a.src_map[my_src];
         if (a.mask && !a.mask[a.mask_perm ? a.mask_perm[pos] : pos]) my_src = -1;
       }
-#if CXG_NT_IDX
       if (PERM) my_vrow = stream_load(a.perm + pos);
       if (WMODE == 1 && !PERM) my_w = stream_load(a.val + pos);
-#else
-      if (PERM) my_vrow = a.perm[pos];
-      if (WMODE == 1 && !PERM) my_w = a.val[pos];
-#endif
     }
     for (int b = 0; b < cn; b += U) {
       vec_t v[U];
@@ -542,11 +520,7 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
       if (row_take > m / L) vxor_add(acc, m);
   };
   auto store_vec = [&](float* dst, vec_t v) {
-#if CXG_NT_OUT
     if (writer) stream_store(dst + col, v);
-#else
-    if (writer) *reinterpret_cast<vec_t*>(dst + col) = v;
-#endif
   };
   auto finish_row = [&]() {
     reduce_groups();
@@ -576,23 +550,13 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     float my_w = 0.f;
     if (lane < cn) {
       const int64_t pos = e0 + c0 + lane;
-#if CXG_NT_IDX
       my_src = (int64_t)stream_load(a.idx + pos);
       if (PERM) my_vrow = stream_load(a.perm + pos);
       if (WMODE == 1 && !PERM) my_w = stream_load(a.val + pos);
-#else
-      my_src = (int64_t)a.idx[pos];
-      if (PERM) my_vrow = a.perm[pos];
-      if (WMODE == 1 && !PERM) my_w = a.val[pos];
-#endif
     }
     auto gather = [&](int e_idx, bool act, vec_t& v, float& w) {
       const int64_t src = shfl_i64(my_src, e_idx & 63);
-#if CXG_NT_GATHER
-      v = (act && col_ok) ? stream_load_vec(a.x + src * a.ldx + col, vec_t{}) : vzero<V>();
-#else
       v = (act && col_ok) ? *reinterpret_cast<const vec_t*>(a.x + src * a.ldx + col) : vzero<V>();
-#endif
       if (WMODE == 1) {
         if (PERM) {
           const int64_t vrow = shfl_i64(my_vrow, e_idx & 63);

@@ -332,6 +332,7 @@ class SageLayerOP(torch.autograd.Function):
     def forward(ctx, x, w_l, b_l, w_r, ptr, idx, num_node):
         n = int(num_node) if int(num_node) != 0 else ptr.shape[0] - 1
         x = x.contiguous()
+        _ops.note_layer(ptr, idx, n, x.shape[0])
         mm_first = w_l.shape[1] > w_l.shape[0]
         aggr = None
         if mm_first:

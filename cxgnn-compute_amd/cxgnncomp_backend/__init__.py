@@ -60,6 +60,8 @@ class _SageFunction(torch.autograd.Function):
             n = ptr.shape[0] - 1
         ctx.n, ctx.mean, ctx.n_src = n, mean, x.shape[0]
         ctx.x_shape = x.shape
+        if ctx.needs_input_grad[0]:
+            _ops.note_layer(ptr, idx, n, x.shape[0])
         x = x.contiguous()
         if edge_value is None:
             ctx.save_for_backward(ptr, idx)

@@ -52,6 +52,8 @@ SIGNATURES = {
     "cxg_head_sum_f32": (_I32, [_P, _P, _I64, _I32, _I32, _P]),
     "cxg_csr_transpose_workspace_bytes": (_SZ, [_I64, _I64]),
     "cxg_csr_transpose_i64": (_I32, [_P, _P, _I64, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
+    "cxg_csr_transpose_prefix_workspace_bytes": (_SZ, [_I64]),
+    "cxg_csr_transpose_prefix_i64": (_I32, [_P, _P, _P, _I64, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
     "cxg_csr_row_ids_i64": (_I32, [_P, _I64, _I64, _P, _P]),
     "cxg_edge_value_degree_f32": (_I32, [_P, _I64, _P, _P]),
     "cxg_pad_rel_i64": (_I32, [_P, _P, _P, _I32, _I32, _I64, _P]),

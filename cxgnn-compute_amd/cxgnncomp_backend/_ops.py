@@ -6,6 +6,7 @@ libcxgnn_hip.so.  Every function raises if a tensor is not a contiguous CUDA
 tensor of the expected dtype -- the kernels index raw memory.
 """
 import collections
+import weakref
 
 import torch
 
@@ -197,6 +198,7 @@ _GRAPH_CACHE_CAP = 8
 def clear_graph_cache():
     _GRAPH_CACHE.clear()
     _DEST_CACHE.clear()
+    _LAYER_HINT.clear()
 
 
 def set_graph_cache_capacity(n):
@@ -230,15 +232,74 @@ def csr_transpose(ptr, idx, n_rows, n_src):
     return ptr_t, idx_t, perm, n_edges
 
 
+def csr_transpose_prefix(whole, ptr, n_rows, n_src):
+    """Transposed graph of the first n_rows rows from the TransposedGraph ``whole`` of more rows of
+    the same (ptr, idx): a stable compaction of its entries (see cxg_csr_transpose_prefix_i64).
+    Returns (ptr_t, idx_t, perm, n_edges)."""
+    lib = _lib.load()
+    n_edges = int(ptr[n_rows].item())
+    dev = ptr.device
+    ptr_t = torch.empty(n_src + 1, dtype=torch.int64, device=dev)
+    idx_t = torch.empty(n_edges, dtype=torch.int64, device=dev)
+    perm = torch.empty(n_edges, dtype=torch.int64, device=dev)
+    ws = _workspace(lib.cxg_csr_transpose_prefix_workspace_bytes(whole.n_edges), dev)
+    with torch.cuda.device(dev):
+        st = lib.cxg_csr_transpose_prefix_i64(whole.ptr_t.data_ptr(), _lib.ptr(whole.idx_t), _lib.ptr(whole.perm),
+                                              whole.n_edges, n_edges, n_src, ptr_t.data_ptr(), _lib.ptr(idx_t),
+                                              _lib.ptr(perm), ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
+    _lib.check(st)
+    return ptr_t, idx_t, perm, n_edges
+
+
+# Largest (rows, sources) a forward pass has aggregated over each graph: the layers of a sampled
+# mini-batch work on nested row prefixes of one CSR, and the backward pass, which meets the
+# smallest layer first, can then sort the largest once and cut the others out of it.
+_LAYER_HINT = collections.OrderedDict()
+
+
+def _graph_id(ptr, idx):
+    return (ptr.data_ptr(), idx.data_ptr(), ptr.shape[0], idx.shape[0], ptr._version, idx._version,
+            ptr.device.index)
+
+
+def note_layer(ptr, idx, n_rows, n_src):
+    """Tell the transposed-graph cache that a layer aggregates rows [0, n_rows) of (ptr, idx)
+    over n_src sources (called by the forward passes whose backward needs the transposed graph)."""
+    gid = _graph_id(ptr, idx)
+    seen = _layer_hint(gid, ptr, idx)
+    if seen is None or n_rows > seen[0]:
+        # weak references: a hint must not outlive its tensors (their addresses get reused)
+        _LAYER_HINT[gid] = (n_rows, max(n_src, seen[1] if seen else 0), weakref.ref(ptr), weakref.ref(idx))
+        while len(_LAYER_HINT) > 64:
+            _LAYER_HINT.popitem(last=False)
+
+
+def _layer_hint(gid, ptr, idx):
+    hint = _LAYER_HINT.get(gid)
+    if hint is None:
+        return None
+    if hint[2]() is not ptr or hint[3]() is not idx:
+        del _LAYER_HINT[gid]
+        return None
+    return hint
+
+
 def transposed(ptr, idx, n_rows, n_src):
     """Cached TransposedGraph of (ptr[:n_rows+1], idx) with n_src source nodes."""
-    key = (ptr.data_ptr(), idx.data_ptr(), ptr.shape[0], idx.shape[0], n_rows, n_src,
-           ptr._version, idx._version, ptr.device.index)
+    gid = _graph_id(ptr, idx)
+    key = gid[:4] + (n_rows, n_src) + gid[4:]
     g = _GRAPH_CACHE.get(key)
     if g is not None:
         _GRAPH_CACHE.move_to_end(key)
         return g
-    ptr_t, idx_t, perm, n_edges = csr_transpose(ptr, idx, n_rows, n_src)
+    whole = None
+    hint = _layer_hint(gid, ptr, idx)
+    if ptr.is_cuda and hint is not None and hint[0] > n_rows and hint[1] >= n_src and _GRAPH_CACHE_CAP > 1:
+        whole = transposed(ptr, idx, hint[0], hint[1])
+    if whole is not None:
+        ptr_t, idx_t, perm, n_edges = csr_transpose_prefix(whole, ptr, n_rows, n_src)
+    else:
+        ptr_t, idx_t, perm, n_edges = csr_transpose(ptr, idx, n_rows, n_src)
     g = TransposedGraph(ptr_t, idx_t, perm, n_edges, n_src, n_rows, (ptr, idx))
     if _GRAPH_CACHE_CAP > 0:
         _GRAPH_CACHE[key] = g

@@ -432,6 +432,23 @@ int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows
                           int64_t* idx_t, int64_t* perm, void* workspace,
                           size_t workspace_bytes, void* stream);
 
+/*
+ * Transposed CSR of the edge prefix [0, edge_limit) of a graph whose whole transposition
+ * (ptr_t_all, idx_t_all, perm_all over n_edges_all edges, from cxg_csr_transpose_i64) is at
+ * hand: the result equals cxg_csr_transpose_i64 of the first rows of that graph, the rows
+ * that own exactly those edges, bit for bit (one scan and one scatter instead of a sort).
+ * The layers of a sampled mini-batch aggregate over nested prefixes of one CSR
+ * (cxgnncomp/model.py:55-71); their backward passes need the transposed graph of every
+ * prefix.  n_cols: sources of the prefix graph (all its edges must have a source below
+ * n_cols, and ptr_t_all must hold at least n_cols + 1 entries); ptr_t gets n_cols + 1
+ * entries, idx_t and perm edge_limit entries.
+ */
+size_t cxg_csr_transpose_prefix_workspace_bytes(int64_t n_edges_all);
+int cxg_csr_transpose_prefix_i64(const int64_t* ptr_t_all, const int64_t* idx_t_all,
+                                 const int64_t* perm_all, int64_t n_edges_all, int64_t edge_limit,
+                                 int64_t n_cols, int64_t* ptr_t, int64_t* idx_t, int64_t* perm,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
 /* rows[k] = row that owns edge position ptr[0] + k, k in [0, n_edges): the
  * device form of `repeat_interleave(arange(n), deg)` used by
  * SpMMValOP.backward (cxgnncomp/graph_kernel.py:31-34). */

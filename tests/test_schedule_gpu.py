@@ -215,3 +215,41 @@ def test_csr_transpose_far_more_columns_than_edges():
     assert np.array_equal(_np(ptr_t), want_ptr)
     assert np.array_equal(_np(idx_t), want_idx)
     assert np.array_equal(_np(perm), want_perm)
+
+
+def test_transposed_graphs_of_nested_layers_are_cut_from_the_largest(monkeypatch):
+    """The layers of a sampled batch are row prefixes of one CSR.  Once a forward pass has
+    announced them, the transposed graph of a smaller layer is compacted out of the largest
+    layer's instead of sorted again: it must equal the direct transposition bit for bit
+    (and both the oracle's)."""
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    ptr, idx, nn, ne = S.sampled_batch(num_seeds=300, fanouts=(7, 5, 3), id_space=200000, seed=9)
+    p, i = ptr.cuda(), idx.cuda()
+    _ops.clear_graph_cache()
+    for k in (2, 1, 0):                                  # forward order: largest layer first
+        _ops.note_layer(p, i, nn[k], nn[k + 1])
+    sorts = []
+    direct = _ops.csr_transpose
+    monkeypatch.setattr(_ops, "csr_transpose", lambda *a: (sorts.append(a[2]), direct(*a))[1])
+    graphs = {}
+    for k in (0, 1, 2):                                  # backward order: smallest layer first
+        announce("transposed prefix layer %d: rows=%d sources=%d" % (k, nn[k], nn[k + 1]))
+        graphs[k] = _ops.transposed(p, i, nn[k], nn[k + 1])
+    assert sorts == [nn[2]]                              # one sort, of the largest layer; the others were cut
+    monkeypatch.undo()
+    for k in (0, 1, 2):
+        g = graphs[k]
+        pt, it, pm, n_e = _ops.csr_transpose(p, i, nn[k], nn[k + 1])
+        assert g.n_edges == n_e == ne[k]
+        assert torch.equal(g.ptr_t, pt) and torch.equal(g.idx_t, it) and torch.equal(g.perm, pm)
+        want = oracle.csr_transpose(ptr.numpy(), idx.numpy(), nn[k], nn[k + 1])
+        assert np.array_equal(_np(g.ptr_t), want[0]) and np.array_equal(_np(g.idx_t), want[1])
+        assert np.array_equal(_np(g.perm), want[2])
+    # direct use of the entry point: an empty prefix and the whole graph as its own prefix
+    whole = _ops.transposed(p, i, nn[2], nn[3])
+    pt, it, pm, n_e = _ops.csr_transpose_prefix(whole, p, nn[2], nn[3])
+    assert torch.equal(pt, whole.ptr_t) and torch.equal(it, whole.idx_t) and torch.equal(pm, whole.perm)
+    pt, it, pm, n_e = _ops.csr_transpose_prefix(whole, p, 0, 5)
+    assert n_e == 0 and it.numel() == 0 and not pt.any()
+    _ops.clear_graph_cache()
