@@ -73,5 +73,39 @@ def build(force=False, jobs=None, verbose=True):
     return LIB
 
 
+EXT_SRC = os.path.join(HERE, "csrc_ext", "backend_ext.cpp")
+EXT_OUT = os.path.join(HERE, "cxgnncomp_backend", "_C.so")
+
+
+def build_ext(force=False, verbose=True):
+    """Compile cxgnncomp_backend/_C.so: the pybind11 / torch C++ host layer (csrc_ext/backend_ext.cpp)
+    over libcxgnn_hip.so.  Host code only, built with g++ against the installed torch."""
+    import sysconfig
+    import torch
+    deps = [EXT_SRC, os.path.join(HERE, "..", "include", "cxgnn_hip.h")]
+    if not force and os.path.exists(EXT_OUT) and os.path.getmtime(EXT_OUT) >= max(os.path.getmtime(d) for d in deps):
+        return EXT_OUT
+    tdir = os.path.dirname(torch.__file__)
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
+           "-I/opt/rocm/include", "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(HERE, "..", "include"),
+           EXT_SRC, "-o", EXT_OUT,
+           "-L" + os.path.join(tdir, "lib"), "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+           "-L" + os.path.dirname(LIB), "-lcxgnn_hip",
+           "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath," + os.path.join(tdir, "lib")]
+    if verbose:
+        print("[build] csrc_ext/backend_ext.cpp", flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("compiling the host extension failed:\n" + r.stdout + r.stderr)
+    if r.stderr.strip() and verbose:
+        print(r.stderr)
+    return EXT_OUT
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
+    build_ext(force="--force" in sys.argv)

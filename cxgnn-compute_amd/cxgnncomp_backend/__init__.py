@@ -11,8 +11,6 @@ Same function names, argument order and meaning.  Differences, all deliberate:
   * the autograd contexts keep the ptr/idx tensors alive instead of raw
     pointers (src/cpp/src/aggr.cu:116-117).
 """
-import enum
-
 import torch
 
 from . import _lib, _ops
@@ -24,227 +22,45 @@ def _lib_version():
 
 
 # --------------------------------------------------------------------------- #
-# sum / mean aggregation  (binding.cpp:15-19, 37-41)
+# Aggregation, SDDMM and edge-attention families: the compiled host layer
+# (csrc_ext/backend_ext.cpp), under the reference's names and argument order.
+#   run_spmm_configurable / _bwd / _int32     src/cpp/src/spmm_host.cu:6-156   (binding.cpp:37-41)
+#   sage_sum_forward / sage_mean_forward / sage_*_forward_edge_value
+#                                             src/cpp/src/aggr.cu:107-303,377-393 -- autograd in C++
+#   spmm_multihead / _bwd / run_spmm_multihead_configurable, SPMM_MULTIHEAD_SCHEDULE
+#                                             src/cpp/src/spmm_host.cu:158-256 (binding.cpp:57-74)
+#   run_sddmm / run_sddmm_vertex_centric      src/cpp/src/sddmm_host.cu:4-59   (binding.cpp:76-79)
+#   edge_attention(ptr, idx, att_dst, att_src, num_edge, relu_l) -- dst before src --,
+#   edge_value_degree, spmv                   src/cpp/src/edge_softmax.cu:97-244 -- autograd in C++
+# The nine launch integers of the *_configurable functions are accepted and ignored.
 # --------------------------------------------------------------------------- #
-def run_spmm_configurable(ptr, idx, vin, num_node, *launch_ints):
-    """out[r] = sum_e vin[idx[e]], r < num_node (src/cpp/src/spmm_host.cu:6-55)."""
-    if vin.dim() != 2:
-        raise ValueError("vin must be 2D")
-    return _ops.spmm(ptr, idx, vin, as_int(num_node))
+_C = _lib.native()
+
+run_spmm_configurable = _C.run_spmm_configurable
+run_spmm_configurable_int32 = _C.run_spmm_configurable_int32
+run_spmm_configurable_bwd = _C.run_spmm_configurable_bwd
+sage_sum_forward = _C.sage_sum_forward
+sage_mean_forward = _C.sage_mean_forward
+sage_sum_forward_edge_value = _C.sage_sum_forward_edge_value
+sage_mean_forward_edge_value = _C.sage_mean_forward_edge_value      # raises, as the reference aborts (aggr.cu:158,163)
+
+SPMM_MULTIHEAD_SCHEDULE = _C.SPMM_MULTIHEAD_SCHEDULE
+Naive, PreReduce, Optimal = _C.Naive, _C.PreReduce, _C.Optimal
+spmm_multihead = _C.spmm_multihead
+spmm_multihead_bwd = _C.spmm_multihead_bwd
+run_spmm_multihead_configurable = _C.run_spmm_multihead_configurable
+
+run_sddmm = _C.run_sddmm
+run_sddmm_vertex_centric = _C.run_sddmm_vertex_centric
+
+edge_attention = _C.edge_attention
+edge_value_degree = _C.edge_value_degree
+spmv = _C.spmv
 
 
-def run_spmm_configurable_int32(ptr, idx, vin, num_node, *launch_ints):
-    """int32 ptr/idx variant (src/cpp/src/spmm_host.cu:99-156)."""
-    if vin.dim() != 2:
-        raise ValueError("vin must be 2D")
-    return _ops.spmm(ptr, idx, vin, as_int(num_node))
-
-
-def run_spmm_configurable_bwd(ptr, idx, vin, grad_vout, num_node, *launch_ints):
-    """grad_vin[s] = sum_{e: idx[e]==s} grad_vout[row(e)], shaped like vin
-    (src/cpp/src/spmm_host.cu:57-97)."""
-    if grad_vout.dim() != 2:
-        raise ValueError("grad_vout must be 2D")
-    n = as_int(num_node)
-    g = _ops.transposed(ptr, idx, n, vin.shape[0])
-    return _ops.spmm(g.ptr_t, g.idx_t, grad_vout.contiguous(), vin.shape[0])
-
-
-class _SageFunction(torch.autograd.Function):
-    """SAGEFunction / SAGEEdgeValueFunction (src/cpp/src/aggr.cu:107-303)."""
-
-    @staticmethod
-    def forward(ctx, x, ptr, idx, edge_value, num_node, mean):
-        n = as_int(num_node)
-        if n == 0:
-            n = ptr.shape[0] - 1
-        ctx.n, ctx.mean, ctx.n_src = n, mean, x.shape[0]
-        ctx.x_shape = x.shape
-        if ctx.needs_input_grad[0]:
-            _ops.note_layer(ptr, idx, n, x.shape[0])
-        x = x.contiguous()
-        if edge_value is None:
-            ctx.save_for_backward(ptr, idx)
-            return _ops.spmm(ptr, idx, x, n, mean=mean)
-        if mean:
-            # aggr.cu:158,163 aborts here with the same message
-            raise ValueError("DO NOT use mean with edge value")
-        edge_value = edge_value.contiguous()
-        x3 = x
-        if edge_value.dim() == 2 and x.dim() != 3:
-            raise ValueError("multi-head edge_value needs input [N, H, C]")
-        ctx.save_for_backward(ptr, idx, x, edge_value)
-        return _ops.spmm(ptr, idx, x3, n, val=edge_value)
-
-    @staticmethod
-    def backward(ctx, grad_out):
-        grad_out = grad_out.contiguous()
-        saved = ctx.saved_tensors
-        ptr, idx = saved[0], saved[1]
-        g = _ops.transposed(ptr, idx, ctx.n, ctx.n_src)
-        if len(saved) == 2:
-            if ctx.mean:
-                inv = _ops.inv_degree_transposed(g, ptr, ctx.n)
-                go = grad_out.reshape(ctx.n, -1)
-                gx = _ops.spmm(g.ptr_t, g.idx_t, go, ctx.n_src, val=inv)
-            else:
-                gx = _ops.spmm(g.ptr_t, g.idx_t, grad_out.reshape(ctx.n, -1), ctx.n_src)
-            return gx.reshape(ctx.x_shape), None, None, None, None, None
-        x, edge_value = saved[2], saved[3]
-        gx = _ops.spmm(g.ptr_t, g.idx_t, grad_out, ctx.n_src, val=edge_value, val_perm=g.perm)
-        gval = None
-        if ctx.needs_input_grad[3]:
-            gval = _ops.sddmm_csr(ptr, idx, x, grad_out, ctx.n, edge_value.shape)
-        return gx.reshape(ctx.x_shape), None, None, gval, None, None
-
-
-def sage_sum_forward(input, ptr, idx, num_node):
-    return _SageFunction.apply(input, ptr, idx, None, num_node, False)
-
-
-def sage_mean_forward(input, ptr, idx, num_node):
-    return _SageFunction.apply(input, ptr, idx, None, num_node, True)
-
-
-def sage_sum_forward_edge_value(input, ptr, idx, edge_value, num_node):
-    return _SageFunction.apply(input, ptr, idx, edge_value, num_node, False)
-
-
-def sage_mean_forward_edge_value(input, ptr, idx, edge_value, num_node):
-    return _SageFunction.apply(input, ptr, idx, edge_value, num_node, True)
-
-
-# --------------------------------------------------------------------------- #
-# multi-head weighted SpMM  (binding.cpp:57-74)
-# --------------------------------------------------------------------------- #
-class SPMM_MULTIHEAD_SCHEDULE(enum.IntEnum):
-    Naive = 0
-    PreReduce = 1
-    Optimal = 2
-
-
-Naive = SPMM_MULTIHEAD_SCHEDULE.Naive
-PreReduce = SPMM_MULTIHEAD_SCHEDULE.PreReduce
-Optimal = SPMM_MULTIHEAD_SCHEDULE.Optimal
-
-
-def edge_value_degree(ptr, num_dst, num_edge):
-    """val[e] = 1/deg(row(e)) (src/cpp/src/edge_softmax.cu:186-214)."""
-    return _ops.edge_value_degree(ptr, as_int(num_dst), as_int(num_edge))
-
-
-def spmm_multihead(ptr, idx, val, vin, num_node, schedule=Optimal, block_size=256):
-    """src/cpp/src/spmm_host.cu:158-196.  Naive: out[r,h,c]; PreReduce/Optimal:
-    out[r,c] summed over heads."""
-    if vin.dim() != 3:
-        raise ValueError("vin must be 3D, [num_node, num_head, feat_len]")
-    if val.dim() != 2:
-        raise ValueError("val must be 2D, [num_edge, num_head]")
-    if val.shape[1] != vin.shape[1]:
-        raise ValueError("num_head mismatch %d %d" % (vin.shape[1], val.shape[1]))
-    out = _ops.spmm(ptr, idx, vin, as_int(num_node), val=val)
-    if SPMM_MULTIHEAD_SCHEDULE(int(schedule)) == SPMM_MULTIHEAD_SCHEDULE.Naive:
-        return out
-    return _ops.head_sum(out)
-
-
-def run_spmm_multihead_configurable(ptr, idx, val, vin, num_node, *launch_ints):
-    """src/cpp/src/spmm_host.cu:216-256: head-pre-reduced output [num_node, feat]."""
-    return spmm_multihead(ptr, idx, val, vin, num_node, PreReduce)
-
-
-def spmm_multihead_bwd(ptr, idx, val, grad_output, grad_x, num_node, schedule=Optimal, block_size=256):
-    """grad_x[idx[e],h,:] += val[e,h] * grad_output[r,h,:] into the caller's grad_x
-    (src/cpp/src/spmm_host.cu:198-214)."""
-    n = as_int(num_node)
-    g = _ops.transposed(ptr, idx, n, grad_x.shape[0])
-    _ops.spmm(g.ptr_t, g.idx_t, grad_output.contiguous(), grad_x.shape[0], val=val, val_perm=g.perm,
-              out=grad_x, accumulate=True)
-
-
-# --------------------------------------------------------------------------- #
-# SDDMM  (binding.cpp:76-79)
-# --------------------------------------------------------------------------- #
-def run_sddmm(src, dst, src_feat, dst_feat, output, num_edge):
-    """output[e,h] = <src_feat[src[e],h,:], dst_feat[dst[e],(h,):]>
-    (src/cpp/src/sddmm_host.cu:4-14).  A 2-D dst_feat is shared by all heads as
-    in the reference kernel; a 3-D dst_feat is taken per head."""
-    _ops.sddmm_coo(src, dst, src_feat, dst_feat, output, as_int(num_edge))
-
-
-def run_sddmm_vertex_centric(ptr, idx, src_feat, dst_feat, num_node, *launch_ints):
-    """Same values in CSR edge order, new [E,H] tensor (src/cpp/src/sddmm_host.cu:16-59)."""
-    return _ops.sddmm_csr(ptr, idx, src_feat, dst_feat, as_int(num_node))
-
-
-# --------------------------------------------------------------------------- #
-# edge attention  (binding.cpp:22-25, 33)
-# --------------------------------------------------------------------------- #
-class _EdgeSoftmaxFunction(torch.autograd.Function):
-    """EdgeSoftMaxFunction (src/cpp/src/edge_softmax.cu:97-177)."""
-
-    @staticmethod
-    def forward(ctx, ptr, idx, att_dst, att_src, num_edge, relu_l):
-        att_dst = att_dst.contiguous()
-        att_src = att_src.contiguous()
-        out, mask = _ops.edge_softmax_fwd(ptr, idx, att_dst, att_src, as_int(num_edge), relu_l)
-        ctx.save_for_backward(ptr, idx, out, mask)
-        ctx.n_dst, ctx.n_src, ctx.slope = att_dst.shape[0], att_src.shape[0], float(relu_l)
-        ctx.mark_non_differentiable(mask)
-        return out
-
-    @staticmethod
-    def backward(ctx, grad_out):
-        ptr, idx, out, mask = ctx.saved_tensors
-        g_dst, t_edge = _ops.edge_softmax_bwd(ptr, out, mask, grad_out.contiguous(), ctx.n_dst, ctx.slope)
-        g = _ops.transposed(ptr, idx, ctx.n_dst, ctx.n_src)
-        g_src = _ops.narrow_gather_sum(g.ptr_t, g.perm, t_edge, ctx.n_src, rows32=_ops.rows32_transposed(g))
-        return None, None, g_dst, g_src, None, None
-
-
-def edge_attention(ptr, idx, att_dst, att_src, num_edge, relu_l):
-    """softmax_row(leaky_relu(att_dst[r] + att_src[idx[e]])) -> [num_edge, heads]
-    (src/cpp/src/edge_softmax.cu:179-184; note dst before src)."""
-    return _EdgeSoftmaxFunction.apply(ptr, idx, att_dst, att_src, num_edge, relu_l)
-
-
-def spmv(ptr, idx, input, num_dst):
-    """out[r] = sum_e input[idx[e]] (src/cpp/src/edge_softmax.cu:234-244)."""
-    return _ops.narrow_gather_sum(ptr, idx, input, as_int(num_dst))
-
-
-# --------------------------------------------------------------------------- #
-# gather (edge -> node scatter-add)  (binding.cpp:19)
-# --------------------------------------------------------------------------- #
-class _GatherFunction(torch.autograd.Function):
-    """GatherFunction (src/cpp/src/aggr.cu:395-448).  Upstream adds every edge row to its
-    node with atomics; here the edge positions are grouped by destination once per
-    destination array (one stable sort, cached) and every node sums its own rows --
-    several times faster than fp32 atomics at these widths, and reproducible."""
-
-    @staticmethod
-    def forward(ctx, input, dest, num_node):
-        n = as_int(num_node)
-        if n <= 0:
-            raise ValueError("num_node must be > 0")
-        ctx.save_for_backward(dest)
-        input = input.contiguous()
-        if input.dim() != 2 or input.shape[0] != dest.shape[0]:
-            raise ValueError("input must be [num_edge, F] with one row per entry of dest")
-        if dest.shape[0] == 0:
-            return torch.zeros((n, input.shape[1]), dtype=torch.float32, device=input.device)
-        g = _ops.dest_groups(dest, n)
-        return _ops.spmm(g.ptr, g.perm, input, n)
-
-    @staticmethod
-    def backward(ctx, grad_out):
-        (dest,) = ctx.saved_tensors
-        return _ops.gather_rows(grad_out.contiguous(), dest), None, None
-
-
-def gather(input, dest, num_node):
-    """out[dest[e]] += input[e], out [num_node, F] (src/cpp/src/aggr.cu:445-448)."""
-    return _GatherFunction.apply(input, dest, num_node)
+# gather(input[E, F], dest[E], num_node): out[dest[e]] += input[e] (src/cpp/src/aggr.cu:395-448,
+# binding.cpp:19); autograd in C++, destination groups cached per destination array
+gather = _C.gather
 
 from ._rel import (aggr_rel, selective_aggr, selective_aggr_bwd, target_aggr,  # noqa: E402,F401
                    target_aggr_backward)

@@ -108,6 +108,26 @@ def load():
     return lib
 
 
+_native_mod = None
+
+
+def native():
+    """The compiled host layer ``cxgnncomp_backend._C`` (csrc_ext/backend_ext.cpp, built by
+    ``build.py``): tensor checks, allocation, the transposed-graph cache and the autograd functions
+    of the aggregation family in C++.  Like the library itself it has no substitute."""
+    global _native_mod
+    if _native_mod is None:
+        load()                         # resolves libcxgnn_hip.so, which the extension links against
+        try:
+            from . import _C
+        except ImportError as exc:
+            raise RuntimeError("the compiled host layer cxgnncomp_backend/_C.so is missing or does not load (%s); "
+                               "build it with `python build.py` in %s"
+                               % (exc, os.path.dirname(os.path.dirname(LIB_PATH)))) from exc
+        _native_mod = _C
+    return _native_mod
+
+
 def check(status):
     if status != 0:
         msg = load().cxg_last_error().decode("utf-8", "replace")

@@ -5,12 +5,13 @@ torch is used for device memory and streams only; all arithmetic happens in
 libcxgnn_hip.so.  Every function raises if a tensor is not a contiguous CUDA
 tensor of the expected dtype -- the kernels index raw memory.
 """
-import collections
-import weakref
 
 import torch
 
 from . import _lib
+from ._lib import native as _native
+
+_C = _native()
 
 SPMM_MEAN = 1
 SPMM_ACCUMULATE = 2
@@ -56,75 +57,9 @@ def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, 
     x is [n_src, F] or [n_src, H, C]; val (optional) is [E] or [E, H].  Returns
     a new [n_rows, ...] tensor unless ``out`` is given.  ``bias`` (with val, without mean:
     one float per column of a row) is added to every output row as it is stored.
+    Checks, allocation and the call into the library happen in the compiled host layer.
     """
-    lib = _lib.load()
-    int32 = ptr.dtype == torch.int32
-    _check_graph(ptr, idx, n_rows, torch.int32 if int32 else torch.int64)
-    _req(x, "x", torch.float32, (2, 3))
-    if x.device != ptr.device:
-        raise ValueError("x and ptr are on different devices")
-    heads = 1
-    channels = x.shape[-1]
-    if val is not None:
-        _req(val, "val", torch.float32, (1, 2))
-        if val.dim() == 2:
-            heads = val.shape[1]
-            if x.dim() != 3 or x.shape[1] != heads:
-                raise ValueError("val has %d heads but x has shape %s" % (heads, tuple(x.shape)))
-        elif x.dim() == 3:
-            if x.shape[1] != 1:
-                raise ValueError("1-D val needs x of shape [N, F] or [N, 1, F]")
-        need = idx.shape[0] if val_perm is None else 0
-        if val.shape[0] < need:
-            raise ValueError("val has %d rows, idx has %d" % (val.shape[0], idx.shape[0]))
-        if val_perm is not None:
-            _req(val_perm, "val_perm", torch.int64, 1)
-            if val_perm.shape[0] < idx.shape[0]:
-                raise ValueError("val_perm shorter than idx")
-    elif x.dim() == 3:
-        channels = x.shape[1] * x.shape[2]
-    row = heads * channels if val is not None else channels
-    out_shape = (n_rows,) + tuple(x.shape[1:])
-    if out is None:
-        out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
-    else:
-        _req(out, "out", torch.float32)
-        if tuple(out.shape) != out_shape:
-            raise ValueError("out has shape %s, expected %s" % (tuple(out.shape), out_shape))
-    if n_rows == 0:
-        return out
-    if bias is not None and val is None:
-        raise ValueError("bias needs edge values")
-    n_cap = idx.shape[0]
-    ws_bytes = lib.cxg_spmm_workspace_bytes(n_cap, row)
-    ws = _workspace(ws_bytes, x.device)
-    flags = (SPMM_MEAN if mean else 0) | (SPMM_ACCUMULATE if accumulate else 0)
-    if n_rows == ptr.shape[0] - 1:
-        flags |= SPMM_HINT_EXACT_EDGES       # all rows of ptr: idx holds exactly their edges
-    stream = _lib.current_stream(x.device)
-    with torch.cuda.device(x.device):
-        if val is None:
-            fn = lib.cxg_spmm_sum_f32_i32 if int32 else lib.cxg_spmm_sum_f32
-            st = fn(ptr.data_ptr(), _lib.ptr(idx), _lib.ptr(x), row, out.data_ptr(), row, n_rows,
-                    n_cap, row, flags, ws.data_ptr(), ws.numel(), stream)
-        else:
-            if int32:
-                raise ValueError("weighted SpMM needs int64 ptr/idx")
-            if bias is not None:
-                _req(bias, "bias", torch.float32, 1)
-                if bias.shape[0] != row or mean:
-                    raise ValueError("bias needs %d floats and no mean" % row)
-                st = lib.cxg_spmm_weighted_bias_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(),
-                                                    _lib.ptr(val_perm), _lib.ptr(x), row, bias.data_ptr(),
-                                                    out.data_ptr(), row, n_rows, n_cap, heads, channels, flags,
-                                                    ws.data_ptr(), ws.numel(), stream)
-            else:
-                st = lib.cxg_spmm_weighted_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(),
-                                               _lib.ptr(val_perm), _lib.ptr(x), row, out.data_ptr(), row,
-                                               n_rows, n_cap, heads, channels, flags, ws.data_ptr(),
-                                               ws.numel(), stream)
-    _lib.check(st)
-    return out
+    return _C.spmm(ptr, idx, x, int(n_rows), mean, val, val_perm, out, accumulate, bias)
 
 
 def spmm_dot_supported(heads, channels):
@@ -177,185 +112,70 @@ def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out):
 # --------------------------------------------------------------------------- #
 # transposed-graph cache
 # --------------------------------------------------------------------------- #
-class TransposedGraph:
-    """CSR of the reversed graph: rows = source nodes, idx_t = destination ids,
-    perm = position of each transposed edge in the original idx array."""
+TransposedGraph = _C.TransposedGraph      # ptr_t, idx_t, perm, n_edges, n_src, n_dst (see csrc_ext/backend_ext.cpp)
 
-    __slots__ = ("ptr_t", "idx_t", "perm", "n_edges", "n_src", "n_dst", "_keep", "_inv_deg_t", "_rows32")
-
-    def __init__(self, ptr_t, idx_t, perm, n_edges, n_src, n_dst, keep):
-        self.ptr_t, self.idx_t, self.perm = ptr_t, idx_t, perm
-        self.n_edges, self.n_src, self.n_dst = n_edges, n_src, n_dst
-        self._keep = keep  # the tensors the key was made from stay alive while cached
-        self._inv_deg_t = None
-        self._rows32 = None
-
-
-_GRAPH_CACHE = collections.OrderedDict()
 _GRAPH_CACHE_CAP = 8
 
 
 def clear_graph_cache():
-    _GRAPH_CACHE.clear()
-    _DEST_CACHE.clear()
-    _LAYER_HINT.clear()
+    _C.clear_graph_cache()
 
 
 def set_graph_cache_capacity(n):
     global _GRAPH_CACHE_CAP
     _GRAPH_CACHE_CAP = max(0, int(n))
-    while len(_GRAPH_CACHE) > _GRAPH_CACHE_CAP:
-        _GRAPH_CACHE.popitem(last=False)
+    _C.set_graph_cache_capacity(_GRAPH_CACHE_CAP)
 
 
 def csr_transpose(ptr, idx, n_rows, n_src):
-    """Uncached transposition; returns (ptr_t, idx_t, perm, n_edges)."""
-    lib = _lib.load()
-    _check_graph(ptr, idx, n_rows)
-    n_edges = int(ptr[n_rows].item())
-    first = int(ptr[0].item())
-    if first != 0:
-        raise ValueError("ptr[0] must be 0")
-    if n_edges > idx.shape[0]:
-        raise ValueError("ptr[num_node]=%d exceeds idx length %d" % (n_edges, idx.shape[0]))
-    dev = ptr.device
-    ptr_t = torch.empty(n_src + 1, dtype=torch.int64, device=dev)
-    idx_t = torch.empty(n_edges, dtype=torch.int64, device=dev)
-    perm = torch.empty(n_edges, dtype=torch.int64, device=dev)
-    ws_bytes = lib.cxg_csr_transpose_workspace_bytes(n_edges, n_src)
-    ws = _workspace(ws_bytes, dev)
-    with torch.cuda.device(dev):
-        st = lib.cxg_csr_transpose_i64(ptr.data_ptr(), _lib.ptr(idx), n_rows, n_src, n_edges,
-                                       ptr_t.data_ptr(), _lib.ptr(idx_t), _lib.ptr(perm),
-                                       ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
-    _lib.check(st)
-    return ptr_t, idx_t, perm, n_edges
+    """Uncached transposition by a stable sort; returns (ptr_t, idx_t, perm, n_edges)."""
+    return _C.csr_transpose(ptr, idx, int(n_rows), int(n_src))
 
 
 def csr_transpose_prefix(whole, ptr, n_rows, n_src):
     """Transposed graph of the first n_rows rows from the TransposedGraph ``whole`` of more rows of
     the same (ptr, idx): a stable compaction of its entries (see cxg_csr_transpose_prefix_i64).
     Returns (ptr_t, idx_t, perm, n_edges)."""
-    lib = _lib.load()
-    n_edges = int(ptr[n_rows].item())
-    dev = ptr.device
-    ptr_t = torch.empty(n_src + 1, dtype=torch.int64, device=dev)
-    idx_t = torch.empty(n_edges, dtype=torch.int64, device=dev)
-    perm = torch.empty(n_edges, dtype=torch.int64, device=dev)
-    ws = _workspace(lib.cxg_csr_transpose_prefix_workspace_bytes(whole.n_edges), dev)
-    with torch.cuda.device(dev):
-        st = lib.cxg_csr_transpose_prefix_i64(whole.ptr_t.data_ptr(), _lib.ptr(whole.idx_t), _lib.ptr(whole.perm),
-                                              whole.n_edges, n_edges, n_src, ptr_t.data_ptr(), _lib.ptr(idx_t),
-                                              _lib.ptr(perm), ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
-    _lib.check(st)
-    return ptr_t, idx_t, perm, n_edges
-
-
-# Largest (rows, sources) a forward pass has aggregated over each graph: the layers of a sampled
-# mini-batch work on nested row prefixes of one CSR, and the backward pass, which meets the
-# smallest layer first, can then sort the largest once and cut the others out of it.
-_LAYER_HINT = collections.OrderedDict()
-
-
-def _graph_id(ptr, idx):
-    return (ptr.data_ptr(), idx.data_ptr(), ptr.shape[0], idx.shape[0], ptr._version, idx._version,
-            ptr.device.index)
+    return _C.csr_transpose_prefix(whole, ptr, int(n_rows), int(n_src))
 
 
 def note_layer(ptr, idx, n_rows, n_src):
     """Tell the transposed-graph cache that a layer aggregates rows [0, n_rows) of (ptr, idx)
-    over n_src sources (called by the forward passes whose backward needs the transposed graph)."""
-    gid = _graph_id(ptr, idx)
-    seen = _layer_hint(gid, ptr, idx)
-    if seen is None or n_rows > seen[0]:
-        # weak references: a hint must not outlive its tensors (their addresses get reused)
-        _LAYER_HINT[gid] = (n_rows, max(n_src, seen[1] if seen else 0), weakref.ref(ptr), weakref.ref(idx))
-        while len(_LAYER_HINT) > 64:
-            _LAYER_HINT.popitem(last=False)
-
-
-def _layer_hint(gid, ptr, idx):
-    hint = _LAYER_HINT.get(gid)
-    if hint is None:
-        return None
-    if hint[2]() is not ptr or hint[3]() is not idx:
-        del _LAYER_HINT[gid]
-        return None
-    return hint
+    over n_src sources (called by the forward passes whose backward needs the transposed graph):
+    the layers of a sampled mini-batch work on nested row prefixes of one CSR, and the backward
+    pass, which meets the smallest layer first, then sorts the largest once and cuts the others
+    out of it."""
+    _C.note_layer(ptr, idx, int(n_rows), int(n_src))
 
 
 def transposed(ptr, idx, n_rows, n_src):
-    """Cached TransposedGraph of (ptr[:n_rows+1], idx) with n_src source nodes."""
-    gid = _graph_id(ptr, idx)
-    key = gid[:4] + (n_rows, n_src) + gid[4:]
-    g = _GRAPH_CACHE.get(key)
-    if g is not None:
-        _GRAPH_CACHE.move_to_end(key)
-        return g
-    whole = None
-    hint = _layer_hint(gid, ptr, idx)
-    if ptr.is_cuda and hint is not None and hint[0] > n_rows and hint[1] >= n_src and _GRAPH_CACHE_CAP > 1:
-        whole = transposed(ptr, idx, hint[0], hint[1])
-    if whole is not None:
-        ptr_t, idx_t, perm, n_edges = csr_transpose_prefix(whole, ptr, n_rows, n_src)
-    else:
-        ptr_t, idx_t, perm, n_edges = csr_transpose(ptr, idx, n_rows, n_src)
-    g = TransposedGraph(ptr_t, idx_t, perm, n_edges, n_src, n_rows, (ptr, idx))
-    if _GRAPH_CACHE_CAP > 0:
-        _GRAPH_CACHE[key] = g
-        while len(_GRAPH_CACHE) > _GRAPH_CACHE_CAP:
-            _GRAPH_CACHE.popitem(last=False)
-    return g
+    """Cached TransposedGraph of (ptr[:n_rows+1], idx) with n_src source nodes (LRU of
+    ``set_graph_cache_capacity`` graphs, kept in the compiled host layer)."""
+    return _C.transposed(ptr, idx, int(n_rows), int(n_src))
 
 
 class DestGroups:
-    """Edge positions grouped by destination: ptr [n+1] and perm [E] (stable), kept with the
-    destination array they were built from."""
+    """Edge positions grouped by destination: ptr [n+1] and perm [E] (stable)."""
 
-    __slots__ = ("ptr", "perm", "_keep")
+    __slots__ = ("ptr", "perm")
 
-    def __init__(self, ptr, perm, keep):
-        self.ptr, self.perm, self._keep = ptr, perm, keep
-
-
-_DEST_CACHE = collections.OrderedDict()
+    def __init__(self, ptr, perm):
+        self.ptr, self.perm = ptr, perm
 
 
 def dest_groups(dest, n_rows):
-    """Cached DestGroups of an edge -> node destination array (one stable sort)."""
-    key = (dest.data_ptr(), dest.shape[0], dest._version, n_rows, dest.device.index)
-    g = _DEST_CACHE.get(key)
-    if g is not None:
-        _DEST_CACHE.move_to_end(key)
-        return g
-    ptr, _, perm = coo_to_csr(dest, dest, n_rows)
-    g = DestGroups(ptr, perm, dest)
-    if _GRAPH_CACHE_CAP > 0:
-        _DEST_CACHE[key] = g
-        while len(_DEST_CACHE) > _GRAPH_CACHE_CAP:
-            _DEST_CACHE.popitem(last=False)
-    return g
+    """DestGroups of an edge -> node destination array (one stable sort, cached in the compiled
+    host layer per destination array)."""
+    return DestGroups(*_C.dest_groups(dest, int(n_rows)))
 
 
 def edge_value_degree(ptr, n_rows, n_edges):
-    lib = _lib.load()
-    _req(ptr, "ptr", torch.int64, 1)
-    if n_rows + 1 > ptr.shape[0]:
-        raise ValueError("num_dst=%d does not fit ptr" % n_rows)
-    out = torch.zeros(n_edges, dtype=torch.float32, device=ptr.device)
-    with torch.cuda.device(ptr.device):
-        st = lib.cxg_edge_value_degree_f32(ptr.data_ptr(), n_rows, out.data_ptr(),
-                                           _lib.current_stream(ptr.device))
-    _lib.check(st)
-    return out
+    return _C.edge_value_degree_raw(ptr, int(n_rows), int(n_edges))
 
 
 def inv_degree_transposed(g, ptr, n_rows):
-    """1/deg(dst) per edge, in transposed edge order (cached on the graph)."""
-    if g._inv_deg_t is None:
-        inv = edge_value_degree(ptr, n_rows, g.n_edges)
-        g._inv_deg_t = inv[g.perm] if g.n_edges > 0 else inv
-    return g._inv_deg_t
+    """1/deg(dst) per edge, in transposed edge order (kept with the graph)."""
+    return _C.inv_degree_transposed(g, ptr, int(n_rows))
 
 
 def csr_row_ids(ptr, n_rows, n_edges):
@@ -372,113 +192,28 @@ def csr_row_ids(ptr, n_rows, n_edges):
 # --------------------------------------------------------------------------- #
 # SDDMM / edge softmax / narrow row sums
 # --------------------------------------------------------------------------- #
-def _feat3(t, name):
-    _req(t, name, torch.float32, (2, 3))
-    return t if t.dim() == 3 else t.unsqueeze(1)
-
-
 def sddmm_csr(ptr, idx, src_feat, dst_feat, n_rows, out_shape=None, out=None):
     """out[e,h] = <src_feat[idx[e],h,:], dst_feat[row(e),(h,):]> in CSR edge order.
 
     src_feat [Ns,H,C] or [Ns,C]; dst_feat [Nd,H,C], or [Nd,C] (shared by all
     heads when H > 1).  Result is [E,H] ([E] when out_shape says so)."""
-    lib = _lib.load()
-    _check_graph(ptr, idx, n_rows)
-    a = _feat3(src_feat, "src_feat")
-    heads, channels = a.shape[1], a.shape[2]
-    _req(dst_feat, "dst_feat", torch.float32, (2, 3))
-    if dst_feat.dim() == 3:
-        b_heads = 1
-        if dst_feat.shape[1] != heads or dst_feat.shape[2] != channels:
-            raise ValueError("dst_feat shape %s does not match src_feat %s"
-                             % (tuple(dst_feat.shape), tuple(src_feat.shape)))
-    else:
-        b_heads = 1 if heads == 1 else 0
-        if dst_feat.shape[1] != channels:
-            raise ValueError("dst_feat has %d channels, src_feat %d" % (dst_feat.shape[1], channels))
-    if dst_feat.shape[0] < n_rows:
-        raise ValueError("dst_feat has fewer rows than num_node")
-    n_cap = idx.shape[0]
-    if out is None:
-        out = torch.zeros((n_cap, heads), dtype=torch.float32, device=a.device)
-    else:
-        _req(out, "out", torch.float32)
-        if out.numel() < n_cap * heads:
-            raise ValueError("output too small")
-    with torch.cuda.device(a.device):
-        st = lib.cxg_sddmm_csr_f32(ptr.data_ptr(), _lib.ptr(idx), a.data_ptr(), dst_feat.data_ptr(),
-                                   out.data_ptr(), n_rows, n_cap, heads, channels, b_heads,
-                                   _lib.current_stream(a.device))
-    _lib.check(st)
-    if out_shape is not None:
-        return out.reshape(out_shape)
-    return out
+    res = _C.sddmm_csr(ptr, idx, src_feat, dst_feat, int(n_rows), out)
+    return res.reshape(out_shape) if out_shape is not None else res
 
 
 def sddmm_coo(src, dst, src_feat, dst_feat, out, n_edges):
-    lib = _lib.load()
-    _req(src, "src", torch.int64, 1)
-    _req(dst, "dst", torch.int64, 1)
-    if src.shape[0] < n_edges or dst.shape[0] < n_edges:
-        raise ValueError("src/dst shorter than num_edge")
-    a = _feat3(src_feat, "src_feat")
-    heads, channels = a.shape[1], a.shape[2]
-    _req(dst_feat, "dst_feat", torch.float32, (2, 3))
-    if dst_feat.dim() == 3:
-        b_heads = 1
-        if dst_feat.shape[1] != heads or dst_feat.shape[2] != channels:
-            raise ValueError("dst_feat shape does not match src_feat")
-    else:
-        b_heads = 1 if heads == 1 else 0
-        if dst_feat.shape[1] != channels:
-            raise ValueError("dst_feat has %d channels, src_feat %d" % (dst_feat.shape[1], channels))
-    _req(out, "output", torch.float32)
-    if out.numel() < n_edges * heads:
-        raise ValueError("output too small")
-    with torch.cuda.device(a.device):
-        st = lib.cxg_sddmm_coo_f32(src.data_ptr(), dst.data_ptr(), a.data_ptr(), dst_feat.data_ptr(),
-                                   out.data_ptr(), n_edges, heads, channels, b_heads,
-                                   _lib.current_stream(a.device))
-    _lib.check(st)
-    return out
+    return _C.sddmm_coo(src, dst, src_feat, dst_feat, out, int(n_edges))
 
 
 def edge_softmax_fwd(ptr, idx, att_dst, att_src, n_edges, slope):
-    lib = _lib.load()
-    _req(att_dst, "att_dst", torch.float32, 2)
-    _req(att_src, "att_src", torch.float32, 2)
-    n_dst, heads = att_dst.shape
-    if att_src.shape[1] != heads:
-        raise ValueError("att_src/att_dst head mismatch")
-    _check_graph(ptr, idx, n_dst)
-    if idx.shape[0] < n_edges:
-        raise ValueError("idx shorter than num_edge")
-    out = torch.empty((n_edges, heads), dtype=torch.float32, device=att_dst.device)
-    mask = torch.empty((n_edges, heads), dtype=torch.bool, device=att_dst.device)
-    with torch.cuda.device(att_dst.device):
-        st = lib.cxg_edge_softmax_fwd_f32(ptr.data_ptr(), _lib.ptr(idx), att_dst.data_ptr(),
-                                          att_src.data_ptr(), _lib.ptr(out), _lib.ptr(mask), n_dst,
-                                          heads, float(slope), _lib.current_stream(att_dst.device))
-    _lib.check(st)
-    return out, mask
+    """(out [n_edges, H], mask [n_edges, H] bool)."""
+    return _C.edge_softmax_fwd(ptr, idx, att_dst, att_src, int(n_edges), float(slope))
 
 
 def edge_softmax_bwd(ptr, out, mask, grad, n_dst, slope):
     """Returns (g_dst [n_dst,H], t_edge [E,H]); rows of t_edge at or past ptr[n_dst] are not
     written (the transposed gather that consumes t_edge never reads them)."""
-    lib = _lib.load()
-    _req(out, "out", torch.float32, 2)
-    _req(grad, "grad", torch.float32, 2)
-    _req(mask, "mask", torch.bool, 2)
-    heads = out.shape[1]
-    g_dst = torch.empty((n_dst, heads), dtype=torch.float32, device=out.device)
-    t_edge = torch.empty_like(out)
-    with torch.cuda.device(out.device):
-        st = lib.cxg_edge_softmax_bwd_f32(ptr.data_ptr(), _lib.ptr(out), _lib.ptr(mask), _lib.ptr(grad),
-                                          _lib.ptr(g_dst), _lib.ptr(t_edge), n_dst, heads, float(slope),
-                                          _lib.current_stream(out.device))
-    _lib.check(st)
-    return g_dst, t_edge
+    return _C.edge_softmax_bwd(ptr, out, mask, grad, int(n_dst), float(slope))
 
 
 def attention_logits(x, att_src, att_dst, n_dst):
@@ -635,50 +370,19 @@ def csr_row_ids32(ptr, n_rows, n_edges):
 
 def rows32_transposed(g):
     """Row (source) id of every edge of a TransposedGraph, built once and kept with it."""
-    if g._rows32 is None:
-        g._rows32 = csr_row_ids32(g.ptr_t, g.n_src, g.n_edges)
-    return g._rows32
+    return _C.rows32_transposed(g)
 
 
 def narrow_gather_sum(ptr, sel, inp, n_rows, rows32=None):
     """out[r,:] = sum_{k in row r} inp[sel[k],:] (sel None: inp[k,:]); inp [M] or [M,W].
     With ``rows32`` (int32 row id per edge of ptr[:n_rows+1], ptr[0] == 0) and W in
     {1, 2, 4, 8} the edge-parallel segmented kernel is used."""
-    lib = _lib.load()
-    _req(ptr, "ptr", torch.int64, 1)
-    if n_rows + 1 > ptr.shape[0]:
-        raise ValueError("num rows does not fit ptr")
-    if sel is not None:
-        _req(sel, "sel", torch.int64, 1)
-    _req(inp, "input", torch.float32, (1, 2))
-    width = 1 if inp.dim() == 1 else inp.shape[1]
-    shape = (n_rows,) if inp.dim() == 1 else (n_rows, width)
-    out = torch.empty(shape, dtype=torch.float32, device=inp.device)
-    with torch.cuda.device(inp.device):
-        if rows32 is not None and width in (1, 2, 4, 8):
-            _req(rows32, "rows32", torch.int32, 1)
-            n_edges = rows32.shape[0]
-            ws = _workspace(lib.cxg_segment_gather_sum_workspace_bytes(n_edges, width), inp.device)
-            st = lib.cxg_segment_gather_sum_f32(_lib.ptr(rows32), ptr.data_ptr(), _lib.ptr(sel), _lib.ptr(inp),
-                                                _lib.ptr(out), n_rows, n_edges, width, ws.data_ptr(), ws.numel(),
-                                                _lib.current_stream(inp.device))
-        else:
-            st = lib.cxg_narrow_gather_sum_f32(ptr.data_ptr(), _lib.ptr(sel), _lib.ptr(inp), _lib.ptr(out),
-                                               n_rows, width, _lib.current_stream(inp.device))
-    _lib.check(st)
-    return out
+    return _C.narrow_gather_sum(ptr, sel, inp, int(n_rows), rows32)
 
 
 def head_sum(x):
     """[N, H, C] -> [N, C], summed over heads."""
-    lib = _lib.load()
-    _req(x, "x", torch.float32, 3)
-    out = torch.empty((x.shape[0], x.shape[2]), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
-        st = lib.cxg_head_sum_f32(_lib.ptr(x), _lib.ptr(out), x.shape[0], x.shape[1], x.shape[2],
-                                  _lib.current_stream(x.device))
-    _lib.check(st)
-    return out
+    return _C.head_sum(x)
 
 
 def scatter_add_rows(inp, dest, n_nodes):
@@ -698,15 +402,7 @@ def scatter_add_rows(inp, dest, n_nodes):
 
 def gather_rows(inp, sel):
     """out[e] = inp[sel[e]]."""
-    lib = _lib.load()
-    _req(inp, "input", torch.float32, 2)
-    _req(sel, "sel", torch.int64, 1)
-    out = torch.empty((sel.shape[0], inp.shape[1]), dtype=torch.float32, device=inp.device)
-    with torch.cuda.device(inp.device):
-        st = lib.cxg_gather_rows_f32(_lib.ptr(inp), _lib.ptr(sel), _lib.ptr(out), sel.shape[0],
-                                     inp.shape[1], _lib.current_stream(inp.device))
-    _lib.check(st)
-    return out
+    return _C.gather_rows(inp, sel)
 
 
 # --------------------------------------------------------------------------- #

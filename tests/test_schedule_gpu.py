@@ -217,7 +217,7 @@ def test_csr_transpose_far_more_columns_than_edges():
     assert np.array_equal(_np(perm), want_perm)
 
 
-def test_transposed_graphs_of_nested_layers_are_cut_from_the_largest(monkeypatch):
+def test_transposed_graphs_of_nested_layers_are_cut_from_the_largest():
     """The layers of a sampled batch are row prefixes of one CSR.  Once a forward pass has
     announced them, the transposed graph of a smaller layer is compacted out of the largest
     layer's instead of sorted again: it must equal the direct transposition bit for bit
@@ -229,15 +229,15 @@ def test_transposed_graphs_of_nested_layers_are_cut_from_the_largest(monkeypatch
     _ops.clear_graph_cache()
     for k in (2, 1, 0):                                  # forward order: largest layer first
         _ops.note_layer(p, i, nn[k], nn[k + 1])
-    sorts = []
-    direct = _ops.csr_transpose
-    monkeypatch.setattr(_ops, "csr_transpose", lambda *a: (sorts.append(a[2]), direct(*a))[1])
+    before = _ops._C.graph_cache_stats()
     graphs = {}
     for k in (0, 1, 2):                                  # backward order: smallest layer first
         announce("transposed prefix layer %d: rows=%d sources=%d" % (k, nn[k], nn[k + 1]))
         graphs[k] = _ops.transposed(p, i, nn[k], nn[k + 1])
-    assert sorts == [nn[2]]                              # one sort, of the largest layer; the others were cut
-    monkeypatch.undo()
+    after = _ops._C.graph_cache_stats()
+    # one sort, of the largest layer; the two smaller graphs were cut out of it
+    assert after["sorts"] - before["sorts"] == 1 and after["cuts"] - before["cuts"] == 2
+    assert graphs[2].n_dst == nn[2] and graphs[0].n_src == nn[1]
     for k in (0, 1, 2):
         g = graphs[k]
         pt, it, pm, n_e = _ops.csr_transpose(p, i, nn[k], nn[k + 1])
