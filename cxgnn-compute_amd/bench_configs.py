@@ -15,6 +15,7 @@ host cores (the restatements of the reference's own PyTorch paths kept with the
 CPU oracle), on bounded samples of the same graphs.
 
 Usage: python bench_configs.py [--configs c1,c2,c3,c4,c5] [--iters 10] [--cold] [--cpu-baseline]
+       python bench_configs.py --configs c5 --c5-steps 20 [--c5-fresh]    (only the sampled-batch training step)
 """
 import argparse
 import json
@@ -33,6 +34,8 @@ MFMA_BF16 = 2500000.0
 
 COLD = False
 CPU_BASELINE = False
+C5_STEPS = 0
+C5_FRESH = False
 _flush = None
 _last_spread = None
 
@@ -474,10 +477,41 @@ def c5(iters):
     layers = [cxgnncomp.MySageConv(128, 256).cuda(), cxgnncomp.MySageConv(256, 256).cuda(),
               cxgnncomp.MySageConv(256, 47).cuda()]
     import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
+    if C5_STEPS > 0:
+        # only the training step, C5_STEPS times: for kernel traces that count launches per batch
+        # (trace N and 2N steps and take the difference) and for the host's share of a step
+        import time
+        xg = x.clone().requires_grad_(True)
+        gout = torch.randn(nn[0], 47, device="cuda")
+
+        def one_step():
+            if C5_FRESH:
+                _ops.clear_graph_cache()        # a new sampled batch: nothing of the graph is cached
+            xg.grad = None
+            h = xg
+            for li, layer in enumerate(layers):
+                h = layer(h, ptr, idx, nn[2 - li])
+                if li < 2:
+                    h = torch.relu(h)
+            h.backward(gout)
+        for _ in range(3):
+            one_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(C5_STEPS):
+            one_step()
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        print(json.dumps({"config": "c5", "op": "3-layer SAGE fwd+bwd, %d steps after 3 warm-up steps, %s"
+                          % (C5_STEPS, "graph cache cleared before every step" if C5_FRESH else "reversed graphs cached"),
+                          "host_enqueue_ms_per_step": round((t1 - t0) * 1e3 / C5_STEPS, 4),
+                          "wall_ms_per_step": round((t2 - t0) * 1e3 / C5_STEPS, 4)}), flush=True)
+        return
     for li, (rows, edges) in enumerate(zip(nn[2::-1], ne[::-1])):
         report("c5", "sage_mean_forward rows=%d edges=%d F=128" % (rows, edges),
                timeit(lambda: B.sage_mean_forward(x, ptr, idx, rows), iters), spmm_bytes(rows, edges, 128), edges * 128)
-    from cxgnncomp_backend import _ops
 
     def prepare_sorts():
         # the reversed graph of each layer by its own stable sort
@@ -524,9 +558,12 @@ def main():
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--cold", action="store_true", help="flush the caches before every timed call")
     ap.add_argument("--cpu-baseline", action="store_true", help="also time the host-side PyTorch restatements")
+    ap.add_argument("--c5-steps", type=int, default=0,
+                    help="c5 only: run just the 3-layer SAGE training step this many times (for launch counting)")
+    ap.add_argument("--c5-fresh", action="store_true", help="with --c5-steps: clear the graph cache before every step")
     args = ap.parse_args()
-    global COLD, CPU_BASELINE
-    COLD, CPU_BASELINE = args.cold, args.cpu_baseline
+    global COLD, CPU_BASELINE, C5_STEPS, C5_FRESH
+    COLD, CPU_BASELINE, C5_STEPS, C5_FRESH = args.cold, args.cpu_baseline, args.c5_steps, args.c5_fresh
     sys.path.insert(0, os.path.dirname(HERE))
     table = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5}
     for name in args.configs.split(","):
