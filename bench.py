@@ -53,7 +53,7 @@ MEASURED_TRAFFIC = {
     "c3_powerlaw_2.45M_nodes_61.9M_edges_F128": {
         "bytes": 25932737128,
         "sources": "5df788eeeb404394",
-        "profile": "profiles/spmm_group_kernel_c3_F128_hbm_traffic.md",
+        "profile": "profiles/spmm_group_kernel_c3_F128_fabric_traffic.md",
     },
 }
 
