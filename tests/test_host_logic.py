@@ -77,6 +77,73 @@ def test_backend_rejects_cpu_tensors_without_touching_the_gpu():
         B.edge_attention(ptr, idx, x, x, 2, 0.2)
 
 
+def test_compiled_host_layer_exports_the_reference_names():
+    """cxgnncomp_backend._C carries the exports the reference writes in C++ (binding.cpp:15-25,
+    37-41, 58-78); the module as a whole carries every name of binding.cpp:14-119."""
+    import cxgnncomp_backend as B
+    from cxgnncomp_backend import _C
+    compiled = ["sage_sum_forward", "sage_mean_forward", "sage_sum_forward_edge_value", "sage_mean_forward_edge_value",
+                "gather", "edge_attention", "edge_value_degree", "spmv", "run_spmm_configurable",
+                "run_spmm_configurable_bwd", "run_spmm_configurable_int32", "spmm_multihead", "spmm_multihead_bwd",
+                "run_spmm_multihead_configurable", "run_sddmm", "run_sddmm_vertex_centric"]
+    for name in compiled:
+        assert getattr(B, name) is getattr(_C, name), name
+    others = ["target_aggr", "target_aggr_backward", "rel_schedule", "selective_aggr", "selective_aggr_bwd",
+              "gen_edge_type_mag240m", "topo_sort", "aggr_rel", "aggr_rel_direct", "aggr_rgcn_direct_func",
+              "typed_linear", "typed_linear_s2e", "typed_linear_s2d", "pad_rel", "pad_rel_idx", "seastar_forward",
+              "seastar_backward", "GSpMM_u_e", "GSpMM_u", "REDUCEOP", "COMPUTEOP", "SPMM_MULTIHEAD_SCHEDULE"]
+    for name in others:
+        assert hasattr(B, name), name
+    # export_values(): the enum members are module attributes too, Optimal is the default schedule
+    assert int(B.Naive) == 0 and int(B.PreReduce) == 1 and int(B.Optimal) == 2
+    assert B.SPMM_MULTIHEAD_SCHEDULE.Optimal == B.Optimal
+    assert "schedule" in B.spmm_multihead.__doc__ and "block_size" in B.spmm_multihead.__doc__
+    assert _C.lib_version() == B._lib_version()
+    assert set(_C.graph_cache_stats()) == {"graphs", "sorts", "cuts"}
+
+
+def test_missing_host_layer_fails_loudly(monkeypatch):
+    import builtins
+    from cxgnncomp_backend import _lib
+    monkeypatch.setattr(_lib, "_native_mod", None)
+    real_import = builtins.__import__
+
+    def no_ext(name, globals=None, locals=None, fromlist=(), level=0):
+        if level == 1 and fromlist and "_C" in fromlist:
+            raise ImportError("simulated: no _C.so")
+        return real_import(name, globals, locals, fromlist, level)
+    monkeypatch.setattr(builtins, "__import__", no_ext)
+    with pytest.raises(RuntimeError, match="compiled host layer"):
+        _lib.native()
+
+
+def test_compiled_host_layer_checks_arguments_before_any_launch():
+    """Argument errors of the C++ layer are ValueErrors raised on the host (the reference exits the
+    process, src/cpp/include/common.h:16-26)."""
+    import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
+    ptr, idx, x = torch.tensor([0, 1, 2]), torch.tensor([1, 0]), torch.randn(2, 4)
+    with pytest.raises(ValueError, match="2D"):
+        B.run_spmm_configurable(ptr, idx, torch.randn(2, 2, 2), 2)
+    with pytest.raises(ValueError, match="3D"):
+        B.spmm_multihead(ptr, idx, torch.rand(2, 2), x, 2)
+    with pytest.raises(ValueError, match="num_head mismatch"):
+        B.spmm_multihead(ptr, idx, torch.rand(2, 3), torch.randn(2, 2, 4), 2)
+    with pytest.raises((ValueError, RuntimeError), match="DO NOT use mean with edge value"):
+        B.sage_mean_forward_edge_value(x, ptr, idx, torch.rand(2), 2)      # aggr.cu:158,163 aborts here
+    with pytest.raises((ValueError, RuntimeError), match="num_node must be > 0"):
+        B.gather(x, idx, 0)
+    with pytest.raises(ValueError, match="CUDA"):
+        B.run_sddmm(idx, idx, x, x, torch.zeros(2, 1), 2)
+    with pytest.raises(ValueError, match="CUDA"):
+        _ops.spmm(ptr, idx, x, 2, val=torch.rand(2))
+    with pytest.raises(ValueError, match="CUDA"):
+        _ops.transposed(ptr, idx, 2, 2)
+    # scalars may arrive as 0-d tensors (cxgnncomp/graph_conv.py:41-50): converted, then checked
+    with pytest.raises(ValueError, match="CUDA"):
+        B.run_spmm_configurable(ptr, idx, x, torch.tensor(2), 0, 0, 0, 0, 0, 0, 0, 0, 0)
+
+
 # ----------------------------------------------------------------------------- scheduling helpers
 def _random_ptr(rng, n, hi):
     deg = rng.integers(0, hi, n)
