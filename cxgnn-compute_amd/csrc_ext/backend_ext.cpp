@@ -7,6 +7,7 @@
 //   SAGEFunction / SAGEEdgeValueFunction   src/cpp/src/aggr.cu:107-303   -> SageFunction
 //   EdgeSoftMaxFunction                    src/cpp/src/edge_softmax.cu:97-177 -> EdgeSoftmaxFunction
 //   GatherFunction                         src/cpp/src/aggr.cu:395-448   -> GatherFunction
+//   AggrRelFunction                        src/cpp/src/rel_spmm.cu:37-136 -> AggrRelFunction
 // together with the plain entry points of the SpMM / SDDMM families (spmm_host.cu, sddmm_host.cu)
 // and the cache of transposed graphs that their backward passes gather over.  The relational,
 // typed-GEMM and scheduling entry points are bound from Python (cxgnncomp_backend/_typed.py,
@@ -690,6 +691,84 @@ struct GatherFunction : public torch::autograd::Function<GatherFunction> {
 };
 
 // ---------------------------------------------------------------------------------------------
+// aggr_rel: relational aggregation over pre-transformed features (AggrRelFunction,
+// src/cpp/src/rel_spmm.cu:37-136): out[r] = sum_e input[etype[e] * N + idx[e]]
+// ---------------------------------------------------------------------------------------------
+// The combined row index etype[e] * N + idx[e] of every edge is kept per (idx, etype): with it the
+// relational gather is the plain SpMM, and its transposed graph (cached like any other) gives the
+// backward pass without the reference's atomics.
+struct RelKeys {
+  Tensor keys, keep_idx, keep_etype;
+};
+using RelKeyId = std::tuple<void*, void*, int64_t, int64_t, int64_t, int64_t, int>;
+struct RelKeyCache {
+  std::mutex mu;
+  std::list<std::pair<RelKeyId, std::shared_ptr<RelKeys>>> lru;
+};
+RelKeyCache& rel_key_cache() {
+  static RelKeyCache* c = new RelKeyCache;   // never destroyed, like the graph cache
+  return *c;
+}
+
+Tensor rel_keys(const Tensor& idx, const Tensor& etype, int64_t n_edges, int64_t stride, int64_t num_rel) {
+  req(idx, "idx", at::kLong, {1});
+  if (!etype.defined() || !etype.is_cuda() || etype.dim() != 1 ||
+      (etype.scalar_type() != at::kInt && etype.scalar_type() != at::kLong))
+    bad("etype must be a 1-D int32 or int64 CUDA tensor");
+  if (idx.size(0) < n_edges || etype.size(0) < n_edges) bad("idx / etype shorter than the rows' edges");
+  RelKeyCache& c = rel_key_cache();
+  const RelKeyId id(idx.data_ptr(), etype.data_ptr(), (int64_t)idx._version(), (int64_t)etype._version(), n_edges, stride,
+                    (int)idx.device().index());
+  {
+    std::lock_guard<std::mutex> lock(c.mu);
+    for (auto it = c.lru.begin(); it != c.lru.end(); ++it)
+      if (it->first == id) {
+        c.lru.splice(c.lru.end(), c.lru, it);
+        return c.lru.back().second->keys;
+      }
+  }
+  const Tensor rel64 = etype.slice(0, 0, n_edges).to(at::kLong);
+  if (n_edges > 0) {
+    const Tensor lim = torch::stack({rel64.min(), rel64.max()}).cpu();
+    if (lim[0].item<int64_t>() < 0 || lim[1].item<int64_t>() >= num_rel)
+      bad(fmt("relation ids must lie in [0, %lld)", (long long)num_rel));
+  }
+  auto k = std::make_shared<RelKeys>();
+  k->keys = rel64 * stride + idx.slice(0, 0, n_edges);
+  k->keep_idx = idx;
+  k->keep_etype = etype;
+  std::lock_guard<std::mutex> lock(c.mu);
+  c.lru.emplace_back(id, k);
+  while (c.lru.size() > 4) c.lru.pop_front();
+  return k->keys;
+}
+
+struct AggrRelFunction : public torch::autograd::Function<AggrRelFunction> {
+  static Tensor forward(AutogradContext* ctx, Tensor input, Tensor ptr, Tensor idx, Tensor etype, int64_t num_node,
+                        int64_t num_rel) {
+    int64_t n = num_node;
+    if (n == 0) n = ptr.size(0) - 1;
+    if (num_rel <= 0 || input.size(0) % num_rel != 0)
+      bad(fmt("input rows (%lld) must be num_rel (%lld) x nodes", (long long)input.size(0), (long long)num_rel));
+    req(ptr, "ptr", at::kLong, {1});
+    if (n < 0 || n + 1 > ptr.size(0)) bad("num_node does not fit ptr");
+    const int64_t stride = input.size(0) / num_rel;
+    const int64_t n_edges = ptr[n].item<int64_t>();
+    const Tensor keys = rel_keys(idx, etype, n_edges, stride, num_rel);
+    ctx->save_for_backward({ptr, keys});
+    ctx->saved_data["n"] = n;
+    ctx->saved_data["rows"] = input.size(0);
+    return spmm_plain(ptr, keys, input.contiguous(), n);
+  }
+  static tensor_list backward(AutogradContext* ctx, tensor_list grads) {
+    const auto saved = ctx->get_saved_variables();
+    const int64_t n = ctx->saved_data["n"].toInt(), rows = ctx->saved_data["rows"].toInt();
+    GraphPtr g = transposed(saved[0], saved[1], n, rows);
+    return {spmm_plain(g->ptr_t, g->idx_t, grads[0].contiguous(), rows), Tensor(), Tensor(), Tensor(), Tensor(), Tensor()};
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
 // entry points under the reference's names
 // ---------------------------------------------------------------------------------------------
 Tensor run_spmm_configurable(const Tensor& ptr, const Tensor& idx, const Tensor& vin, const py::object& num_node,
@@ -765,13 +844,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
       std::lock_guard<std::mutex> lock(cache().mu);
       cache().clear();
     }
-    std::lock_guard<std::mutex> lock(dest_cache().mu);
-    dest_cache().lru.clear();
+    {
+      std::lock_guard<std::mutex> lock(dest_cache().mu);
+      dest_cache().lru.clear();
+    }
+    std::lock_guard<std::mutex> lock(rel_key_cache().mu);
+    rel_key_cache().lru.clear();
   });
   m.def("gather_rows", &gather_rows);
   m.def("dest_groups", [](const Tensor& dest, int64_t n_rows) {
     DestPtr g = dest_groups(dest, n_rows);
     return std::make_tuple(g->ptr, g->perm);
+  });
+  m.def("aggr_rel", [](const Tensor& input, const Tensor& ptr, const Tensor& idx, const Tensor& etype,
+                       const py::object& num_node, const py::object& num_rel) {
+    return AggrRelFunction::apply(input, ptr, idx, etype, as_int(num_node), as_int(num_rel));
   });
   m.def("gather", [](const Tensor& input, const Tensor& dest, const py::object& num_node) {
     return GatherFunction::apply(input, dest, as_int(num_node));

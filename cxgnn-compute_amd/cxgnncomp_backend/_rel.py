@@ -1,7 +1,6 @@
 """Masked / targeted / relational aggregation of the reference backend
 (binding.cpp:26-31, 45-47) on top of cxg_spmm_ext_f32 and
 cxg_spmm_scatter_atomic_f32."""
-import collections
 
 import torch
 
@@ -98,55 +97,7 @@ def target_aggr_backward(grad_in, ptr, idx, targets, grad_out, num_node):
     spmm_ext(g.ptr_t, g.idx_t, grad_in, grad_out.shape[0], grad_out, accumulate=True, src_map=targets)
 
 
-_KEY_CACHE = collections.OrderedDict()
-
-
-def _rel_keys(idx, etype, n_edges, stride, num_rel):
-    """Combined row index etype[e] * stride + idx[e] of every edge, kept per (idx, etype):
-    with it the relational gather is the plain SpMM, and its transposed graph (cached
-    like any other) gives the backward pass without atomics."""
-    key = (idx.data_ptr(), etype.data_ptr(), idx._version, etype._version, n_edges, stride, idx.device.index)
-    k = _KEY_CACHE.get(key)
-    if k is not None:
-        _KEY_CACHE.move_to_end(key)
-        return k[0]
-    rel64 = etype[:n_edges].to(torch.int64)
-    if n_edges and (int(rel64.min()) < 0 or int(rel64.max()) >= num_rel):
-        raise ValueError("relation ids must lie in [0, %d)" % num_rel)
-    k = rel64 * stride + idx[:n_edges]
-    _KEY_CACHE[key] = (k, idx, etype)
-    while len(_KEY_CACHE) > 4:
-        _KEY_CACHE.popitem(last=False)
-    return k
-
-
-class _AggrRelFunction(torch.autograd.Function):
-    """AggrRelFunction (src/cpp/src/rel_spmm.cu:37-136).  Upstream's backward scatters with
-    atomics; here it is the gather over the transposed graph of the combined index."""
-
-    @staticmethod
-    def forward(ctx, input, ptr, idx, etype, num_node, num_rel):
-        n = as_int(num_node)
-        if n == 0:
-            n = ptr.shape[0] - 1
-        num_rel = int(num_rel)
-        if input.shape[0] % num_rel != 0:
-            raise ValueError("input rows (%d) must be num_rel (%d) x nodes" % (input.shape[0], num_rel))
-        stride = input.shape[0] // num_rel
-        n_edges = int(ptr[n].item())
-        keys = _rel_keys(idx, etype, n_edges, stride, num_rel)
-        ctx.save_for_backward(ptr, keys)
-        ctx.n, ctx.rows = n, input.shape[0]
-        return _ops.spmm(ptr, keys, input.contiguous(), n)
-
-    @staticmethod
-    def backward(ctx, grad_out):
-        ptr, keys = ctx.saved_tensors
-        g = _ops.transposed(ptr, keys, ctx.n, ctx.rows)
-        return _ops.spmm(g.ptr_t, g.idx_t, grad_out.contiguous(), ctx.rows), None, None, None, None, None
-
-
-def aggr_rel(input, ptr, idx, etype, num_node, num_rel):
-    """out[r] = sum_e input[etype[e]*N + idx[e]], input [num_rel*N, F], etype int32
-    (src/cpp/src/rel_spmm.cu:66-70)."""
-    return _AggrRelFunction.apply(input, ptr, idx, etype, num_node, num_rel)
+# aggr_rel(input, ptr, idx, etype, num_node, num_rel): out[r] = sum_e input[etype[e]*N + idx[e]],
+# input [num_rel*N, F], etype int32 (AggrRelFunction, src/cpp/src/rel_spmm.cu:37-136, :66-70): autograd
+# in the compiled host layer, over the cached combined index and its transposed graph.
+aggr_rel = _lib.native().aggr_rel

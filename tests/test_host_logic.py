@@ -82,14 +82,14 @@ def test_compiled_host_layer_exports_the_reference_names():
     37-41, 58-78); the module as a whole carries every name of binding.cpp:14-119."""
     import cxgnncomp_backend as B
     from cxgnncomp_backend import _C
-    compiled = ["sage_sum_forward", "sage_mean_forward", "sage_sum_forward_edge_value", "sage_mean_forward_edge_value",
+    compiled = ["aggr_rel", "sage_sum_forward", "sage_mean_forward", "sage_sum_forward_edge_value", "sage_mean_forward_edge_value",
                 "gather", "edge_attention", "edge_value_degree", "spmv", "run_spmm_configurable",
                 "run_spmm_configurable_bwd", "run_spmm_configurable_int32", "spmm_multihead", "spmm_multihead_bwd",
                 "run_spmm_multihead_configurable", "run_sddmm", "run_sddmm_vertex_centric"]
     for name in compiled:
         assert getattr(B, name) is getattr(_C, name), name
     others = ["target_aggr", "target_aggr_backward", "rel_schedule", "selective_aggr", "selective_aggr_bwd",
-              "gen_edge_type_mag240m", "topo_sort", "aggr_rel", "aggr_rel_direct", "aggr_rgcn_direct_func",
+              "gen_edge_type_mag240m", "topo_sort", "aggr_rel_direct", "aggr_rgcn_direct_func",
               "typed_linear", "typed_linear_s2e", "typed_linear_s2d", "pad_rel", "pad_rel_idx", "seastar_forward",
               "seastar_backward", "GSpMM_u_e", "GSpMM_u", "REDUCEOP", "COMPUTEOP", "SPMM_MULTIHEAD_SCHEDULE"]
     for name in others:
