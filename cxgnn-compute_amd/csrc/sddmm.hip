@@ -360,8 +360,10 @@ __global__ __launch_bounds__(kBlock) void sddmm_multi_kernel(SddmmArgs a) {
     const int cn = (n - c0) < CXG_WAVE ? (n - c0) : CXG_WAVE;
     int64_t my_src = 0, my_dst = 0;
     if (lane < cn) {
-      my_src = COO ? a.src[e0 + c0 + lane] : a.idx[e0 + c0 + lane];
-      if (COO) my_dst = a.dst[e0 + c0 + lane];
+      // index streams and products are touched once: non-temporal, so that they do not push
+      // gathered rows out of the L2
+      my_src = stream_load((COO ? a.src : a.idx) + e0 + c0 + lane);
+      if (COO) my_dst = stream_load(a.dst + e0 + c0 + lane);
     }
     auto fetch = [&](int jj, bool act, vec_t& va, vec_t& vb) {
       const int64_t src = sd_shfl_i64(my_src, jj & 63);
@@ -405,9 +407,9 @@ __global__ __launch_bounds__(kBlock) void sddmm_multi_kernel(SddmmArgs a) {
     }
     __builtin_amdgcn_wave_barrier();                 // the tile is complete (one wave, in-order LDS)
     if (ldo == H) {
-      for (int i = lane; i < cn * H; i += CXG_WAVE) a.out[(e0 + c0) * H + i] = res[i];
+      for (int i = lane; i < cn * H; i += CXG_WAVE) stream_store(a.out + (e0 + c0) * H + i, res[i]);
     } else {
-      for (int i = lane; i < cn * H; i += CXG_WAVE) a.out[(e0 + c0 + i / H) * ldo + i % H] = res[i];
+      for (int i = lane; i < cn * H; i += CXG_WAVE) stream_store(a.out + (e0 + c0 + i / H) * ldo + i % H, res[i]);
     }
     __builtin_amdgcn_wave_barrier();                 // read before the next step overwrites it
   }
