@@ -383,6 +383,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const bool k_ok = 4 * c4 < K;
   const float* A = reinterpret_cast<const float*>(g.a);
   float4 areg0[NLD], areg1[NLD];             // rows of the next two tiles, in flight
+  unsigned live0 = 0, live1 = 0;             // bit i: row i of the set exists (its values are zeroed otherwise)
   // Row tables (source and destination row of every row of a tile; -1: no such row).
   // Given row maps (MAPPED) are fetched for ALL the block's tiles before the first tile,
   // beside the consumers' weight loads: the loads of a wave complete in order, so a map
@@ -400,22 +401,33 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   // to an address that does and zeroed when the tile is staged): with no branch around a
   // load the compiler counts the loads in flight exactly and waits only for the older of
   // the two register sets.
-  auto gload = [&](float4 (&areg)[NLD], int t) {
+  // Which rows exist is noted here, as a bit mask that travels with the register set: the
+  // staging code then runs from the loaded registers alone, with no table look-up (an LDS
+  // read and a wait per row) between the conversions.
+  auto gload = [&](float4 (&areg)[NLD], unsigned& live_mask, int t) {
     const int tc = t < n_tiles ? t : n_tiles - 1;
+    unsigned mask = 0;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int64_t sidx = s_src[tc % SLOTS][i * RPI + rsub];
+      int64_t sidx;
+      if constexpr (MAPPED) {
+        sidx = s_src[tc % SLOTS][i * RPI + rsub];
+      } else {
+        sidx = row0 + (int64_t)tc * kBM + i * RPI + rsub;
+        if (sidx >= row_end) sidx = -1;
+      }
+      mask |= (sidx >= 0 ? 1u : 0u) << i;
       areg[i] = *reinterpret_cast<const float4*>(A + (sidx >= 0 ? sidx : 0) * g.lda + (k_ok ? 4 * c4 : 0));
     }
+    live_mask = mask;
   };
   // split the rows held in areg and write the parts of tile t into its LDS half
-  auto stage = [&](const float4 (&areg)[NLD], int t) {
+  auto stage = [&](const float4 (&areg)[NLD], unsigned live_mask, int t) {
     uint16_t (*dst)[kBM][KP] = Ap[t & 1];
-    const int tc = t < n_tiles ? t : n_tiles - 1;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int row = i * RPI + rsub;
-      const bool live = k_ok && s_src[tc % SLOTS][row] >= 0;
+      const bool live = k_ok && ((live_mask >> i) & 1u) != 0;
       const float v[4] = {live ? areg[i].x : 0.f, live ? areg[i].y : 0.f, live ? areg[i].z : 0.f,
                           live ? areg[i].w : 0.f};
       v4bf part[NS];
@@ -565,10 +577,10 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       for (int t = 0; t < 4; ++t) maps_fill(t);
     }
     __syncthreads();                         // row tables visible
-    gload(areg0, 0);
-    gload(areg1, 1);
-    stage(areg0, 0);
-    gload(areg0, 2);
+    gload(areg0, live0, 0);
+    gload(areg1, live1, 1);
+    stage(areg0, live0, 0);
+    gload(areg0, live0, 2);
     // Two iterations per trip, so that each register set keeps a fixed role.  The loop is
     // left with `return`, never through a path that rejoins the loop head with the two
     // register sets in the other order: the compiler, which counts the loads in flight
@@ -578,13 +590,13 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       if (t >= n_tiles) return;
       __syncthreads();
       maps_fill(t + 4);
-      stage(areg1, t + 1);
-      gload(areg1, t + 3);
+      stage(areg1, live1, t + 1);
+      gload(areg1, live1, t + 3);
       if (t + 1 >= n_tiles) return;
       __syncthreads();
       maps_fill(t + 5);
-      stage(areg0, t + 2);
-      gload(areg0, t + 4);
+      stage(areg0, live0, t + 2);
+      gload(areg0, live0, t + 4);
     }
   }
 }

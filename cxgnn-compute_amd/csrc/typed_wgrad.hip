@@ -155,22 +155,27 @@ void typed_wgrad_split_kernel(WgradArgs g) {
     // Loads are issued unconditionally: rows and columns that do not exist are redirected
     // to an address that does and zeroed when the tile is staged (a select between a
     // loaded vector and a zero vector made the compiler route the load through scratch).
-    auto gload = [&](float4 (&r4)[4], int t) {
+    // (which rows exist is noted as a bit mask that travels with the register set, so that
+    // the staging code needs no table look-up between its conversions)
+    auto gload = [&](float4 (&r4)[4], unsigned& live_mask, int t) {
       const int tc = t < n_tiles ? t : n_tiles - 1;
+      unsigned mask = 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int64_t ridx = row_index(tc, mg * 4 + i);
+        mask |= (ridx >= 0 ? 1u : 0u) << i;
         r4[i] = *reinterpret_cast<const float4*>(base + (ridx >= 0 ? ridx : 0) * ld);
       }
+      live_mask = mask;
     };
     // registers (4 rows x 4 columns) -> LDS [column][4 consecutive rows], split into parts
-    auto stage_tile = [&](const float4 (&r4)[4], int t) {
+    auto stage_tile = [&](const float4 (&r4)[4], unsigned live_mask, int t) {
       if (t >= n_tiles) return;
       const tile_t dst = tile_buf(operand, t & 1);
       float v[4][4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const bool live = col_ok && row_index(t, mg * 4 + i) >= 0;
+        const bool live = col_ok && ((live_mask >> i) & 1u) != 0;
         v[i][0] = live ? r4[i].x : 0.f;
         v[i][1] = live ? r4[i].y : 0.f;
         v[i][2] = live ? r4[i].z : 0.f;
@@ -191,11 +196,12 @@ void typed_wgrad_split_kernel(WgradArgs g) {
       }
     };
     float4 r0[4], r1[4];                               // rows of two tiles in flight
+    unsigned live0 = 0, live1 = 0;
     __syncthreads();                                   // #1: the row maps are there
-    gload(r0, 0);
-    gload(r1, 1);
-    stage_tile(r0, 0);
-    gload(r0, 2);
+    gload(r0, live0, 0);
+    gload(r1, live1, 1);
+    stage_tile(r0, live0, 0);
+    gload(r0, live0, 2);
     __syncthreads();                                   // #2: tile 0 is staged
     // iteration t: stage tile t+1, barrier, load tile t+3.  Two iterations per trip, so that
     // both register sets keep their place in the order of the loads, and no path other than
@@ -203,13 +209,13 @@ void typed_wgrad_split_kernel(WgradArgs g) {
     // flight statically and would otherwise wait for all of them there).  (Rows of four
     // tiles in flight instead of two were measured: slower, 2.30 against 2.12 ms.)
     for (int t = 0;; t += 2) {
-      stage_tile(r1, t + 1);
+      stage_tile(r1, live1, t + 1);
       __syncthreads();
-      gload(r1, t + 3);
+      gload(r1, live1, t + 3);
       if (t + 1 >= n_tiles) return;
-      stage_tile(r0, t + 2);
+      stage_tile(r0, live0, t + 2);
       __syncthreads();
-      gload(r0, t + 4);
+      gload(r0, live0, t + 4);
       if (t + 2 >= n_tiles) return;
     }
   }
