@@ -351,6 +351,8 @@ def c4(iters):
            flops, MFMA_F32)
     report("c4", "rgcn fused gather-GEMM-scatter fp32 as 6 bf16 products", timeit(lambda: fused("split6"), iters),
            fused_bytes, flops)
+    report("c4", "rgcn fused gather-GEMM-scatter fp32 as 3 scaled fp16 products (default)",
+           timeit(lambda: fused("split_f16"), iters), fused_bytes, flops)
     # the same result without atomics: one GEMM row per edge written in CSR order, then
     # the sum over each destination's consecutive rows (the sparse strategy of the layer)
     tmp = torch.empty(E, K, device="cuda")
@@ -359,7 +361,7 @@ def c4(iters):
     def per_edge():
         _typed.typed_gemm(x, w, seg, E, src_idx=src, dst_idx=perm, out=tmp)
         B._ops.spmm(ptr, pos, tmp, N)
-    report("c4", "rgcn gather-GEMM into per-edge rows + segment sum (no atomics), 6 bf16 products",
+    report("c4", "rgcn gather-GEMM into per-edge rows + segment sum (no atomics), 3 scaled fp16 products",
            timeit(per_edge, iters), fused_bytes + 8 * E * K, flops)
     del tmp, pos
     x16 = x.to(torch.bfloat16)
@@ -375,6 +377,9 @@ def c4(iters):
     report("c4", "typed GEMM edge->edge fp32 (E x 128 x 128, sorted rows)",
            timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="fp32"), iters),
            E * 8 * K + 4 * R * K * K, flops, MFMA_F32)
+    report("c4", "typed GEMM edge->edge fp32 as 3 scaled fp16 products (default)",
+           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="split_f16"), iters),
+           E * 8 * K + 4 * R * K * K, flops)
     for prec, nprod in (("split6", 6), ("split3", 3)):
         report("c4", "typed GEMM edge->edge fp32 as %d bf16 products" % nprod,
                timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision=prec), iters),
@@ -404,7 +409,7 @@ def c4(iters):
     report("c4", "aggr_rel forward + backward (gather over the transposed combined index) F=128", timeit(aggr_rel_step, iters))
     del xr, xrg
     oe2 = torch.zeros(E, K, device="cuda")
-    report("c4", "typed_linear_s2e (out[e] += x[src[e]] W[type[e]]), 6 bf16 products",
+    report("c4", "typed_linear_s2e (out[e] += x[src[e]] W[type[e]]), 3 scaled fp16 products",
            timeit(lambda: B.typed_linear_s2e(x, w, oe2, idx, rel32), max(2, iters // 2)),
            E * (4 * K + 8 * K + 12) + 4 * R * K * K, flops)
     del oe2

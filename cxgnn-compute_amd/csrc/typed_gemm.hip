@@ -27,6 +27,8 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 constexpr int kBM = 64;
 constexpr int kThreads = 256;
@@ -321,6 +323,53 @@ __device__ __forceinline__ void split_bf16(float x, __bf16 (&p)[NS]) {
   }
 }
 
+// Scaled fp16 parts (F16): every A row and every W column is scaled by a power of two that
+// brings its largest magnitude into [2^14, 2^15) and split into TWO fp16 parts,
+// h0 = fp16(x s), h1 = fp16(x s - h0): 22 significant bits.  a*b is accumulated from
+// a0*b1, a1*b0, a0*b0 (the dropped a1*b1 is below 2^-22 |ab|) on v_mfma_f32_32x32x16_f16,
+// and the accumulator is multiplied by the two inverse scales when the tile is stored.
+// Three matrix instructions and two LDS parts per k-step instead of six and three, at
+// 2^-21 per product (fp32 itself rounds every product to 2^-24).  An element far below
+// its row's maximum loses low bits of h1 to the fp16 exponent range, which is an error
+// below 2^-29 of the row maximum -- invisible next to the rounding of the larger terms
+// of the same dot product.  bf16 has no such range limit but only 8 bits per part.
+//
+// scale 2^(14 - e) and its inverse for a maximum with biased exponent `eb` (e = eb - 127);
+// all-zero (or denormal) rows / columns get scale 0, rows with an infinity or NaN scale 1.
+__device__ __forceinline__ void pow2_scales(unsigned max_bits, float& scale, float& inv) {
+  const int eb = (int)(max_bits >> 23);
+  scale = 0.f;
+  inv = 0.f;
+  if (eb == 255) {
+    scale = 1.f;
+    inv = 1.f;
+  } else if (eb >= 15) {
+    scale = __uint_as_float((unsigned)(268 - eb) << 23);
+    inv = __uint_as_float((unsigned)(eb - 14) << 23);
+  }
+}
+
+// Largest value over the aligned group of LANES lanes (8, 16 or 32) that holds a row, in every
+// lane of the group: butterfly steps through data-parallel moves inside a 16-lane row (lane ^ 1,
+// lane ^ 2, mirror of the row's halves, mirror of the row) and one swizzle for lane ^ 16.
+template <int CTRL>
+__device__ __forceinline__ unsigned dpp_max_u32(unsigned m) {
+  const unsigned o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)m, CTRL, 0xf, 0xf, false);
+  return o > m ? o : m;
+}
+template <int LANES>
+__device__ __forceinline__ unsigned group_max_u32(unsigned m) {
+  m = dpp_max_u32<0xB1>(m);                  // quad_perm [1,0,3,2]
+  m = dpp_max_u32<0x4E>(m);                  // quad_perm [2,3,0,1]
+  m = dpp_max_u32<0x141>(m);                 // row_half_mirror
+  if (LANES >= 16) m = dpp_max_u32<0x140>(m);   // row_mirror
+  if (LANES >= 32) {
+    const unsigned o = (unsigned)__builtin_amdgcn_ds_swizzle((int)m, 0x401F);   // lane ^ 16
+    m = o > m ? o : m;
+  }
+  return m;
+}
+
 constexpr int kSplitThreads = 512;         // waves 0-3 consume, waves 4-7 produce
 constexpr int kMapSlots = 8;               // no row maps given: the row tables of tiles t-1 .. t+5 are live at once
 constexpr int kMappedTiles = 16;           // row maps given: a block keeps the maps of ALL its tiles in LDS, so it
@@ -328,9 +377,10 @@ constexpr int kMappedTiles = 16;           // row maps given: a block keeps the 
 constexpr int kCP = 40;                    // floats per staged output row: 32 + pad; rows r and
                                            // r + 4 (the two halves of a wave) land 32 banks apart
 
-template <int KS, int NS, bool MAPPED>
+template <int KS, int NS, bool MAPPED, bool F16>
 __global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void typed_gemm_split_kernel(GemmArgs g, int G) {
+  static_assert(!F16 || NS == 2, "the fp16 form has two parts");
   constexpr int KP = KS * 16 + 8;          // padded LDS row (bf16 elements)
   constexpr int LPR = KS * 4;              // lanes per A row, one float4 each
   constexpr int RPI = 256 / LPR;           // rows per load instruction (256 producer threads)
@@ -345,6 +395,9 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   int64_t (*s_dst)[kBM] = s_src + SLOTS;
   float (*Cw)[kCP] = reinterpret_cast<float (*)[kCP]>(reinterpret_cast<unsigned char*>(s_dst + SLOTS)) +
                      (size_t)(threadIdx.x >> 6 & 3) * kBM;
+  // F16: inverse row scales of the two staged tiles, [2][kBM] floats behind the four staging areas
+  float (*s_inv)[kBM] = reinterpret_cast<float (*)[kBM]>(
+      reinterpret_cast<unsigned char*>(s_dst + SLOTS) + (size_t)4 * kBM * kCP * sizeof(float));
   const int64_t span = (int64_t)kBM * G;
   int rel = -1;
   int64_t row0 = 0, row_end = 0;
@@ -424,22 +477,55 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   // split the rows held in areg and write the parts of tile t into its LDS half
   auto stage = [&](const float4 (&areg)[NLD], unsigned live_mask, int t) {
     uint16_t (*dst)[kBM][KP] = Ap[t & 1];
+    unsigned row_max[NLD];                   // F16: largest magnitude of each row (bit pattern)
+    if constexpr (F16) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const bool live = k_ok && ((live_mask >> i) & 1u) != 0;
+        unsigned m = 0;
+        const float v[4] = {areg[i].x, areg[i].y, areg[i].z, areg[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned b = live ? (__float_as_uint(v[j]) & 0x7fffffffu) : 0u;
+          m = b > m ? b : m;
+        }
+        row_max[i] = m;
+      }
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) row_max[i] = group_max_u32<LPR>(row_max[i]);
+    }
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int row = i * RPI + rsub;
       const bool live = k_ok && ((live_mask >> i) & 1u) != 0;
       const float v[4] = {live ? areg[i].x : 0.f, live ? areg[i].y : 0.f, live ? areg[i].z : 0.f,
                           live ? areg[i].w : 0.f};
-      v4bf part[NS];
+      if constexpr (F16) {
+        float scale, inv;
+        pow2_scales(row_max[i], scale, inv);
+        v4h part[2];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        __bf16 parts[NS];
-        split_bf16<NS>(v[j], parts);
+        for (int j = 0; j < 4; ++j) {
+          const float xs = v[j] * scale;
+          const _Float16 h0 = (_Float16)xs;
+          part[0][j] = h0;
+          part[1][j] = (_Float16)(xs - (float)h0);
+        }
 #pragma unroll
-        for (int q = 0; q < NS; ++q) part[q][j] = parts[q];
+        for (int q = 0; q < 2; ++q) *reinterpret_cast<v4h*>(&dst[q][row][4 * c4]) = part[q];
+        if (c4 == 0) s_inv[t & 1][row] = inv;
+      } else {
+        v4bf part[NS];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          __bf16 parts[NS];
+          split_bf16<NS>(v[j], parts);
+#pragma unroll
+          for (int q = 0; q < NS; ++q) part[q][j] = parts[q];
+        }
+#pragma unroll
+        for (int q = 0; q < NS; ++q) *reinterpret_cast<v4bf*>(&dst[q][row][4 * c4]) = part[q];
       }
-#pragma unroll
-      for (int q = 0; q < NS; ++q) *reinterpret_cast<v4bf*>(&dst[q][row][4 * c4]) = part[q];
     }
   };
 
@@ -454,20 +540,53 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   // (the two kinds of waves run separate loops with the same number of barriers, so the
   // registers of one role are not live in the other)
   if (consumer) {
-    v8bf bw[NS][KS];                         // this wave's 32 columns of W[rel], split
+    v8bf bw[NS][KS];                         // this wave's 32 columns of W[rel], split (F16: fp16 bit patterns)
+    float inv_w = 1.f;                       // F16: inverse scale of this lane's column
     {
       const float* W = reinterpret_cast<const float*>(g.w) + (int64_t)rel * K * N;
       const int col = n0 + wave * 32 + (lane & 31);
+      if constexpr (F16) {
+        float wv[KS][8];
+        unsigned m = 0;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
+        for (int s = 0; s < KS; ++s) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int k = s * 16 + (lane >> 5) * 8 + j;
-          const float w = (k < K && col < N) ? W[(int64_t)k * N + col] : 0.f;
-          __bf16 parts[NS];
-          split_bf16<NS>(w, parts);
+          for (int j = 0; j < 8; ++j) {
+            const int k = s * 16 + (lane >> 5) * 8 + j;
+            wv[s][j] = (k < K && col < N) ? W[(int64_t)k * N + col] : 0.f;
+            const unsigned b = __float_as_uint(wv[s][j]) & 0x7fffffffu;
+            m = b > m ? b : m;
+          }
+        }
+        // the other half of the column's k range sits in lane ^ 32
+        const unsigned o = (unsigned)__shfl_xor((int)m, 32, CXG_WAVE);
+        m = o > m ? o : m;
+        float scale;
+        pow2_scales(m, scale, inv_w);
 #pragma unroll
-          for (int q = 0; q < NS; ++q) bw[q][s][j] = parts[q];
+        for (int s = 0; s < KS; ++s) {
+          v8h h0, h1;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float xs = wv[s][j] * scale;
+            h0[j] = (_Float16)xs;
+            h1[j] = (_Float16)(xs - (float)h0[j]);
+          }
+          bw[0][s] = __builtin_bit_cast(v8bf, h0);
+          bw[1][s] = __builtin_bit_cast(v8bf, h1);
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int k = s * 16 + (lane >> 5) * 8 + j;
+            const float w = (k < K && col < N) ? W[(int64_t)k * N + col] : 0.f;
+            __bf16 parts[NS];
+            split_bf16<NS>(w, parts);
+#pragma unroll
+            for (int q = 0; q < NS; ++q) bw[q][s][j] = parts[q];
+          }
         }
       }
     }
@@ -536,8 +655,26 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
           for (int i = 0; i <= order; ++i)
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
-              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s & 1][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
+              if constexpr (F16)
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, ap[s & 1][mt][i]),
+                                                                 __builtin_bit_cast(v8h, bw[order - i][s]), acc[mt], 0, 0, 0);
+              else
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s & 1][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
             }
+      }
+      if constexpr (F16) {
+        // undo the scales: accumulator element i of tile half mt is row
+        // mt*32 + (i>>2)*8 + (lane>>5)*4 + (i&3), this lane's column
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float4 ri = *reinterpret_cast<const float4*>(&s_inv[t & 1][mt * 32 + q * 8 + (lane >> 5) * 4]);
+            acc[mt][q * 4 + 0] *= ri.x * inv_w;
+            acc[mt][q * 4 + 1] *= ri.y * inv_w;
+            acc[mt][q * 4 + 2] *= ri.z * inv_w;
+            acc[mt][q * 4 + 3] *= ri.w * inv_w;
+          }
       }
       if (drain) {
 #pragma unroll
@@ -722,7 +859,7 @@ hipError_t allow_lds(KernelT kernel, size_t bytes) {
 int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64_t M, int K, int N,
                int R, unsigned flags) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
-  CXG_REQUIRE((flags & ~15u) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE((flags & ~31u) == 0, CXG_ERR_ARG, "unknown flag");
   if (M == 0) return CXG_OK;
   CXG_REQUIRE(a && w && c && seg, CXG_ERR_ARG, "null pointer");
   return CXG_OK;
@@ -742,7 +879,7 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   cxg::GemmArgs g{a, lda, w, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
                   (int)(flags & 1u), (int)((flags >> 1) & 1u)};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3)) && K <= 128 && (K & 3) == 0 && (lda & 3) == 0 &&
+  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && K <= 128 && (K & 3) == 0 && (lda & 3) == 0 &&
       ((uintptr_t)a & 15) == 0) {
     // 64*G rows per block: up to 32 tiles (16 with row maps, which the block keeps in LDS)
     // while the launch keeps a few thousand blocks
@@ -754,22 +891,26 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
     const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
     CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
     const dim3 grid((unsigned)n_blocks);
-#define CXG_SPLIT_LAUNCH(KS, NSV, MAP)                                                         \
+#define CXG_SPLIT_LAUNCH(KS, NSV, MAP, HALF)                                                   \
   do {                                                                                         \
-    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_gemm_split_kernel<KS, NSV, MAP>, lds));            \
-    hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, NSV, MAP>), grid, dim3(cxg::kSplitThreads), lds, st, \
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_gemm_split_kernel<KS, NSV, MAP, HALF>, lds));      \
+    hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, NSV, MAP, HALF>), grid, dim3(cxg::kSplitThreads), lds, st, \
                        g, G);                                                                  \
   } while (0)
 #define CXG_SPLIT(KS)                                                                          \
   do {                                                                                         \
-    const int ns = (flags & CXG_GEMM_SPLIT_BF16X3) ? 2 : 3;                                    \
+    const bool half = (flags & CXG_GEMM_SPLIT_F16X3) != 0;                                     \
+    const int ns = (half || (flags & CXG_GEMM_SPLIT_BF16X3)) ? 2 : 3;                          \
     const size_t lds = (size_t)2 * ns * cxg::kBM * (KS * 16 + 8) * sizeof(uint16_t) +          \
                        (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) + \
-                       (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float);                        \
-    if (ns == 2 && mapped) CXG_SPLIT_LAUNCH(KS, 2, true);                                      \
-    else if (ns == 2) CXG_SPLIT_LAUNCH(KS, 2, false);                                          \
-    else if (mapped) CXG_SPLIT_LAUNCH(KS, 3, true);                                            \
-    else CXG_SPLIT_LAUNCH(KS, 3, false);                                                       \
+                       (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float) +                       \
+                       (size_t)2 * cxg::kBM * sizeof(float);                                   \
+    if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                                   \
+    else if (half) CXG_SPLIT_LAUNCH(KS, 2, false, true);                                       \
+    else if (ns == 2 && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, false);                          \
+    else if (ns == 2) CXG_SPLIT_LAUNCH(KS, 2, false, false);                                   \
+    else if (mapped) CXG_SPLIT_LAUNCH(KS, 3, true, false);                                     \
+    else CXG_SPLIT_LAUNCH(KS, 3, false, false);                                                \
   } while (0)
     if (K <= 32) CXG_SPLIT(2);
     else if (K <= 64) CXG_SPLIT(4);

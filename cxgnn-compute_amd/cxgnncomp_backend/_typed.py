@@ -13,14 +13,18 @@ GEMM_ACCUMULATE = 1
 GEMM_ATOMIC = 2
 GEMM_SPLIT_BF16X6 = 4
 GEMM_SPLIT_BF16X3 = 8
+GEMM_SPLIT_F16X3 = 16
 
-# How fp32 typed GEMMs multiply: "split6" (six bf16 partial products per fp32
-# product: fp32-accurate and HBM bound for K <= 128), "split3" (three partial
-# products, relative error below 2^-16 per product), "fp32" (v_mfma_f32_32x32x2_f32) or
-# "bf16" (operands rounded to bf16, one bf16 MFMA product, fp32 accumulation; weight
-# gradients then use "split3").
-GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split6")
-_PRECISION_FLAGS = {"fp32": 0, "split6": GEMM_SPLIT_BF16X6, "split3": GEMM_SPLIT_BF16X3}
+# How fp32 typed GEMMs multiply: "split_f16" (the default: rows of A and columns of W scaled by
+# powers of two and split into two fp16 parts, three fp16 MFMA products per fp32 product, 2^-21
+# per product -- fp32-grade -- and HBM bound for K <= 128), "split6" (six bf16 partial products,
+# 2^-24), "split3" (three bf16 partial products, relative error below 2^-16 per product), "fp32"
+# (v_mfma_f32_32x32x2_f32) or "bf16" (operands rounded to bf16, one bf16 MFMA product, fp32
+# accumulation; weight gradients then use "split3").  Weight gradients, whose reduction runs
+# over the rows, take "split6" for "split_f16".
+GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split_f16")
+_PRECISION_FLAGS = {"fp32": 0, "split6": GEMM_SPLIT_BF16X6, "split3": GEMM_SPLIT_BF16X3,
+                    "split_f16": GEMM_SPLIT_F16X3}
 
 
 def rel_segment(types, num_rel):
@@ -47,9 +51,10 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
                accumulate=False, atomic=False, bf16=False, precision=None):
     """out[dst(i)] (=|+=) a[src(i)] @ w[r] for rows i of segment r (see cxg_typed_gemm_f32).
 
-    a [*, K] fp32, w [R, K, N] fp32.  precision "split6" (the default, see
-    GEMM_PRECISION) forms every fp32 product from six bf16 partial products
-    (fp32-accurate), "split3" from three (relative error per product < 2^-16, the
+    a [*, K] fp32, w [R, K, N] fp32.  precision "split_f16" (the default, see
+    GEMM_PRECISION) forms every fp32 product from three fp16 partial products of
+    row- / column-scaled operands (2^-21 per product), "split6" from six bf16 partial
+    products (2^-24), "split3" from three (relative error per product < 2^-16, the
     reference's tl.dot is TF32); "fp32" forces v_mfma_f32_32x32x2_f32.  With bf16=True or
     precision "bf16" the operands are rounded to bf16 (W transposed to [R, N, K]) and multiplied
     on the bf16 matrix cores with fp32 accumulation."""

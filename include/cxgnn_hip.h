@@ -266,6 +266,7 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
 #define CXG_GEMM_ATOMIC 2u     /* add with fp32 atomics (several rows share a dst) */
 #define CXG_GEMM_SPLIT_BF16X6 4u /* fp32 products as 6 bf16 partial products (fp32-accurate) */
 #define CXG_GEMM_SPLIT_BF16X3 8u /* fp32 products as 3 bf16 partial products (2^-16 / product) */
+#define CXG_GEMM_SPLIT_F16X3 16u /* fp32 products as 3 fp16 partial products of row- / column-scaled operands (2^-21 / product) */
 
 /*
  * C[dst(i), :] = A[src(i), :] @ W[r] for the rows i in [seg_ptr[r], seg_ptr[r+1]),
@@ -279,7 +280,14 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
  * six (three) partial products whose magnitude is above 2^-24 (2^-16) of |ab|:
  * X6 is as accurate as an fp32 FMA chain, X3 is off by at most 2^-16 per product
  * (the reference's tl.dot runs in TF32, 2^-11); both are HBM bound instead of
- * matrix-core bound.  Other shapes ignore the two flags.  Replaces
+ * matrix-core bound.  With CXG_GEMM_SPLIT_F16X3 (same shape conditions) every row of
+ * A and every column of W is scaled by a power of two that brings its largest
+ * magnitude into [2^14, 2^15) and split into two fp16 parts (22 significant bits);
+ * a*b is accumulated on v_mfma_f32_32x32x16_f16 from three partial products and the
+ * scales are undone when the row is stored: 2^-21 per product, half the matrix
+ * instructions and two thirds of the LDS traffic of X6.  Rows or columns whose largest
+ * magnitude is below 2^-112 count as zero; a row holding an infinity or NaN comes out
+ * non-finite.  Other shapes ignore the three flags.  Replaces
  * typed_matmul
  * (cxgnncomp/codegen/triton_typed_matmul.py:752-860: src_idx only = its
  * "single index" kernel with dst = src, seq_output = dst NULL, both = double

@@ -1,9 +1,10 @@
 """Typed GEMM (MFMA), relation segmentation, pad_rel and the fused RGCN op
 through cxgnncomp_backend vs the oracle.
 
-Every fp32 test runs three times: with the fp32 MFMA kernel ("fp32") and with
-the default six-product bf16 split ("split6", fp32-accurate) at 1e-4 relative /
-1e-5 absolute at O(1) output scale, and with the three-product split ("split3":
+Every fp32 test runs four times: with the fp32 MFMA kernel ("fp32"), with the
+default three-product split of scaled fp16 parts ("split_f16", 2^-21 per product) and
+with the six-product bf16 split ("split6", 2^-24) at 1e-4 relative /
+1e-5 absolute at O(1) output scale, and with the three-product bf16 split ("split3":
 operands keep 16 significant bits and the lo*lo product is dropped, so each
 product is off by at most 3 * 2^-18 = 1.1e-5 relative; over K <= 256 terms of
 an O(1) row that is 1e-4 relative / 4e-5 absolute, stated here and checked
@@ -23,7 +24,7 @@ pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-4, 1e-5
 
 
-@pytest.fixture(autouse=True, params=["fp32", "split6", "split3"])
+@pytest.fixture(autouse=True, params=["fp32", "split_f16", "split6", "split3"])
 def gemm_precision(request):
     """Runs every test of this file under both multiplication modes; ATOL follows."""
     from cxgnncomp_backend import _typed
@@ -242,3 +243,45 @@ def test_typed_gemm_wgrad(K, N, R, M):
     again = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg, M, R, src_idx=src.cuda()[perm], dst_idx=dst.cuda()[perm])
     assert torch.equal(gw, again)                                   # deterministic
     assert _typed.typed_gemm_wgrad(torch.zeros(4, 130).cuda(), g.cuda(), seg, 0, R) is None   # K > 128: not taken
+
+
+@pytest.mark.parametrize("K,N", [(128, 128), (64, 96), (20, 40)])
+def test_typed_gemm_scaled_fp16_dynamic_range(K, N):
+    """The three-product form on scaled fp16 parts keeps fp32-grade accuracy whatever the scale of
+    a row or of a weight column: rows spread over e^+-9, elements inside a row over e^+-4.5, rows
+    at 1e-30 and 1e+15, all-zero rows, weight columns over e^+-9.  The error of every output is
+    bounded against sum_k |x||w| of its dot product -- what the rounding of an fp32 product chain is
+    relative to -- with 2e-6 (fp32 MFMA: 9e-7 on this input, six bf16 products: 6e-7, three bf16
+    products: 2e-5).  An infinity in a row makes that row non-finite, as in fp32."""
+    from cxgnncomp_backend import _typed
+    M, R = 6000, 3
+    gen = torch.Generator().manual_seed(K * N)
+    x = torch.randn(M, K, generator=gen)
+    x *= torch.exp(torch.randn(M, 1, generator=gen) * 3)
+    x *= torch.exp(torch.randn(M, K, generator=gen) * 1.5)
+    x[:50] = 0
+    x[50:100] *= 1e-30
+    x[100:150] *= 1e15
+    w = torch.randn(R, K, N, generator=gen) * torch.exp(torch.randn(R, 1, N, generator=gen) * 3)
+    w[1, :, 3] = 0                                                  # an all-zero weight column
+    seg = torch.tensor([0, 2500, 2501, M], dtype=torch.int64)
+    announce("typed_gemm split_f16 dynamic range K=%d N=%d" % (K, N))
+    out = _typed.typed_gemm(x.cuda(), w.cuda(), seg.cuda(), M, precision="split_f16").cpu().double()
+    ref = torch.empty(M, N, dtype=torch.float64)
+    mag = torch.empty(M, N, dtype=torch.float64)
+    for r in range(R):
+        b, e = int(seg[r]), int(seg[r + 1])
+        ref[b:e] = x[b:e].double() @ w[r].double()
+        mag[b:e] = x[b:e].double().abs() @ w[r].double().abs()
+    assert torch.isfinite(out).all()
+    assert torch.equal(out[:50], torch.zeros(50, N, dtype=torch.float64))
+    # rows whose largest magnitude is an fp32 denormal (below 2^-112 here: the 1e-30 rows times
+    # e^-9) are treated as zero rows; everything else obeys the bound
+    err = (out - ref).abs()
+    ok = err <= 2e-6 * mag + 1e-33
+    assert ok.all(), "worst error / sum|x||w| = %.3e" % float((err / mag.clamp_min(1e-300))[~ok].max())
+    xi = x.clone()
+    xi[7, 5] = float("inf")
+    bad = _typed.typed_gemm(xi.cuda(), w.cuda(), seg.cuda(), M, precision="split_f16").cpu()
+    assert not torch.isfinite(bad[7]).any() or (w[0, 5] == 0).any()
+    assert torch.isfinite(bad[8]).all()
