@@ -321,6 +321,36 @@ def test_c4_typed_linear_s2d_full_size(hetero, hetero_ref):
     _close_scaled(out, want + 0.5, 1e-4, 1e-5, "typed_linear_s2d")
 
 
+def test_c4_edge_row_gemm_and_weight_gradient_full_size(hetero, hetero_ref):
+    """The typed GEMM and its weight gradient over the 20 M relation-sorted edge rows with row
+    maps: at this size a GEMM block holds its largest number of mapped tiles (16) and a
+    weight-gradient chunk its largest number of mapped rows (2,048).  Checks: the per-edge product
+    rows, written at the edges' CSR positions and summed per destination by the plain SpMM, are the
+    fused aggregation (float64 reference on every row); a sample of single edge rows against
+    float64; the weight gradient over the edge rows against the float64 one, and deterministic."""
+    from cxgnncomp_backend import _ops, _typed
+    ptr, idx, etype, rows, x, w, g = hetero
+    want_out, _, want_gw = hetero_ref
+    perm, seg = _typed.rel_segment(etype.int(), C4_R)
+    src, dst = idx[perm], rows[perm]
+    announce("typed GEMM with gather and scatter maps at 20M edge rows")
+    per_edge = torch.empty(C4_E, C4_K, device="cuda")
+    _typed.typed_gemm(x, w, seg, C4_E, src_idx=src, dst_idx=perm, out=per_edge)
+    pick = torch.randint(0, C4_E, (4096,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(5))
+    rel_of = etype[pick]
+    want_rows = torch.bmm(x[idx[pick]].double().unsqueeze(1), w.double()[rel_of]).squeeze(1)
+    _close_scaled(per_edge[pick], want_rows, 1e-4, 1e-5, "per-edge product rows", floor=float(want_rows.abs().max()))
+    out = _ops.spmm(ptr, torch.arange(C4_E, device="cuda"), per_edge, C4_N)
+    del per_edge
+    _close_scaled(out, want_out, 1e-4, 1e-5, "sum of the per-edge rows")
+    announce("weight gradient with row maps at 20M edge rows")
+    gw = _typed.typed_gemm_wgrad(x, g, seg, C4_E, C4_R, src_idx=src, dst_idx=dst)
+    assert gw is not None
+    _close_scaled(gw, want_gw, 1e-4, 1e-5, "weight gradient over edge rows", floor=float(want_gw.abs().max()))
+    again = _typed.typed_gemm_wgrad(x, g, seg, C4_E, C4_R, src_idx=src, dst_idx=dst)
+    assert torch.equal(gw, again)
+
+
 def test_c4_rel_schedule_full_size(hetero):
     """The 16 per-relation sub-graphs of the 20M-edge graph, bit for bit against the CPU oracle."""
     import cxgnncomp_backend as B
