@@ -329,10 +329,11 @@ __device__ __forceinline__ void split_bf16(float x, __bf16 (&p)[NS]) {
 // a0*b1, a1*b0, a0*b0 (the dropped a1*b1 is below 2^-22 |ab|) on v_mfma_f32_32x32x16_f16,
 // and the accumulator is multiplied by the two inverse scales when the tile is stored.
 // Three matrix instructions and two LDS parts per k-step instead of six and three, at
-// 2^-21 per product (fp32 itself rounds every product to 2^-24).  An element far below
-// its row's maximum loses low bits of h1 to the fp16 exponent range, which is an error
-// below 2^-29 of the row maximum -- invisible next to the rounding of the larger terms
-// of the same dot product.  bf16 has no such range limit but only 8 bits per part.
+// 2^-21 per product (fp32 itself rounds every product to 2^-24).  The matrix instruction
+// keeps fp16 subnormals, so an element keeps its 22 bits down to 2^-17 of its row's
+// maximum and is off by at most 2^-39 of that maximum below -- invisible next to the
+// rounding of the larger terms of the same dot product.  bf16 has no such range limit
+// but only 8 bits per part.
 //
 // scale 2^(14 - e) and its inverse for a maximum with biased exponent `eb` (e = eb - 127);
 // all-zero (or denormal) rows / columns get scale 0, rows with an infinity or NaN scale 1.

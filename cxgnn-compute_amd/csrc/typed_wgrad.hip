@@ -30,6 +30,8 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kXcds = 8;                 // accelerator dies of an MI355X, one L2 each
@@ -85,24 +87,57 @@ __device__ __forceinline__ bool locate_chunk(const int64_t* __restrict__ seg, in
 // tile, so a chunk has at most kMappedRows rows then.  The loads of a wave complete in order:
 // a map load inside the tile loop would make its wave wait for the row loads issued before
 // it, the loads that are meant to stay in flight while two tiles are staged.
+//
+// Scaled fp16 parts (F16): two fp16 parts per operand and three products instead of three bf16
+// parts and six products.  fp16's exponent range is narrow, so the values are scaled by a power
+// of two first -- and since the reduction runs over the rows, a scale may depend on the column
+// only.  A producer wave owns the same 32 columns of its operand through all tiles of the chunk
+// and scales them by 2^(14 - e), e the exponent of the largest magnitude it has met in those
+// columns SO FAR in the chunk (it only grows); the consumer keeps each accumulator block in
+// the units of the current scales, multiplies it by the (rare) power-of-two step when a scale
+// grows, and undoes the final scales when it stores.  The matrix instruction keeps fp16
+// subnormals, so an element keeps 22 significant bits down to 2^-17 of its column group's
+// largest magnitude and is off by at most 2^-39 of that magnitude below.
 constexpr int kWgThreads = 768;
 constexpr int kMappedRows = 2048;
+constexpr int kExpBytes = 64;            // F16: biased exponents [operand][tile buffer][column group] as int
 
 template <int NS>
 constexpr size_t wgrad_lds_bytes(bool mapped) {
-  return (size_t)2 * 2 * NS * 128 * kMP * sizeof(uint16_t) + (mapped ? (size_t)2 * kMappedRows * sizeof(int64_t) : 0);
+  return (size_t)2 * 2 * NS * 128 * kMP * sizeof(uint16_t) + kExpBytes +
+         (mapped ? (size_t)2 * kMappedRows * sizeof(int64_t) : 0);
 }
 
-template <int NS, bool MAPPED>
+template <int CTRL>
+__device__ __forceinline__ unsigned dpp_max_u32(unsigned m) {
+  const unsigned o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)m, CTRL, 0xf, 0xf, false);
+  return o > m ? o : m;
+}
+// largest value over the wave, wave-uniform
+__device__ __forceinline__ unsigned wave_max_u32(unsigned m) {
+  m = dpp_max_u32<0xB1>(m);                  // quad_perm [1,0,3,2]
+  m = dpp_max_u32<0x4E>(m);                  // quad_perm [2,3,0,1]
+  m = dpp_max_u32<0x141>(m);                 // row_half_mirror
+  m = dpp_max_u32<0x140>(m);                 // row_mirror
+  const unsigned a = (unsigned)__builtin_amdgcn_readlane((int)m, 0), b = (unsigned)__builtin_amdgcn_readlane((int)m, 16);
+  const unsigned c = (unsigned)__builtin_amdgcn_readlane((int)m, 32), d = (unsigned)__builtin_amdgcn_readlane((int)m, 48);
+  const unsigned ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
+}
+
+template <int NS, bool MAPPED, bool F16>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(3)))
 void typed_wgrad_split_kernel(WgradArgs g) {
+  static_assert(!F16 || NS == 2, "the fp16 form has two parts");
   extern __shared__ __attribute__((aligned(16))) uint16_t s_tiles[];
   typedef uint16_t (*tile_t)[128][kMP];                       // [part][column][row]
-  // s_tiles: At[2][NS][128][kMP], then Gt[2][NS][128][kMP], then (MAPPED) s_map[2][kMappedRows]
+  // s_tiles: At[2][NS][128][kMP], then Gt[2][NS][128][kMP], then s_exp[2][2][4], then (MAPPED)
+  // s_map[2][kMappedRows]
   auto tile_buf = [&](int operand, int b) -> tile_t {
     return reinterpret_cast<tile_t>(s_tiles + (size_t)(2 * operand + b) * NS * 128 * kMP);
   };
-  int64_t* const s_map = reinterpret_cast<int64_t*>(s_tiles + (size_t)4 * NS * 128 * kMP);   // [operand][row of the chunk]
+  int (*s_exp)[2][4] = reinterpret_cast<int (*)[2][4]>(s_tiles + (size_t)4 * NS * 128 * kMP);   // [operand][buffer][column group]
+  int64_t* const s_map = reinterpret_cast<int64_t*>(reinterpret_cast<unsigned char*>(s_exp) + kExpBytes);   // [operand][row of the chunk]
   // The column tiles of one row chunk get consecutive slots of one XCD (blocks go to
   // the 8 XCDs round-robin by index), so the chunk's A rows are fetched into one L2.
   const int n_ct = (g.N + 127) / 128;
@@ -169,6 +204,7 @@ void typed_wgrad_split_kernel(WgradArgs g) {
       live_mask = mask;
     };
     // registers (4 rows x 4 columns) -> LDS [column][4 consecutive rows], split into parts
+    int e_run = 0;                                     // F16: largest biased exponent met in this wave's columns
     auto stage_tile = [&](const float4 (&r4)[4], unsigned live_mask, int t) {
       if (t >= n_tiles) return;
       const tile_t dst = tile_buf(operand, t & 1);
@@ -180,6 +216,35 @@ void typed_wgrad_split_kernel(WgradArgs g) {
         v[i][1] = live ? r4[i].y : 0.f;
         v[i][2] = live ? r4[i].z : 0.f;
         v[i][3] = live ? r4[i].w : 0.f;
+      }
+      if constexpr (F16) {
+        unsigned m = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const unsigned b = __float_as_uint(v[i][c]) & 0x7fffffffu;
+            m = b > m ? b : m;
+          }
+        int eb = (int)(wave_max_u32(m) >> 23);
+        eb = eb > 254 ? 254 : eb;                      // an infinity or NaN still comes out non-finite
+        e_run = eb > e_run ? eb : e_run;
+        const float scale = e_run >= 15 ? __uint_as_float((unsigned)(268 - e_run) << 23) : 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          v4h out[2];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float xs = v[i][c] * scale;
+            const _Float16 h0 = (_Float16)xs;
+            out[0][i] = h0;
+            out[1][i] = (_Float16)(xs - (float)h0);
+          }
+#pragma unroll
+          for (int q = 0; q < 2; ++q) *reinterpret_cast<v4h*>(&dst[q][4 * c4 + c][mg * 4]) = out[q];
+        }
+        if (lane == 0) s_exp[operand][t & 1][pwave] = e_run;
+        return;
       }
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
@@ -227,11 +292,28 @@ void typed_wgrad_split_kernel(WgradArgs g) {
   for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[nb][i] = 0.f;
+  int e_a = 0, e_g[4] = {0, 0, 0, 0};                  // F16: the exponents the accumulator blocks are scaled by
   if (n_tiles > 0) {
     __syncthreads();                                   // #1
     __syncthreads();                                   // #2
     for (int t = 0; t < n_tiles; ++t) {
       const tile_t At = tile_buf(0, t & 1), Gt = tile_buf(1, t & 1);
+      if constexpr (F16) {
+        // a scale that grew since the last tile: bring the accumulator block to the new units
+        const int na = s_exp[0][t & 1][wave];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+          const int ng = s_exp[1][t & 1][nb];
+          const int d = (na - e_a) + (ng - e_g[nb]);   // >= 0: the exponents only grow
+          if (d != 0) {
+            const float f = d >= 126 ? 0.f : __uint_as_float((unsigned)(127 - d) << 23);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nb][i] *= f;
+          }
+          e_g[nb] = ng;
+        }
+        e_a = na;
+      }
 #pragma unroll
       for (int ms = 0; ms < kMT / 16; ++ms) {
         const int m = ms * 16 + (lane >> 5) * 8;
@@ -246,11 +328,27 @@ void typed_wgrad_split_kernel(WgradArgs g) {
 #pragma unroll
           for (int order = NS - 1; order >= 0; --order)
 #pragma unroll
-            for (int i = 0; i <= order; ++i)
-              acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[order - i], acc[nb], 0, 0, 0);
+            for (int i = 0; i <= order; ++i) {
+              if constexpr (F16)
+                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, af[i]),
+                                                                 __builtin_bit_cast(v8h, bf[order - i]), acc[nb], 0, 0, 0);
+              else
+                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[order - i], acc[nb], 0, 0, 0);
+            }
         }
       }
       __syncthreads();   // tile t+1 is staged, and every wave is done with tile t
+    }
+  }
+  if constexpr (F16) {
+    // undo the scales 2^(14 - (e - 127)) of the two operands, the smaller factor first
+    const float fa = e_a >= 15 ? __uint_as_float((unsigned)(e_a - 14) << 23) : 0.f;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      const float fg = e_g[nb] >= 15 ? __uint_as_float((unsigned)(e_g[nb] - 14) << 23) : 0.f;
+      const float f1 = fa < fg ? fa : fg, f2 = fa < fg ? fg : fa;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nb][i] = acc[nb][i] * f1 * f2;
     }
   }
   // partial[chunk][k][n] (zeros for chunk numbers past the last relation)
@@ -339,7 +437,8 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
                              int64_t M, int K, int N, int R, float* gw, unsigned flags, void* workspace,
                              size_t workspace_bytes, void* stream) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
-  CXG_REQUIRE((flags & ~(CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3)) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE((flags & ~(CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) == 0, CXG_ERR_ARG,
+              "unknown flag");
   CXG_REQUIRE(gw && seg_ptr, CXG_ERR_ARG, "null gw/seg_ptr");
   CXG_REQUIRE(M == 0 || (a && g), CXG_ERR_ARG, "null a/g");
   CXG_REQUIRE(K <= 128 && (K & 3) == 0 && (N & 3) == 0 && (lda & 3) == 0 && (ldg & 3) == 0 &&
@@ -359,17 +458,20 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
   cxg::WgradArgs wa{a, lda, g, ldg, src_idx, dst_idx, seg_ptr, reinterpret_cast<float*>(workspace),
                     M, K, N, R, rows};
   const dim3 grid((unsigned)(chunks * n_ct)), block(cxg::kWgThreads);
-#define CXG_WGRAD_LAUNCH(NSV, MAP)                                                                        \
+#define CXG_WGRAD_LAUNCH(NSV, MAP, HALF)                                                                  \
   do {                                                                                                    \
-    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_wgrad_split_kernel<NSV, MAP>, cxg::wgrad_lds_bytes<NSV>(MAP))); \
-    hipLaunchKernelGGL((cxg::typed_wgrad_split_kernel<NSV, MAP>), grid, block, cxg::wgrad_lds_bytes<NSV>(MAP), st, wa); \
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_wgrad_split_kernel<NSV, MAP, HALF>, cxg::wgrad_lds_bytes<NSV>(MAP))); \
+    hipLaunchKernelGGL((cxg::typed_wgrad_split_kernel<NSV, MAP, HALF>), grid, block, cxg::wgrad_lds_bytes<NSV>(MAP), st, wa); \
   } while (0)
-  if (flags & CXG_GEMM_SPLIT_BF16X3) {
-    if (mapped) CXG_WGRAD_LAUNCH(2, true);
-    else CXG_WGRAD_LAUNCH(2, false);
+  if (flags & CXG_GEMM_SPLIT_F16X3) {
+    if (mapped) CXG_WGRAD_LAUNCH(2, true, true);
+    else CXG_WGRAD_LAUNCH(2, false, true);
+  } else if (flags & CXG_GEMM_SPLIT_BF16X3) {
+    if (mapped) CXG_WGRAD_LAUNCH(2, true, false);
+    else CXG_WGRAD_LAUNCH(2, false, false);
   } else {
-    if (mapped) CXG_WGRAD_LAUNCH(3, true);
-    else CXG_WGRAD_LAUNCH(3, false);
+    if (mapped) CXG_WGRAD_LAUNCH(3, true, false);
+    else CXG_WGRAD_LAUNCH(3, false, false);
   }
 #undef CXG_WGRAD_LAUNCH
   CXG_LAUNCH_CHECK("typed_wgrad_split_kernel");

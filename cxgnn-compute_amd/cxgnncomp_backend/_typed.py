@@ -20,8 +20,9 @@ GEMM_SPLIT_F16X3 = 16
 # per product -- fp32-grade -- and HBM bound for K <= 128), "split6" (six bf16 partial products,
 # 2^-24), "split3" (three bf16 partial products, relative error below 2^-16 per product), "fp32"
 # (v_mfma_f32_32x32x2_f32) or "bf16" (operands rounded to bf16, one bf16 MFMA product, fp32
-# accumulation; weight gradients then use "split3").  Weight gradients, whose reduction runs
-# over the rows, take "split6" for "split_f16".
+# accumulation; weight gradients then use "split3").  The weight-gradient kernel has the same
+# forms; its "split_f16" scales per 32-column group instead of per row, since its reduction runs
+# over the rows.
 GEMM_PRECISION = os.environ.get("CXGNN_GEMM_PRECISION", "split_f16")
 _PRECISION_FLAGS = {"fp32": 0, "split6": GEMM_SPLIT_BF16X6, "split3": GEMM_SPLIT_BF16X3,
                     "split_f16": GEMM_SPLIT_F16X3}
@@ -260,7 +261,8 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     if K % 4 or N % 4 or (K > 128 and num_rel != 1):
         return None
     precision = precision or GEMM_PRECISION
-    flags = GEMM_SPLIT_BF16X3 if precision in ("split3", "bf16") else GEMM_SPLIT_BF16X6
+    flags = (GEMM_SPLIT_F16X3 if precision == "split_f16" else
+             GEMM_SPLIT_BF16X3 if precision in ("split3", "bf16") else GEMM_SPLIT_BF16X6)
     gw = torch.empty((num_rel, K, N), dtype=torch.float32, device=a.device)
     with torch.cuda.device(a.device):
         for k0 in range(0, K, 128):

@@ -314,7 +314,11 @@ int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, flo
  * rows give zeros.  A is [*, K] (row stride lda), G is [*, N] (row stride ldg);
  * src / dst / seg_ptr as in cxg_typed_gemm_f32.  fp32 operands multiplied as six
  * (CXG_GEMM_SPLIT_BF16X6 or no flag) or three (CXG_GEMM_SPLIT_BF16X3) bf16 partial
- * products on v_mfma_f32_32x32x16_bf16; partial sums over row chunks are added in
+ * products on v_mfma_f32_32x32x16_bf16, or (CXG_GEMM_SPLIT_F16X3) as three fp16
+ * partial products of operands scaled by a power of two per group of 32 columns and
+ * row chunk (the scale follows the largest magnitude met so far in the chunk; an
+ * element keeps 22 significant bits down to 2^-17 of that magnitude); partial sums
+ * over row chunks are added in
  * chunk order by a second kernel (deterministic).  Needs K <= 128, K, N, lda, ldg
  * multiples of 4 and 16-byte aligned operands (otherwise CXG_ERR_UNSUPPORTED).
  * Replaces the per-relation torch.mm of TypedLinearE2EOP.backward and

@@ -285,3 +285,36 @@ def test_typed_gemm_scaled_fp16_dynamic_range(K, N):
     bad = _typed.typed_gemm(xi.cuda(), w.cuda(), seg.cuda(), M, precision="split_f16").cpu()
     assert not torch.isfinite(bad[7]).any() or (w[0, 5] == 0).any()
     assert torch.isfinite(bad[8]).all()
+
+
+@pytest.mark.parametrize("K,N,M", [(128, 128, 30000), (64, 96, 9000), (20, 40, 5000)])
+def test_typed_gemm_wgrad_scaled_fp16_dynamic_range(K, N, M):
+    """The weight gradient on scaled fp16 parts: its scales depend on the column group only and
+    follow the largest magnitude met so far in the chunk, so rows of very different size share a
+    scale.  Rows spread over e^+-9 (both operands, independently), elements over e^+-3, blocks of
+    all-zero rows, the first rows tiny (the scales have to grow inside a chunk): the error of
+    every gw element is bounded against sum_i |a||g| of its reduction with 4e-6 (measured 6e-7;
+    six bf16 products: 5e-7, three bf16 products: 2e-5 on this input)."""
+    from cxgnncomp_backend import _typed
+    R = 3
+    gen = torch.Generator().manual_seed(K + N + M)
+    a = torch.randn(M, K, generator=gen) * torch.exp(torch.randn(M, 1, generator=gen) * 3)
+    a *= torch.exp(torch.randn(M, K, generator=gen))
+    g = torch.randn(M, N, generator=gen) * torch.exp(torch.randn(M, 1, generator=gen) * 3)
+    g *= torch.exp(torch.randn(M, N, generator=gen))
+    a[:300] *= 1e-12
+    g[:300] *= 1e-9
+    a[1000:1400] = 0
+    g[1200:1500] = 0
+    seg = torch.tensor([0, M // 2, M // 2 + 1, M], dtype=torch.int64)
+    announce("typed_gemm_wgrad split_f16 dynamic range K=%d N=%d M=%d" % (K, N, M))
+    gw = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg.cuda(), M, R, precision="split_f16")
+    assert gw is not None and bool(torch.isfinite(gw).all())
+    gw = gw.cpu().double()
+    for r in range(R):
+        b, e = int(seg[r]), int(seg[r + 1])
+        want = a[b:e].double().t() @ g[b:e].double()
+        mag = a[b:e].double().abs().t() @ g[b:e].double().abs()
+        err = (gw[r] - want).abs()
+        ok = err <= 4e-6 * mag + 1e-30
+        assert ok.all(), "relation %d: worst error / sum|a||g| = %.3e" % (r, float((err / mag.clamp_min(1e-300))[~ok].max()))
