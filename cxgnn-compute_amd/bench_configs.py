@@ -389,6 +389,18 @@ def c4(iters):
            timeit(lambda: _typed.typed_gemm(xe16, w, seg, E, out=oe, bf16=True), iters),
            E * 6 * K + 2 * R * K * K, flops, MFMA_BF16)
     del xe, oe, xe16
+    # the hidden-256 shape of a deeper relational model: 5M rows x 256 x 256
+    E2, K2 = 5000000, 256
+    x2 = torch.randn(E2, K2, device="cuda") / 8
+    w2 = torch.randn(R, K2, K2, device="cuda") * 0.02
+    seg2 = (seg.double() * (E2 / E)).long()
+    seg2[-1] = E2
+    o2 = torch.empty(E2, K2, device="cuda")
+    for prec, what in (("fp32", "fp32 MFMA"), ("split_f16", "3 scaled fp16 products (default)")):
+        report("c4", "typed GEMM 5M rows x 256 x 256, %s" % what,
+               timeit(lambda: _typed.typed_gemm(x2, w2, seg2, E2, out=o2, precision=prec), iters),
+               E2 * 8 * K2 + 4 * R * K2 * K2, 2.0 * E2 * K2 * K2, MFMA_F32 if prec == "fp32" else None)
+    del x2, w2, o2
     global _last_spread
     t_mm = (E / N) * timeit(lambda: torch.mm(x, w[0]), iters)
     _last_spread = tuple((E / N) * v for v in _last_spread)

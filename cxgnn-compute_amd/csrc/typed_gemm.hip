@@ -368,6 +368,10 @@ __device__ __forceinline__ unsigned group_max_u32(unsigned m) {
     const unsigned o = (unsigned)__builtin_amdgcn_ds_swizzle((int)m, 0x401F);   // lane ^ 16
     m = o > m ? o : m;
   }
+  if (LANES >= 64) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)m, 0), hi = (unsigned)__builtin_amdgcn_readlane((int)m, 32);
+    m = lo > hi ? lo : hi;
+  }
   return m;
 }
 
@@ -394,11 +398,11 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   uint16_t (*Ap)[NS][kBM][KP] = reinterpret_cast<uint16_t (*)[NS][kBM][KP]>(smem);
   int64_t (*s_src)[kBM] = reinterpret_cast<int64_t (*)[kBM]>(smem + sizeof(uint16_t) * 2 * NS * kBM * KP);
   int64_t (*s_dst)[kBM] = s_src + SLOTS;
-  float (*Cw)[kCP] = reinterpret_cast<float (*)[kCP]>(reinterpret_cast<unsigned char*>(s_dst + SLOTS)) +
+  // F16: inverse row scales of the two staged tiles, [2][kBM] floats; then the staging areas (the
+  // widest form, KS = 16, has no room for them and stores from the accumulators)
+  float (*s_inv)[kBM] = reinterpret_cast<float (*)[kBM]>(s_dst + SLOTS);
+  float (*Cw)[kCP] = reinterpret_cast<float (*)[kCP]>(reinterpret_cast<unsigned char*>(s_inv + 2)) +
                      (size_t)(threadIdx.x >> 6 & 3) * kBM;
-  // F16: inverse row scales of the two staged tiles, [2][kBM] floats behind the four staging areas
-  float (*s_inv)[kBM] = reinterpret_cast<float (*)[kBM]>(
-      reinterpret_cast<unsigned char*>(s_dst + SLOTS) + (size_t)4 * kBM * kCP * sizeof(float));
   const int64_t span = (int64_t)kBM * G;
   int rel = -1;
   int64_t row0 = 0, row_end = 0;
@@ -428,7 +432,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
   // stores (or read-add-stores) of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
-  const bool wide_store = !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
+  const bool wide_store = KS <= 8 && !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
                           ((uintptr_t)g.c & 15) == 0;
 
   // ---- producer state -------------------------------------------------------------
@@ -547,16 +551,32 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       const float* W = reinterpret_cast<const float*>(g.w) + (int64_t)rel * K * N;
       const int col = n0 + wave * 32 + (lane & 31);
       if constexpr (F16) {
-        float wv[KS][8];
+        // the column's largest magnitude, then its scaled parts; eight k-steps (64 values) are
+        // loaded at a time, and a column of more than that is read twice (the second time out
+        // of the caches)
+        constexpr int HS = KS < 8 ? KS : 8;    // k-steps per batch
+        float wv[HS][8];
+        auto w_load = [&](int s0) {
+#pragma unroll
+          for (int s = 0; s < HS; ++s) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int k = (s0 + s) * 16 + (lane >> 5) * 8 + j;
+              wv[s][j] = (k < K && col < N) ? W[(int64_t)k * N + col] : 0.f;
+            }
+          }
+        };
         unsigned m = 0;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
+        for (int s0 = 0; s0 < KS; s0 += HS) {
+          w_load(s0);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int k = s * 16 + (lane >> 5) * 8 + j;
-            wv[s][j] = (k < K && col < N) ? W[(int64_t)k * N + col] : 0.f;
-            const unsigned b = __float_as_uint(wv[s][j]) & 0x7fffffffu;
-            m = b > m ? b : m;
+          for (int s = 0; s < HS; ++s) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const unsigned b = __float_as_uint(wv[s][j]) & 0x7fffffffu;
+              m = b > m ? b : m;
+            }
           }
         }
         // the other half of the column's k range sits in lane ^ 32
@@ -565,16 +585,20 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
         float scale;
         pow2_scales(m, scale, inv_w);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          v8h h0, h1;
+        for (int s0 = 0; s0 < KS; s0 += HS) {
+          if (KS > HS) w_load(s0);             // one batch: the values are still there
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const float xs = wv[s][j] * scale;
-            h0[j] = (_Float16)xs;
-            h1[j] = (_Float16)(xs - (float)h0[j]);
+          for (int s = 0; s < HS; ++s) {
+            v8h h0, h1;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float xs = wv[s][j] * scale;
+              h0[j] = (_Float16)xs;
+              h1[j] = (_Float16)(xs - (float)h0[j]);
+            }
+            bw[0][s0 + s] = __builtin_bit_cast(v8bf, h0);
+            bw[1][s0 + s] = __builtin_bit_cast(v8bf, h1);
           }
-          bw[0][s] = __builtin_bit_cast(v8bf, h0);
-          bw[1][s] = __builtin_bit_cast(v8bf, h1);
         }
       } else {
 #pragma unroll
@@ -597,7 +621,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
     // instructions, so four times the bytes in flight for the same depth of the memory
     // queue.  The eight pieces of tile t-1 are read back and stored between the k-steps
     // of tile t, in the shadow of its MFMAs.
-    constexpr int PPS = 8 / KS;              // pieces per k-step
+    constexpr int PPS = KS <= 8 ? 8 / KS : 1;   // pieces per k-step
     auto piece_read = [&](int it) -> float4 {
       return *reinterpret_cast<const float4*>(&Cw[it * 8 + (lane >> 3)][(lane & 7) * 4]);
     };
@@ -650,6 +674,8 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
           }
         }
         // the two accumulators alternate, so consecutive MFMAs never depend on each other
+        // (k-steps past K multiply zeros: a test of K around them was measured and costs more
+        // than it saves, 1.49 -> 1.91 ms at K = 128 -- it breaks the schedule of the loop)
 #pragma unroll
         for (int order = NS - 1; order >= 0; --order)
 #pragma unroll
@@ -880,8 +906,12 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   cxg::GemmArgs g{a, lda, w, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
                   (int)(flags & 1u), (int)((flags >> 1) & 1u)};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && K <= 128 && (K & 3) == 0 && (lda & 3) == 0 &&
-      ((uintptr_t)a & 15) == 0) {
+  // Two fp16 parts of a 256-wide tile still fit the LDS: K up to 256 takes the fp16 form when the
+  // 256 x 128 tile is mostly used (measured against the fp32 instructions at 7.3 M rows: K = 256,
+  // N = 256 10.6 -> 5.8 ms, N = 128 5.3 -> 3.3 ms; K = 160, N = 64 2.0 -> 2.5 ms).
+  const bool wide_k = (flags & CXG_GEMM_SPLIT_F16X3) && K > 128 && K <= 256 && K >= 176 && N >= 96;
+  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
+      (lda & 3) == 0 && ((uintptr_t)a & 15) == 0) {
     // 64*G rows per block: up to 32 tiles (16 with row maps, which the block keeps in LDS)
     // while the launch keeps a few thousand blocks
     const bool mapped = src_idx || dst_idx;
@@ -904,7 +934,7 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
     const int ns = (half || (flags & CXG_GEMM_SPLIT_BF16X3)) ? 2 : 3;                          \
     const size_t lds = (size_t)2 * ns * cxg::kBM * (KS * 16 + 8) * sizeof(uint16_t) +          \
                        (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) + \
-                       (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float) +                       \
+                       (KS <= 8 ? (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float) : 0) +       \
                        (size_t)2 * cxg::kBM * sizeof(float);                                   \
     if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                                   \
     else if (half) CXG_SPLIT_LAUNCH(KS, 2, false, true);                                       \
@@ -915,7 +945,14 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   } while (0)
     if (K <= 32) CXG_SPLIT(2);
     else if (K <= 64) CXG_SPLIT(4);
-    else CXG_SPLIT(8);
+    else if (K <= 128) CXG_SPLIT(8);
+    else {                                   // 128 < K <= 256: the fp16 form only
+      const size_t lds = (size_t)2 * 2 * cxg::kBM * (16 * 16 + 8) * sizeof(uint16_t) +
+                         (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) +
+                         (size_t)2 * cxg::kBM * sizeof(float);
+      if (mapped) CXG_SPLIT_LAUNCH(16, 2, true, true);
+      else CXG_SPLIT_LAUNCH(16, 2, false, true);
+    }
 #undef CXG_SPLIT_LAUNCH
 #undef CXG_SPLIT
     CXG_LAUNCH_CHECK("typed_gemm_split_kernel");

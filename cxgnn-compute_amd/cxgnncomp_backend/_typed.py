@@ -250,15 +250,15 @@ def _edge_positions(n, device):
 
 def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=None, precision=None):
     """gw[r] = sum over the rows i of segment r of a[src(i)]^T (x) g[dst(i)] -> [num_rel, K, N]
-    (see cxg_typed_gemm_wgrad_f32).  One launch takes K <= 128; a single-relation product
-    with a wider K runs as one launch per 128 columns of ``a``, each writing its own rows
-    of gw.  Returns None for shapes the kernel does not take (K > 128 with several
-    relations, or K / N not multiples of 4)."""
+    (see cxg_typed_gemm_wgrad_f32).  One launch takes K <= 128; a wider K runs as one launch per
+    128 columns of ``a`` (a single relation writes its rows of gw in place, several relations go
+    through a [num_rel, 128, N] buffer per slice).  Returns None for shapes the kernel does not
+    take (K or N not multiples of 4)."""
     lib = _lib.load()
     _req(a, "a", torch.float32, 2)
     _req(g, "g", torch.float32, 2)
     K, N = a.shape[1], g.shape[1]
-    if K % 4 or N % 4 or (K > 128 and num_rel != 1):
+    if K % 4 or N % 4:
         return None
     precision = precision or GEMM_PRECISION
     flags = (GEMM_SPLIT_F16X3 if precision == "split_f16" else
@@ -267,12 +267,16 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     with torch.cuda.device(a.device):
         for k0 in range(0, K, 128):
             kb = min(128, K - k0)
+            direct = num_rel == 1 or kb == K
+            part = gw if direct else torch.empty((num_rel, kb, N), dtype=torch.float32, device=a.device)
             ws = _workspace(lib.cxg_typed_gemm_wgrad_workspace_bytes(m_rows, kb, N, num_rel), a.device)
             st = lib.cxg_typed_gemm_wgrad_f32(a.data_ptr() + 4 * k0, K, g.data_ptr(), N, _lib.ptr(src_idx),
                                               _lib.ptr(dst_idx), seg_ptr.data_ptr(), m_rows, kb, N, num_rel,
-                                              gw.data_ptr() + 4 * k0 * N, flags, ws.data_ptr(), ws.numel(),
-                                              _lib.current_stream(a.device))
+                                              part.data_ptr() + (4 * k0 * N if direct else 0), flags, ws.data_ptr(),
+                                              ws.numel(), _lib.current_stream(a.device))
             _lib.check(st)
+            if not direct:
+                gw[:, k0:k0 + kb, :] = part
     return gw
 
 

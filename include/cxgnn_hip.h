@@ -285,7 +285,8 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
  * magnitude into [2^14, 2^15) and split into two fp16 parts (22 significant bits);
  * a*b is accumulated on v_mfma_f32_32x32x16_f16 from three partial products and the
  * scales are undone when the row is stored: 2^-21 per product, half the matrix
- * instructions and two thirds of the LDS traffic of X6.  Rows or columns whose largest
+ * instructions and two thirds of the LDS traffic of X6; this form also takes
+ * 176 <= K <= 256 when N >= 96.  Rows or columns whose largest
  * magnitude is below 2^-112 count as zero; a row holding an infinity or NaN comes out
  * non-finite.  Other shapes ignore the three flags.  Replaces
  * typed_matmul

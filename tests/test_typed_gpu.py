@@ -216,11 +216,12 @@ def test_rgcn_fused_forward_backward(K, N, R, strategy, monkeypatch):
 
 
 @pytest.mark.parametrize("K,N,R,M", [(128, 128, 16, 5000), (64, 48, 3, 1000), (4, 256, 1, 3000), (128, 2048, 1, 700),
-                                     (32, 40, 4, 70000), (12, 20, 5, 1)])
+                                     (32, 40, 4, 70000), (12, 20, 5, 1), (256, 128, 5, 3000), (200, 64, 1, 900)])
 def test_typed_gemm_wgrad(K, N, R, M):
     """gw[r] = sum over the rows of relation r of a[src]^T (x) g[dst], against per-relation
     float64 products; covers several column tiles (N = 2048), K far below one tile (K = 4),
-    many row chunks (M = 70000) and relations without rows."""
+    K above one launch's 128 (in slices, one and several relations), many row chunks (M = 70000)
+    and relations without rows."""
     from cxgnncomp_backend import _typed
     gen = torch.Generator().manual_seed(K + N + M)
     n_a, n_g = max(1, M // 2), max(1, M // 3)
@@ -242,7 +243,7 @@ def test_typed_gemm_wgrad(K, N, R, M):
     assert_close(_np(gw), want.numpy(), RTOL, 2 * ATOL, "wgrad")
     again = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg, M, R, src_idx=src.cuda()[perm], dst_idx=dst.cuda()[perm])
     assert torch.equal(gw, again)                                   # deterministic
-    assert _typed.typed_gemm_wgrad(torch.zeros(4, 130).cuda(), g.cuda(), seg, 0, R) is None   # K > 128: not taken
+    assert _typed.typed_gemm_wgrad(torch.zeros(4, 130).cuda(), g.cuda(), seg, 0, R) is None   # K not a multiple of 4: not taken
 
 
 @pytest.mark.parametrize("K,N", [(128, 128), (64, 96), (20, 40)])
