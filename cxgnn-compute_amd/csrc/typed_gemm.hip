@@ -545,6 +545,13 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   // (the two kinds of waves run separate loops with the same number of barriers, so the
   // registers of one role are not live in the other)
   if (consumer) {
+    if (n0 + wave * 32 >= N) {
+      // all 32 columns of this wave lie past N (N <= 96 in the last column tile): nothing to
+      // multiply or store, only the barriers of the block
+      __syncthreads();
+      for (int t = 0; t < n_tiles; ++t) __syncthreads();
+      return;
+    }
     v8bf bw[NS][KS];                         // this wave's 32 columns of W[rel], split (F16: fp16 bit patterns)
     float inv_w = 1.f;                       // F16: inverse scale of this lane's column
     {
