@@ -286,6 +286,15 @@ void typed_wgrad_split_kernel(WgradArgs g) {
   }
 
   // ---- consumers --------------------------------------------------------------------
+  if (wave * 32 >= K) {
+    // this wave's 32 rows of gw lie past K: nothing to multiply or store, only the barriers
+    if (n_tiles > 0) {
+      __syncthreads();                                 // #1
+      __syncthreads();                                 // #2
+      for (int t = 0; t < n_tiles; ++t) __syncthreads();
+    }
+    return;
+  }
   float* const part = g.partial + ((size_t)chunk * K) * (size_t)N;
   v16f acc[4];
 #pragma unroll
