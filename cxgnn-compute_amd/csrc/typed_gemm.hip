@@ -655,20 +655,28 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
-      // operands of k-step s+1 are read while step s multiplies (two register sets)
-      v8bf ap[2][2][NS];
+      // operands of k-step s+1 are read while step s multiplies (two register sets); with one
+      // part per operand a k-step is two matrix instructions only, too short to cover an LDS
+      // read, so the operands of the whole tile are read up front then (one set per k-step)
+      constexpr int SETS = NS == 1 ? KS : 2;
+      v8bf ap[SETS][2][NS];
       auto read_ap = [&](int s) {
         const int k = s * 16 + (lane >> 5) * 8;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int q = 0; q < NS; ++q)
-            ap[s & 1][mt][q] = *reinterpret_cast<const v8bf*>(&src[q][mt * 32 + (lane & 31)][k]);
+            ap[s % SETS][mt][q] = *reinterpret_cast<const v8bf*>(&src[q][mt * 32 + (lane & 31)][k]);
       };
-      read_ap(0);
+      if constexpr (NS == 1) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) read_ap(s);
+      } else {
+        read_ap(0);
+      }
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
-        if (s + 1 < KS) read_ap(s + 1);
+        if (NS > 1 && s + 1 < KS) read_ap(s + 1);
         if (drain) {
           if (s > 0) {
 #pragma unroll
@@ -690,10 +698,10 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
               if constexpr (F16)
-                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, ap[s & 1][mt][i]),
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, ap[s % SETS][mt][i]),
                                                                  __builtin_bit_cast(v8h, bw[order - i][s]), acc[mt], 0, 0, 0);
               else
-                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s & 1][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s % SETS][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
             }
       }
       if constexpr (F16) {
@@ -893,7 +901,7 @@ hipError_t allow_lds(KernelT kernel, size_t bytes) {
 int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64_t M, int K, int N,
                int R, unsigned flags) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
-  CXG_REQUIRE((flags & ~31u) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE((flags & ~63u) == 0, CXG_ERR_ARG, "unknown flag");
   if (M == 0) return CXG_OK;
   CXG_REQUIRE(a && w && c && seg, CXG_ERR_ARG, "null pointer");
   return CXG_OK;
@@ -917,7 +925,7 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   // 256 x 128 tile is mostly used (measured against the fp32 instructions at 7.3 M rows: K = 256,
   // N = 256 10.6 -> 5.8 ms, N = 128 5.3 -> 3.3 ms; K = 160, N = 64 2.0 -> 2.5 ms).
   const bool wide_k = (flags & CXG_GEMM_SPLIT_F16X3) && K > 128 && K <= 256 && K >= 176 && N >= 96;
-  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
+  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3 | CXG_GEMM_ROUND_BF16)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
       (lda & 3) == 0 && ((uintptr_t)a & 15) == 0) {
     // 64*G rows per block: up to 32 tiles (16 with row maps, which the block keeps in LDS)
     // while the launch keeps a few thousand blocks
@@ -938,12 +946,14 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
 #define CXG_SPLIT(KS)                                                                          \
   do {                                                                                         \
     const bool half = (flags & CXG_GEMM_SPLIT_F16X3) != 0;                                     \
-    const int ns = (half || (flags & CXG_GEMM_SPLIT_BF16X3)) ? 2 : 3;                          \
+    const int ns = (flags & CXG_GEMM_ROUND_BF16) ? 1 : (half || (flags & CXG_GEMM_SPLIT_BF16X3)) ? 2 : 3; \
     const size_t lds = (size_t)2 * ns * cxg::kBM * (KS * 16 + 8) * sizeof(uint16_t) +          \
                        (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) + \
                        (KS <= 8 ? (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float) : 0) +       \
                        (size_t)2 * cxg::kBM * sizeof(float);                                   \
-    if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                                   \
+    if (ns == 1 && mapped) CXG_SPLIT_LAUNCH(KS, 1, true, false);                               \
+    else if (ns == 1) CXG_SPLIT_LAUNCH(KS, 1, false, false);                                   \
+    else if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                              \
     else if (half) CXG_SPLIT_LAUNCH(KS, 2, false, true);                                       \
     else if (ns == 2 && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, false);                          \
     else if (ns == 2) CXG_SPLIT_LAUNCH(KS, 2, false, false);                                   \

@@ -14,6 +14,7 @@ GEMM_ATOMIC = 2
 GEMM_SPLIT_BF16X6 = 4
 GEMM_SPLIT_BF16X3 = 8
 GEMM_SPLIT_F16X3 = 16
+GEMM_ROUND_BF16 = 32
 
 # How fp32 typed GEMMs multiply: "split_f16" (the default: rows of A and columns of W scaled by
 # powers of two and split into two fp16 parts, three fp16 MFMA products per fp32 product, 2^-21
@@ -97,7 +98,13 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
         flags |= _PRECISION_FLAGS[precision]
     stream = _lib.current_stream(a.device)
     with torch.cuda.device(a.device):
-        if bf16:
+        if bf16 and a.dtype == torch.float32 and K <= 128 and K % 4 == 0:
+            # fp32 operands rounded to bf16 inside the kernel: no conversion pass over a and w
+            _req(w, "weights", torch.float32, 3)
+            st = lib.cxg_typed_gemm_f32(a.data_ptr(), K, w.data_ptr(), out.data_ptr(), N,
+                                        _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
+                                        m_rows, K, N, R, (flags & (GEMM_ACCUMULATE | GEMM_ATOMIC)) | GEMM_ROUND_BF16, stream)
+        elif bf16:
             a16 = a if a.dtype == torch.bfloat16 else a.to(torch.bfloat16)
             wt16 = w.detach().transpose(1, 2).contiguous().to(torch.bfloat16)
             st = lib.cxg_typed_gemm_bf16(a16.data_ptr(), K, wt16.data_ptr(), out.data_ptr(), N,

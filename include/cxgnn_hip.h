@@ -267,6 +267,7 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
 #define CXG_GEMM_SPLIT_BF16X6 4u /* fp32 products as 6 bf16 partial products (fp32-accurate) */
 #define CXG_GEMM_SPLIT_BF16X3 8u /* fp32 products as 3 bf16 partial products (2^-16 / product) */
 #define CXG_GEMM_SPLIT_F16X3 16u /* fp32 products as 3 fp16 partial products of row- / column-scaled operands (2^-21 / product) */
+#define CXG_GEMM_ROUND_BF16 32u /* fp32 operands rounded to bf16 as they are staged, one bf16 MFMA product, fp32 accumulation */
 
 /*
  * C[dst(i), :] = A[src(i), :] @ W[r] for the rows i in [seg_ptr[r], seg_ptr[r+1]),
@@ -288,7 +289,10 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
  * instructions and two thirds of the LDS traffic of X6; this form also takes
  * 176 <= K <= 256 when N >= 96.  Rows or columns whose largest
  * magnitude is below 2^-112 count as zero; a row holding an infinity or NaN comes out
- * non-finite.  Other shapes ignore the three flags.  Replaces
+ * non-finite.  With CXG_GEMM_ROUND_BF16 (K <= 128) the fp32 operands are rounded to
+ * bf16 (nearest even) on their way into the LDS and the registers and multiplied with
+ * one bf16 MFMA per k-step: the result of cxg_typed_gemm_bf16 on the rounded operands
+ * without a conversion pass.  Other shapes ignore these flags.  Replaces
  * typed_matmul
  * (cxgnncomp/codegen/triton_typed_matmul.py:752-860: src_idx only = its
  * "single index" kernel with dst = src, seq_output = dst NULL, both = double
