@@ -319,3 +319,42 @@ def test_typed_gemm_wgrad_scaled_fp16_dynamic_range(K, N, M):
         err = (gw[r] - want).abs()
         ok = err <= 4e-6 * mag + 1e-30
         assert ok.all(), "relation %d: worst error / sum|a||g| = %.3e" % (r, float((err / mag.clamp_min(1e-300))[~ok].max()))
+
+
+@pytest.mark.parametrize("M", [1, 63, 64, 65, 1100])
+@pytest.mark.parametrize("K,N", [(128, 128), (4, 4), (36, 72), (256, 96)])
+def test_typed_gemm_small_shapes_and_skipped_rows(M, K, N):
+    """Row counts around one 64-row tile and past one block's 16 mapped tiles, K and N far below
+    and above a tile, and row maps with negative entries (a negative source or destination skips
+    the row, which is how the reference's padded layouts are accepted): forward product into
+    scattered rows and the weight gradient, against float64."""
+    from cxgnncomp_backend import _typed
+    R = 3
+    gen = torch.Generator().manual_seed(M * 1000 + K + N)
+    n_a = 2 * M + 3
+    a = torch.randn(n_a, K, generator=gen) / K ** 0.5
+    w = torch.randn(R, K, N, generator=gen)
+    types = torch.sort(torch.randint(0, R, (M,), generator=gen))[0]
+    seg = torch.zeros(R + 1, dtype=torch.int64)
+    seg[1:] = torch.bincount(types, minlength=R).cumsum(0)
+    src = torch.randint(0, n_a, (M,), generator=gen)
+    dst = torch.randperm(M + 5, generator=gen)[:M]                  # unique destinations
+    skip = torch.rand(M, generator=gen) < 0.2
+    src_m = torch.where(skip & (torch.arange(M) % 2 == 0), torch.full_like(src, -1), src)
+    dst_m = torch.where(skip & (torch.arange(M) % 2 == 1), torch.full_like(dst, -7), dst)
+    announce("typed_gemm M=%d K=%d N=%d with skipped rows" % (M, K, N))
+    out = torch.full((M + 5, N), 3.0).cuda()
+    _typed.typed_gemm(a.cuda(), w.cuda(), seg.cuda(), M, src_idx=src_m.cuda(), dst_idx=dst_m.cuda(), out=out)
+    want = torch.full((M + 5, N), 3.0, dtype=torch.float64)
+    for i in range(M):
+        if not bool(skip[i]):
+            want[dst[i]] = a[src[i]].double() @ w[types[i]].double()
+    assert_close(_np(out), want.numpy(), RTOL, 2 * ATOL, "typed_gemm with skipped rows")
+    g = torch.randn(M + 5, N, generator=gen)
+    gw = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg.cuda(), M, R, src_idx=src_m.cuda(), dst_idx=dst_m.cuda())
+    want_gw = torch.zeros(R, K, N, dtype=torch.float64)
+    for i in range(M):
+        if not bool(skip[i]):
+            want_gw[types[i]] += torch.outer(a[src[i]].double(), g[dst[i]].double())
+    scale = max(1.0, float(want_gw.abs().max()))
+    assert_close(_np(gw) / scale, want_gw.numpy() / scale, RTOL, 2 * ATOL, "wgrad with skipped rows")
