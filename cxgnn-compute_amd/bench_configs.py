@@ -475,6 +475,13 @@ def c4(iters):
         layer(xg, ptr, idx, etype, N).backward(gout)
     report("c4", "MyRGCNConv layer fwd+bwd (typed transform, relational aggregate, /deg)",
            timeit(layer_step, max(2, iters // 3)))
+    layer16 = cxgnncomp.MyRGCNConv(K, K, R, precision="bf16").cuda()
+
+    def layer16_step():
+        xg.grad = None
+        layer16(xg, ptr, idx, etype, N).backward(gout)
+    report("c4", "MyRGCNConv layer fwd+bwd, bf16 variant (operands of the forward and input-gradient GEMMs rounded to bf16)",
+           timeit(layer16_step, max(2, iters // 3)))
     if CPU_BASELINE:
         from oracle import pyref
         rows = N // 32
