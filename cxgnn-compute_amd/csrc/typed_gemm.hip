@@ -655,28 +655,20 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
-      // operands of k-step s+1 are read while step s multiplies (two register sets); with one
-      // part per operand a k-step is two matrix instructions only, too short to cover an LDS
-      // read, so the operands of the whole tile are read up front then (one set per k-step)
-      constexpr int SETS = NS == 1 ? KS : 2;
-      v8bf ap[SETS][2][NS];
+      // operands of k-step s+1 are read while step s multiplies (two register sets)
+      v8bf ap[2][2][NS];
       auto read_ap = [&](int s) {
         const int k = s * 16 + (lane >> 5) * 8;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int q = 0; q < NS; ++q)
-            ap[s % SETS][mt][q] = *reinterpret_cast<const v8bf*>(&src[q][mt * 32 + (lane & 31)][k]);
+            ap[s & 1][mt][q] = *reinterpret_cast<const v8bf*>(&src[q][mt * 32 + (lane & 31)][k]);
       };
-      if constexpr (NS == 1) {
-#pragma unroll
-        for (int s = 0; s < KS; ++s) read_ap(s);
-      } else {
-        read_ap(0);
-      }
+      read_ap(0);
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
-        if (NS > 1 && s + 1 < KS) read_ap(s + 1);
+        if (s + 1 < KS) read_ap(s + 1);
         if (drain) {
           if (s > 0) {
 #pragma unroll
@@ -698,10 +690,10 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
               if constexpr (F16)
-                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, ap[s % SETS][mt][i]),
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, ap[s & 1][mt][i]),
                                                                  __builtin_bit_cast(v8h, bw[order - i][s]), acc[mt], 0, 0, 0);
               else
-                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s % SETS][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ap[s & 1][mt][i], bw[order - i][s], acc[mt], 0, 0, 0);
             }
       }
       if constexpr (F16) {
@@ -788,7 +780,10 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 // -- one 16-byte load per k-step straight from W^T [R, N, K]; A rows are fetched
 // as 16-byte-per-lane segments (8 bf16) and go to LDS unchanged; the loads of the
 // next two tiles are in flight while the current one is multiplied.
-template <int KS>
+// AF32: A and W ([R, K, N]) are fp32 in memory and rounded to bf16 (nearest even) on their way
+// into the LDS and the registers -- the same result as rounding them beforehand, without the
+// conversion passes and the bf16 copies.
+template <int KS, bool AF32>
 __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(GemmArgs g, int G) {
   constexpr int KP = KS * 16 + 8;          // padded LDS row (bf16 elements)
   constexpr int LPR = KS * 2;              // lanes per A row, 8 bf16 each
@@ -819,7 +814,18 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
   v8bf bw[KS];
-  {
+  if constexpr (AF32) {
+    const float* W = reinterpret_cast<const float*>(g.w) + (int64_t)rel * K * N;
+    const int col = n0 + wave * 32 + (lane & 31);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = s * 16 + (lane >> 5) * 8 + j;
+        bw[s][j] = (__bf16)((k < K && col < N) ? W[(int64_t)k * N + col] : 0.f);
+      }
+    }
+  } else {
     const uint16_t* Wt = reinterpret_cast<const uint16_t*>(g.w) + (int64_t)rel * N * K;
     const int col = n0 + wave * 32 + (lane & 31);
 #pragma unroll
@@ -834,6 +840,8 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
   const int c8 = tid % LPR, rsub = tid / LPR;
   const bool k_ok = 8 * c8 < K;
   const uint16_t* A = reinterpret_cast<const uint16_t*>(g.a);
+  const float* Af = reinterpret_cast<const float*>(g.a);
+  constexpr int NREG = AF32 ? 2 * NLD : NLD;     // 16-byte registers per set: a row segment is 8 values
   auto load_maps = [&](int t) {
     if (tid < kBM && t < n_tiles) {
       const int64_t gr = row0 + (int64_t)t * kBM + tid;
@@ -847,18 +855,36 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
       s_dst[t % 3][tid] = didx;
     }
   };
-  auto gload = [&](uint4 (&areg)[NLD], int t) {
+  auto gload = [&](uint4 (&areg)[NREG], int t) {
     if (t >= n_tiles) return;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int64_t sidx = s_src[t % 3][i * RPI + rsub];
-      areg[i] = (sidx >= 0 && k_ok) ? *reinterpret_cast<const uint4*>(A + sidx * g.lda + 8 * c8)
-                                    : make_uint4(0u, 0u, 0u, 0u);
+      const bool ok = sidx >= 0 && k_ok;
+      if constexpr (AF32) {
+        const uint4* p = reinterpret_cast<const uint4*>(Af + sidx * g.lda + 8 * c8);
+        areg[2 * i] = ok ? p[0] : make_uint4(0u, 0u, 0u, 0u);
+        areg[2 * i + 1] = ok ? p[1] : make_uint4(0u, 0u, 0u, 0u);
+      } else {
+        areg[i] = ok ? *reinterpret_cast<const uint4*>(A + sidx * g.lda + 8 * c8) : make_uint4(0u, 0u, 0u, 0u);
+      }
     }
   };
-  auto tile_step = [&](uint4 (&areg)[NLD], int t) {
+  auto tile_step = [&](uint4 (&areg)[NREG], int t) {
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) *reinterpret_cast<uint4*>(&Ap[i * RPI + rsub][8 * c8]) = areg[i];
+    for (int i = 0; i < NLD; ++i) {
+      if constexpr (AF32) {
+        const uint4 lo = areg[2 * i], hi = areg[2 * i + 1];
+        const float f[8] = {__uint_as_float(lo.x), __uint_as_float(lo.y), __uint_as_float(lo.z), __uint_as_float(lo.w),
+                            __uint_as_float(hi.x), __uint_as_float(hi.y), __uint_as_float(hi.z), __uint_as_float(hi.w)};
+        v8bf r;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = (__bf16)f[j];
+        *reinterpret_cast<v8bf*>(&Ap[i * RPI + rsub][8 * c8]) = r;
+      } else {
+        *reinterpret_cast<uint4*>(&Ap[i * RPI + rsub][8 * c8]) = areg[i];
+      }
+    }
     load_maps(t + 2);
     __syncthreads();
     gload(areg, t + 2);
@@ -878,7 +904,7 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
     store_tile<128, 2>(g, acc, s_dst[t % 3], 0, wave, lane, n0);
     __syncthreads();
   };
-  uint4 areg0[NLD], areg1[NLD];
+  uint4 areg0[NREG], areg1[NREG];
   load_maps(0);
   load_maps(1);
   __syncthreads();
@@ -921,11 +947,24 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   cxg::GemmArgs g{a, lda, w, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
                   (int)(flags & 1u), (int)((flags >> 1) & 1u)};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if ((flags & CXG_GEMM_ROUND_BF16) && K <= 128 && (K & 7) == 0 && (lda & 7) == 0 && ((uintptr_t)a & 15) == 0) {
+    int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));
+    G = G < 1 ? 1 : (G > 32 ? 32 : G);
+    const int64_t n_chunks = cxg::ceil_div(cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R, cxg::kXcds) * cxg::kXcds;
+    const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
+    CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
+    const dim3 grid((unsigned)n_blocks), block(cxg::kThreads);
+    if (K <= 32) hipLaunchKernelGGL((cxg::typed_gemm_bf16_resident_kernel<2, true>), grid, block, 0, st, g, G);
+    else if (K <= 64) hipLaunchKernelGGL((cxg::typed_gemm_bf16_resident_kernel<4, true>), grid, block, 0, st, g, G);
+    else hipLaunchKernelGGL((cxg::typed_gemm_bf16_resident_kernel<8, true>), grid, block, 0, st, g, G);
+    CXG_LAUNCH_CHECK("typed_gemm_bf16_resident_kernel");
+    return CXG_OK;
+  }
   // Two fp16 parts of a 256-wide tile still fit the LDS: K up to 256 takes the fp16 form when the
   // 256 x 128 tile is mostly used (measured against the fp32 instructions at 7.3 M rows: K = 256,
   // N = 256 10.6 -> 5.8 ms, N = 128 5.3 -> 3.3 ms; K = 160, N = 64 2.0 -> 2.5 ms).
   const bool wide_k = (flags & CXG_GEMM_SPLIT_F16X3) && K > 128 && K <= 256 && K >= 176 && N >= 96;
-  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3 | CXG_GEMM_ROUND_BF16)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
+  if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
       (lda & 3) == 0 && ((uintptr_t)a & 15) == 0) {
     // 64*G rows per block: up to 32 tiles (16 with row maps, which the block keeps in LDS)
     // while the launch keeps a few thousand blocks
@@ -946,14 +985,12 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
 #define CXG_SPLIT(KS)                                                                          \
   do {                                                                                         \
     const bool half = (flags & CXG_GEMM_SPLIT_F16X3) != 0;                                     \
-    const int ns = (flags & CXG_GEMM_ROUND_BF16) ? 1 : (half || (flags & CXG_GEMM_SPLIT_BF16X3)) ? 2 : 3; \
+    const int ns = (half || (flags & CXG_GEMM_SPLIT_BF16X3)) ? 2 : 3;                          \
     const size_t lds = (size_t)2 * ns * cxg::kBM * (KS * 16 + 8) * sizeof(uint16_t) +          \
                        (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) + \
                        (KS <= 8 ? (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float) : 0) +       \
                        (size_t)2 * cxg::kBM * sizeof(float);                                   \
-    if (ns == 1 && mapped) CXG_SPLIT_LAUNCH(KS, 1, true, false);                               \
-    else if (ns == 1) CXG_SPLIT_LAUNCH(KS, 1, false, false);                                   \
-    else if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                              \
+    if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                                   \
     else if (half) CXG_SPLIT_LAUNCH(KS, 2, false, true);                                       \
     else if (ns == 2 && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, false);                          \
     else if (ns == 2) CXG_SPLIT_LAUNCH(KS, 2, false, false);                                   \
@@ -1005,9 +1042,9 @@ int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, flo
     const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
     CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
     const dim3 grid((unsigned)n_blocks), block(cxg::kThreads);
-    if (K <= 32) hipLaunchKernelGGL(cxg::typed_gemm_bf16_resident_kernel<2>, grid, block, 0, st, g, G);
-    else if (K <= 64) hipLaunchKernelGGL(cxg::typed_gemm_bf16_resident_kernel<4>, grid, block, 0, st, g, G);
-    else hipLaunchKernelGGL(cxg::typed_gemm_bf16_resident_kernel<8>, grid, block, 0, st, g, G);
+    if (K <= 32) hipLaunchKernelGGL((cxg::typed_gemm_bf16_resident_kernel<2, false>), grid, block, 0, st, g, G);
+    else if (K <= 64) hipLaunchKernelGGL((cxg::typed_gemm_bf16_resident_kernel<4, false>), grid, block, 0, st, g, G);
+    else hipLaunchKernelGGL((cxg::typed_gemm_bf16_resident_kernel<8, false>), grid, block, 0, st, g, G);
     CXG_LAUNCH_CHECK("typed_gemm_bf16_resident_kernel");
     return CXG_OK;
   }

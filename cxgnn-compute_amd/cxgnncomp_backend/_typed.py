@@ -98,7 +98,7 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
         flags |= _PRECISION_FLAGS[precision]
     stream = _lib.current_stream(a.device)
     with torch.cuda.device(a.device):
-        if bf16 and a.dtype == torch.float32 and K <= 128 and K % 4 == 0:
+        if bf16 and a.dtype == torch.float32 and K <= 128 and K % 8 == 0:
             # fp32 operands rounded to bf16 inside the kernel: no conversion pass over a and w
             _req(w, "weights", torch.float32, 3)
             st = lib.cxg_typed_gemm_f32(a.data_ptr(), K, w.data_ptr(), out.data_ptr(), N,

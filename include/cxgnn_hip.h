@@ -289,10 +289,11 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
  * instructions and two thirds of the LDS traffic of X6; this form also takes
  * 176 <= K <= 256 when N >= 96.  Rows or columns whose largest
  * magnitude is below 2^-112 count as zero; a row holding an infinity or NaN comes out
- * non-finite.  With CXG_GEMM_ROUND_BF16 (K <= 128) the fp32 operands are rounded to
- * bf16 (nearest even) on their way into the LDS and the registers and multiplied with
- * one bf16 MFMA per k-step: the result of cxg_typed_gemm_bf16 on the rounded operands
- * without a conversion pass.  Other shapes ignore these flags.  Replaces
+ * non-finite.  With CXG_GEMM_ROUND_BF16 (K <= 128, K and lda multiples of 8) the fp32
+ * operands are rounded to bf16 (nearest even) on their way into the LDS and the
+ * registers and multiplied with one bf16 MFMA per k-step: bit for bit the result of
+ * cxg_typed_gemm_bf16 on operands rounded beforehand, without the conversion passes.
+ * Other shapes ignore these flags.  Replaces
  * typed_matmul
  * (cxgnncomp/codegen/triton_typed_matmul.py:752-860: src_idx only = its
  * "single index" kernel with dst = src, seq_output = dst NULL, both = double
