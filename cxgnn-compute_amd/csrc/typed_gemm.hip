@@ -46,6 +46,10 @@ struct GemmArgs {
   int64_t M;
   int K, N, R;
   int accumulate, atomic;
+  // epilogue of the split kernel: C[d, n] = (A W)[., n] + bias[r, n] + addend[d, n] (either may be null)
+  const float* bias;
+  const float* addend;
+  int64_t ldd;
 };
 
 // Tile number -> (relation, first row, end of the relation's rows).  Every thread
@@ -71,7 +75,7 @@ __device__ __forceinline__ bool locate_tile(const int64_t* __restrict__ seg, int
 // four groups of four consecutive rows; the destination rows of a group are fetched from
 // LDS together (they are 32 contiguous bytes) and the four stores follow without waits.
 // MODE 0: store, 1: read-add-store, 2: fp32 atomic add.
-template <int BN, int MT, int MODE>
+template <int BN, int MT, int MODE, bool EPI = false>
 __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&acc)[MT],
                                                 const int64_t* s_dst, int wm, int wn, int lane, int n0) {
   const int col = n0 + wn * 32 + (lane & 31);
@@ -90,7 +94,8 @@ __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&
       for (int j = 0; j < 4; ++j) {
         if (d[j] < 0) continue;
         float* p = base + d[j] * ldc;
-        const float v = acc[mt][q * 4 + j];
+        float v = acc[mt][q * 4 + j];
+        if (EPI && g.addend) v += g.addend[d[j] * g.ldd + col];
         if (MODE == 2) unsafeAtomicAdd(p, v);
         else if (MODE == 1) *p += v;
         else *p = v;
@@ -99,12 +104,12 @@ __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&
   }
 }
 
-template <int BN, int MT>
+template <int BN, int MT, bool EPI = false>
 __device__ __forceinline__ void store_tile(const GemmArgs& g, const v16f (&acc)[MT],
                                            const int64_t* s_dst, int wm, int wn, int lane, int n0) {
-  if (g.atomic) store_tile_mode<BN, MT, 2>(g, acc, s_dst, wm, wn, lane, n0);
-  else if (g.accumulate) store_tile_mode<BN, MT, 1>(g, acc, s_dst, wm, wn, lane, n0);
-  else store_tile_mode<BN, MT, 0>(g, acc, s_dst, wm, wn, lane, n0);
+  if (g.atomic) store_tile_mode<BN, MT, 2, EPI>(g, acc, s_dst, wm, wn, lane, n0);
+  else if (g.accumulate) store_tile_mode<BN, MT, 1, EPI>(g, acc, s_dst, wm, wn, lane, n0);
+  else store_tile_mode<BN, MT, 0, EPI>(g, acc, s_dst, wm, wn, lane, n0);
 }
 
 __device__ __forceinline__ void load_row_maps(const GemmArgs& g, int64_t row0, int64_t row_end,
@@ -382,7 +387,9 @@ constexpr int kMappedTiles = 16;           // row maps given: a block keeps the 
 constexpr int kCP = 40;                    // floats per staged output row: 32 + pad; rows r and
                                            // r + 4 (the two halves of a wave) land 32 banks apart
 
-template <int KS, int NS, bool MAPPED, bool F16>
+// EPI: bias and addend of GemmArgs are honoured (a separate instantiation: the extra loads and
+// adds in the consumers' loop cost the plain form a tenth of its speed otherwise).
+template <int KS, int NS, bool MAPPED, bool F16, bool EPI = false>
 __global__ __launch_bounds__(kSplitThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void typed_gemm_split_kernel(GemmArgs g, int G) {
   static_assert(!F16 || NS == 2, "the fp16 form has two parts");
@@ -433,7 +440,8 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 
   // stores (or read-add-stores) of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
   const bool wide_store = KS <= 8 && !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
-                          ((uintptr_t)g.c & 15) == 0;
+                          ((uintptr_t)g.c & 15) == 0 &&
+                          (!EPI || !g.addend || ((g.ldd & 3) == 0 && ((uintptr_t)g.addend & 15) == 0));
 
   // ---- producer state -------------------------------------------------------------
   const int ptid = tid & 255;
@@ -634,16 +642,25 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
     };
     auto piece_row = [&](int it, int t) -> int64_t { return s_dst[t % SLOTS][it * 8 + (lane >> 3)]; };
     const bool add_old = g.accumulate != 0;
+    const bool add_row = EPI && g.addend != nullptr;
     auto piece_store = [&](const float4& v, int64_t d) {
       if (d < 0) return;
       float4* const p = reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wave * 32 + (lane & 7) * 4);
-      if (add_old) {
-        const float4 o = *p;
+      if (add_old || add_row) {
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (add_old) o = *p;
+        if (add_row) {
+          const float4 r = *reinterpret_cast<const float4*>(g.addend + d * g.ldd + n0 + wave * 32 + (lane & 7) * 4);
+          o = make_float4(o.x + r.x, o.y + r.y, o.z + r.z, o.w + r.w);
+        }
         *p = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
       } else {
         *p = v;
       }
     };
+    // this lane's accumulator column and its bias
+    const int col_own = n0 + wave * 32 + (lane & 31);
+    const float bias_own = (EPI && g.bias && col_own < N) ? g.bias[(int64_t)rel * N + col_own] : 0.f;
     for (int t = 0; t < n_tiles; ++t) {
       __syncthreads();
       const uint16_t (*src)[kBM][KP] = Ap[t & 1];
@@ -714,6 +731,12 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
         for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u]);
       }
+      if (EPI && g.bias) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mt][i] += bias_own;
+      }
       if (wide_store) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -721,7 +744,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
           for (int i = 0; i < 16; ++i)
             Cw[mt * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)][lane & 31] = acc[mt][i];
       } else {
-        store_tile<128, 2>(g, acc, s_dst[t % SLOTS], 0, wave, lane, n0);
+        store_tile<128, 2, EPI>(g, acc, s_dst[t % SLOTS], 0, wave, lane, n0);
       }
     }
     if (wide_store) {
@@ -938,16 +961,19 @@ int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64
 
 extern "C" {
 
-int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, int64_t ldc,
-                       const int64_t* src_idx, const int64_t* dst_idx, const int64_t* seg_ptr,
-                       int64_t M, int K, int N, int R, unsigned flags, void* stream) {
+static int typed_gemm_f32_impl(const float* a, int64_t lda, const float* w, const float* bias, const float* addend,
+                               int64_t ldd, float* c, int64_t ldc, const int64_t* src_idx, const int64_t* dst_idx,
+                               const int64_t* seg_ptr, int64_t M, int K, int N, int R, unsigned flags, void* stream) {
   int rc = cxg::check_args(a, w, c, seg_ptr, M, K, N, R, flags);
   if (rc || M == 0) return rc;
   CXG_REQUIRE(lda >= K && ldc >= N, CXG_ERR_ARG, "row stride smaller than row");
   cxg::GemmArgs g{a, lda, w, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
-                  (int)(flags & 1u), (int)((flags >> 1) & 1u)};
+                  (int)(flags & 1u), (int)((flags >> 1) & 1u), bias, addend, ldd};
+  const bool epilogue = bias || addend;
+  CXG_REQUIRE(!epilogue || ((flags & CXG_GEMM_SPLIT_F16X3) && !src_idx && !dst_idx), CXG_ERR_UNSUPPORTED,
+              "bias / addend are taken by the fp16 split form without row maps");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if ((flags & CXG_GEMM_ROUND_BF16) && K <= 128 && (K & 7) == 0 && (lda & 7) == 0 && ((uintptr_t)a & 15) == 0) {
+  if (!epilogue && (flags & CXG_GEMM_ROUND_BF16) && K <= 128 && (K & 7) == 0 && (lda & 7) == 0 && ((uintptr_t)a & 15) == 0) {
     int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));
     G = G < 1 ? 1 : (G > 32 ? 32 : G);
     const int64_t n_chunks = cxg::ceil_div(cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R, cxg::kXcds) * cxg::kXcds;
@@ -966,22 +992,27 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   const bool wide_k = (flags & CXG_GEMM_SPLIT_F16X3) && K > 128 && K <= 256 && K >= 176 && N >= 96;
   if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
       (lda & 3) == 0 && ((uintptr_t)a & 15) == 0) {
-    // 64*G rows per block: up to 32 tiles (16 with row maps, which the block keeps in LDS)
-    // while the launch keeps a few thousand blocks
+    // 64*G rows per block, up to 32 tiles (16 with row maps, which the block keeps in LDS).  A
+    // CU runs one block at a time and a block first loads and splits its weight slab, so few
+    // large blocks beat many small ones: the number of rounds of one block per CU that the
+    // largest blocks would need, then the block size that fills those rounds evenly.
     const bool mapped = src_idx || dst_idx;
     const int g_max = mapped ? cxg::kMappedTiles : 32;
-    int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));
+    const int64_t tiles = cxg::ceil_div(M, cxg::kBM) * cxg::ceil_div(N, 128);
+    const int64_t rounds = cxg::ceil_div(tiles, (int64_t)256 * g_max);
+    int G = (int)cxg::ceil_div(tiles, 256 * (rounds < 1 ? 1 : rounds));
     G = G < 1 ? 1 : (G > g_max ? g_max : G);
     const int64_t n_chunks = cxg::ceil_div(cxg::ceil_div(M, (int64_t)cxg::kBM * G) + R, cxg::kXcds) * cxg::kXcds;
     const int64_t n_blocks = n_chunks * cxg::ceil_div(N, 128);
     CXG_REQUIRE(n_blocks < (int64_t)1 << 31, CXG_ERR_UNSUPPORTED, "too many tiles for one launch");
     const dim3 grid((unsigned)n_blocks);
-#define CXG_SPLIT_LAUNCH(KS, NSV, MAP, HALF)                                                   \
+#define CXG_SPLIT_LAUNCH_E(KS, NSV, MAP, HALF, EPI)                                            \
   do {                                                                                         \
-    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_gemm_split_kernel<KS, NSV, MAP, HALF>, lds));      \
-    hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, NSV, MAP, HALF>), grid, dim3(cxg::kSplitThreads), lds, st, \
-                       g, G);                                                                  \
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_gemm_split_kernel<KS, NSV, MAP, HALF, EPI>, lds)); \
+    hipLaunchKernelGGL((cxg::typed_gemm_split_kernel<KS, NSV, MAP, HALF, EPI>), grid, dim3(cxg::kSplitThreads), lds, \
+                       st, g, G);                                                              \
   } while (0)
+#define CXG_SPLIT_LAUNCH(KS, NSV, MAP, HALF) CXG_SPLIT_LAUNCH_E(KS, NSV, MAP, HALF, false)
 #define CXG_SPLIT(KS)                                                                          \
   do {                                                                                         \
     const bool half = (flags & CXG_GEMM_SPLIT_F16X3) != 0;                                     \
@@ -990,7 +1021,8 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
                        (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) + \
                        (KS <= 8 ? (size_t)4 * cxg::kBM * cxg::kCP * sizeof(float) : 0) +       \
                        (size_t)2 * cxg::kBM * sizeof(float);                                   \
-    if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                                   \
+    if (epilogue) CXG_SPLIT_LAUNCH_E(KS, 2, false, true, true);                                \
+    else if (half && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, true);                              \
     else if (half) CXG_SPLIT_LAUNCH(KS, 2, false, true);                                       \
     else if (ns == 2 && mapped) CXG_SPLIT_LAUNCH(KS, 2, true, false);                          \
     else if (ns == 2) CXG_SPLIT_LAUNCH(KS, 2, false, false);                                   \
@@ -1004,14 +1036,18 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
       const size_t lds = (size_t)2 * 2 * cxg::kBM * (16 * 16 + 8) * sizeof(uint16_t) +
                          (size_t)2 * (mapped ? cxg::kMappedTiles : cxg::kMapSlots) * cxg::kBM * sizeof(int64_t) +
                          (size_t)2 * cxg::kBM * sizeof(float);
-      if (mapped) CXG_SPLIT_LAUNCH(16, 2, true, true);
+      if (epilogue) CXG_SPLIT_LAUNCH_E(16, 2, false, true, true);
+      else if (mapped) CXG_SPLIT_LAUNCH(16, 2, true, true);
       else CXG_SPLIT_LAUNCH(16, 2, false, true);
     }
 #undef CXG_SPLIT_LAUNCH
+#undef CXG_SPLIT_LAUNCH_E
 #undef CXG_SPLIT
     CXG_LAUNCH_CHECK("typed_gemm_split_kernel");
     return CXG_OK;
   }
+  CXG_REQUIRE(!epilogue, CXG_ERR_UNSUPPORTED,
+              "bias / addend need a split form and its shapes (K <= 128, or 176 <= K <= 256 with N >= 96 for the fp16 form)");
   const unsigned tiles = (unsigned)(cxg::ceil_div(M, cxg::kBM) + R);
   if (N > 64) {
     hipLaunchKernelGGL(cxg::typed_gemm_f32_kernel<128>, dim3(tiles, (unsigned)cxg::ceil_div(N, 128)),
@@ -1021,6 +1057,22 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, in
   }
   CXG_LAUNCH_CHECK("typed_gemm_f32_kernel");
   return CXG_OK;
+}
+
+int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c, int64_t ldc,
+                       const int64_t* src_idx, const int64_t* dst_idx, const int64_t* seg_ptr,
+                       int64_t M, int K, int N, int R, unsigned flags, void* stream) {
+  return typed_gemm_f32_impl(a, lda, w, nullptr, nullptr, 0, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R, flags,
+                             stream);
+}
+
+int cxg_typed_gemm_epilogue_f32(const float* a, int64_t lda, const float* w, const float* bias, const float* addend,
+                                int64_t ldd, float* c, int64_t ldc, const int64_t* src_idx, const int64_t* dst_idx,
+                                const int64_t* seg_ptr, int64_t M, int K, int N, int R, unsigned flags, void* stream) {
+  CXG_REQUIRE(!(flags & (CXG_GEMM_ATOMIC | CXG_GEMM_ACCUMULATE)), CXG_ERR_ARG,
+              "bias / addend do not go with accumulation into C (pass C as the addend instead)");
+  CXG_REQUIRE(!addend || ldd >= N, CXG_ERR_ARG, "addend row stride smaller than row");
+  return typed_gemm_f32_impl(a, lda, w, bias, addend, ldd, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R, flags, stream);
 }
 
 int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, float* c, int64_t ldc,

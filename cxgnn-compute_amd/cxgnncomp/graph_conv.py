@@ -321,6 +321,24 @@ def _weight_grad(x, g):
     return full[0].t() if full is not None else g2.t() @ x2      # shapes that kernel does not take
 
 
+def _mm(x, w_kn, bias=None, addend=None):
+    """x @ w_kn + bias + addend: the typed GEMM as one segment where it takes the shapes
+    (bias and addend go into its epilogue), the library GEMM otherwise."""
+    out = _typed.dense_linear(x, w_kn, bias, addend)
+    if out is not None:
+        return out
+    if addend is not None:
+        out = torch.addmm(addend, x, w_kn)
+        return out if bias is None else out.add_(bias)
+    return torch.addmm(bias, x, w_kn) if bias is not None else x @ w_kn
+
+
+def _mm_add_(out, x, w_kn):
+    """out += x @ w_kn in place (out may be a leading slice of a larger tensor)."""
+    if not _typed.dense_linear_add_(out, x, w_kn):
+        out.addmm_(x, w_kn)
+
+
 class SageLayerOP(torch.autograd.Function):
     """``MySageConv.forward`` on CUDA tensors as one autograd node: mean aggregation and
     ``lin_l`` in the cheaper order, plus the root term ``lin_r(x[:num_node])`` added by the
@@ -336,12 +354,14 @@ class SageLayerOP(torch.autograd.Function):
         mm_first = w_l.shape[1] > w_l.shape[0]
         aggr = None
         if mm_first:
-            out = _ops.spmm(ptr, idx, F.linear(x, w_l, b_l), n, mean=True)
+            out = _ops.spmm(ptr, idx, _mm(x, w_l.t(), b_l), n, mean=True)
+            if w_r is not None:
+                _mm_add_(out, x[:n], w_r.t())
         else:
             aggr = _ops.spmm(ptr, idx, x, n, mean=True)
-            out = F.linear(aggr, w_l, b_l)
-        if w_r is not None:
-            out.addmm_(x[:n], w_r.t())
+            out = _mm(aggr, w_l.t(), b_l)
+            if w_r is not None:
+                out = _mm(x[:n], w_r.t(), None, out)
         ctx.n, ctx.mm_first = n, mm_first
         ctx.save_for_backward(x, w_l, w_r, ptr, idx, aggr)
         return out
@@ -363,32 +383,35 @@ class SageLayerOP(torch.autograd.Function):
             if need_bl:
                 gb_l = _ops.column_sum(g_t)
             if need_x:
-                gx = g_t @ w_l
+                gx = _mm(g_t, w_l)
         else:
             if need_wl:
                 gw_l = _weight_grad(aggr, g)
             if need_bl:
                 gb_l = _ops.column_sum(g)
             if need_x:
-                gx = _ops.spmm(tg.ptr_t, tg.idx_t, g @ w_l, n_src, val=inv)
+                gx = _ops.spmm(tg.ptr_t, tg.idx_t, _mm(g, w_l), n_src, val=inv)
         if w_r is not None:
             if need_wr:
                 gw_r = _weight_grad(x[:n], g)
             if need_x:
-                gx[:n].addmm_(g, w_r)
+                _mm_add_(gx[:n], g, w_r)
         return gx, gw_l, gb_l, gw_r, None, None, None
 
 
 class LinearOP(torch.autograd.Function):
-    """``F.linear(x, weight, bias) (+ addend)`` whose weight gradient g^T x, a product with
-    one very long reduction axis (every node) and a small output, runs on the typed
-    weight-gradient kernel as a single segment; the library GEMM serves the forward pass
-    (bias and addend go into its epilogue instead of separate element-wise passes), the
-    input gradient and the shapes that kernel does not take."""
+    """``F.linear(x, weight, bias) (+ addend)`` on the typed kernels as a single segment: the
+    forward product and the input gradient on the split GEMM (bias and addend go into its
+    epilogue instead of separate element-wise passes), the weight gradient g^T x -- one very
+    long reduction axis (every node), a small output -- on the weight-gradient kernel.  The
+    library GEMM serves the shapes those kernels do not take (few rows, wide K)."""
 
     @staticmethod
     def forward(ctx, x, weight, bias=None, addend=None):
         ctx.save_for_backward(x, weight)
+        out = _typed.dense_linear(x, weight.t(), bias, addend)
+        if out is not None:
+            return out
         if addend is None:
             return F.linear(x, weight, bias)
         out = torch.addmm(addend, x, weight.t())
@@ -399,12 +422,15 @@ class LinearOP(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         gx = gw = gb = None
         if ctx.needs_input_grad[0]:
-            gx = g @ weight
+            gx = _typed.dense_linear(g, weight) if g.dim() == 2 else None
+            if gx is None:
+                gx = g @ weight
         if ctx.needs_input_grad[1]:
             gw = _weight_grad(x, g)
         if ctx.needs_input_grad[2]:
             gb = _ops.column_sum(g.reshape(-1, g.shape[-1]).contiguous())
-        return gx, gw, gb, (g if ctx.needs_input_grad[3] else None)
+        grads = (gx, gw, gb, g)              # bias and addend are optional arguments of apply()
+        return tuple(grads[i] if need else None for i, need in enumerate(ctx.needs_input_grad))
 
 
 def linear(x, weight, bias=None, addend=None):
@@ -456,7 +482,7 @@ class GatLayerOP(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w, att_src, att_dst, bias, ptr, idx, num_dst, num_src, num_edge, slope, heads, concat):
         H, C = heads, w.shape[0] // heads
-        xs = F.linear(x[:num_src], w).view(-1, H, C)
+        xs = _mm(x[:num_src], w.t()).view(-1, H, C)
         a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
         ev, mask = _ops.edge_softmax_fwd(ptr, idx, a_dst, a_src, num_edge, slope)
         if concat:
@@ -496,7 +522,7 @@ class GatLayerOP(torch.autograd.Function):
         g_xs2 = g_xs.view(-1, H * C)
         g_x = g_w = None
         if ctx.needs_input_grad[0]:
-            g_x = g_xs2 @ w
+            g_x = _mm(g_xs2, w)
             if g_x.shape[0] < x.shape[0]:
                 g_x = torch.cat([g_x, g_x.new_zeros(x.shape[0] - g_x.shape[0], g_x.shape[1])])
         if ctx.needs_input_grad[1]:

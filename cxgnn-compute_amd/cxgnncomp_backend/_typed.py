@@ -120,6 +120,75 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
 
 
 # --------------------------------------------------------------------------- #
+# dense x @ W (+ bias) (+ addend) as a typed GEMM with one relation
+# --------------------------------------------------------------------------- #
+DENSE_MIN_ROWS = 4096        # below this the launch is latency bound either way
+DENSE_WIDE_MIN_ROWS = 100000
+_one_seg = {}
+
+
+def _one_segment(m_rows, device):
+    key = (int(m_rows), str(device))
+    seg = _one_seg.get(key)
+    if seg is None:
+        if len(_one_seg) > 64:
+            _one_seg.clear()
+        seg = _one_seg[key] = torch.tensor([0, int(m_rows)], dtype=torch.int64, device=device)
+    return seg
+
+
+def dense_linear(x, w_kn, bias=None, addend=None):
+    """x [M, K] @ w_kn [K, N] + bias [N] + addend [M, N] (either may be None) as a typed GEMM over
+    one segment, bias and addend added to the accumulator before the rows are stored.  Returns
+    None for inputs the split kernels do not take (the caller then uses the library GEMM):
+    other dtypes or layouts, few rows, K above 128 (256 when K >= 176, N >= 96, at least 10^5
+    rows and no addend), K not a multiple of 4, a default precision other than the fp16 split
+    form."""
+    flags = _PRECISION_FLAGS.get(GEMM_PRECISION, 0)
+    if flags != GEMM_SPLIT_F16X3 or not x.is_cuda or x.dim() != 2 or x.dtype != torch.float32 or w_kn.dtype != torch.float32:
+        return None
+    M, K = x.shape
+    N = w_kn.shape[1]
+    # the 256-wide form stores from the accumulators (no staged 16-byte stores): it beats the
+    # library from about 10^5 rows on and not with an addend (measured on 4 k - 2.4 M rows)
+    wide = 176 <= K <= 256 and N >= 96 and addend is None and M >= DENSE_WIDE_MIN_ROWS
+    if M < DENSE_MIN_ROWS or K % 4 or not (K <= 128 or wide) or w_kn.shape[0] != K:
+        return None
+    if not x.is_contiguous() or x.data_ptr() % 16:
+        return None
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
+        return None
+    if addend is not None and (addend.dtype != torch.float32 or tuple(addend.shape) != (M, N)
+                               or not addend.is_contiguous()):
+        return None
+    lib = _lib.load()
+    w_kn = w_kn.contiguous()
+    out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_typed_gemm_epilogue_f32(x.data_ptr(), K, w_kn.data_ptr(), _lib.ptr(bias), _lib.ptr(addend), N,
+                                             out.data_ptr(), N, None, None, _one_segment(M, x.device).data_ptr(),
+                                             M, K, N, 1, flags, _lib.current_stream(x.device))
+    _lib.check(st)
+    return out
+
+
+def dense_linear_add_(out, x, w_kn):
+    """out [M, N] += x [M, K] @ w_kn [K, N] in place through the typed GEMM (one segment);
+    False when the shapes are not taken (nothing is written then)."""
+    if (GEMM_PRECISION != "split_f16" or not x.is_cuda or x.dim() != 2 or x.dtype != torch.float32
+            or out.dtype != torch.float32 or w_kn.dtype != torch.float32):
+        return False
+    M, K = x.shape
+    N = w_kn.shape[1]
+    if (M < DENSE_MIN_ROWS or K % 4 or K > 128 or tuple(out.shape) != (M, N)
+            or not x.is_contiguous() or not out.is_contiguous() or x.data_ptr() % 16):
+        return False
+    typed_gemm(x, w_kn.contiguous().unsqueeze(0), _one_segment(M, x.device), M, out=out, accumulate=True,
+               precision="split_f16")
+    return True
+
+
+# --------------------------------------------------------------------------- #
 # pad_rel / pad_rel_idx  (binding.cpp:51-52)
 # --------------------------------------------------------------------------- #
 def _pad_rel(rel, idx, count, thres, num_rel, base):

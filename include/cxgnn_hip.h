@@ -306,6 +306,22 @@ int cxg_typed_gemm_f32(const float* a, int64_t lda, const float* w, float* c,
                        const int64_t* seg_ptr, int64_t M, int K, int N, int R,
                        unsigned flags, void* stream);
 
+/*
+ * cxg_typed_gemm_f32 with an epilogue: C[dst(i), :] = A[src(i), :] @ W[r] + bias[r, :] +
+ * addend[dst(i), :] (bias [R, N] and addend [*, N] with row stride ldd; either may be
+ * NULL), added to the accumulator before the row is stored, so neither costs a pass over
+ * C.  Taken by the fp16 split form only (CXG_GEMM_SPLIT_F16X3 and its shapes, no row maps;
+ * otherwise CXG_ERR_UNSUPPORTED), not with CXG_GEMM_ACCUMULATE or CXG_GEMM_ATOMIC (the
+ * addend may be C itself: a row is read before it is written).  With R = 1 and seg_ptr =
+ * {0, M} this is F.linear(x, W^T, bias) (+ addend), which is what the layers of the
+ * reference's models call (cxgnncomp/graph_conv.py:132-178 lin_l / lin_r / linear).
+ */
+int cxg_typed_gemm_epilogue_f32(const float* a, int64_t lda, const float* w, const float* bias,
+                                const float* addend, int64_t ldd, float* c, int64_t ldc,
+                                const int64_t* src_idx, const int64_t* dst_idx,
+                                const int64_t* seg_ptr, int64_t M, int K, int N, int R,
+                                unsigned flags, void* stream);
+
 /* Same contraction with bf16 operands on v_mfma_f32_32x32x16_bf16: A is bf16
  * [*, K], w_t is the transposed weight stack W^T as bf16 [R, N, K]; C stays fp32.
  * K and lda must be multiples of 8. */

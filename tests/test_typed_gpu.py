@@ -358,3 +358,134 @@ def test_typed_gemm_small_shapes_and_skipped_rows(M, K, N):
             want_gw[types[i]] += torch.outer(a[src[i]].double(), g[dst[i]].double())
     scale = max(1.0, float(want_gw.abs().max()))
     assert_close(_np(gw) / scale, want_gw.numpy() / scale, RTOL, 2 * ATOL, "wgrad with skipped rows")
+
+
+@pytest.mark.parametrize("M,K,N,R", [(5000, 128, 128, 1), (4097, 64, 200, 1), (9000, 36, 72, 3), (70, 128, 256, 2),
+                                     (120000, 256, 128, 1), (6000, 200, 96, 2)])
+@pytest.mark.parametrize("with_bias,with_addend", [(True, False), (False, True), (True, True)])
+def test_typed_gemm_epilogue_bias_and_addend(M, K, N, R, with_bias, with_addend, gemm_precision):
+    """cxg_typed_gemm_epilogue_f32 through the C ABI: per-relation bias rows and an addend with
+    a row stride wider than N are added before the store; against float64, and against the
+    plain entry point followed by the two additions (same products, so the same bits up to the
+    order of the last two additions)."""
+    from cxgnncomp_backend import _lib, _typed
+    if gemm_precision != "split_f16":
+        pytest.skip("the entry point takes its form from its flags: runs once")
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(M + K + N + R)
+    a = (torch.randn(M, K, generator=gen) / K ** 0.5).cuda()
+    w = torch.randn(R, K, N, generator=gen).cuda()
+    cuts = torch.sort(torch.randint(0, M + 1, (R - 1,), generator=gen))[0]
+    seg = torch.cat([torch.zeros(1, dtype=torch.int64), cuts, torch.tensor([M])]).cuda()
+    bias = torch.randn(R, N, generator=gen).cuda() if with_bias else None
+    ldd = N + 12
+    addend_buf = torch.randn(M, ldd, generator=gen).cuda() if with_addend else None
+    out = torch.full((M, N), 7.0).cuda()
+    announce("typed_gemm_epilogue M=%d K=%d N=%d R=%d bias=%s addend=%s" % (M, K, N, R, with_bias, with_addend))
+    st = lib.cxg_typed_gemm_epilogue_f32(a.data_ptr(), K, w.data_ptr(), _lib.ptr(bias), _lib.ptr(addend_buf), ldd,
+                                         out.data_ptr(), N, None, None, seg.data_ptr(), M, K, N, R,
+                                         _typed.GEMM_SPLIT_F16X3, _lib.current_stream(a.device))
+    _lib.check(st)
+    torch.cuda.synchronize()
+    seg_h = seg.cpu().tolist()
+    want = torch.empty(M, N, dtype=torch.float64)
+    for r in range(R):
+        lo, hi = seg_h[r], seg_h[r + 1]
+        want[lo:hi] = a[lo:hi].double().cpu() @ w[r].double().cpu()
+        if with_bias:
+            want[lo:hi] += bias[r].double().cpu()
+    if with_addend:
+        want += addend_buf[:, :N].double().cpu()
+    assert_close(_np(out), want.numpy(), RTOL, 2 * ATOL, "typed_gemm_epilogue")
+    plain = _typed.typed_gemm(a, w, seg, M, precision="split_f16")
+    if with_bias:
+        plain = plain + bias[torch.bucketize(torch.arange(M, device="cuda"), seg[1:], right=True)]
+    if with_addend:
+        plain = plain + addend_buf[:, :N]
+    assert float((plain - out).abs().max()) <= 4e-6 * float(want.abs().max())
+
+
+def test_typed_gemm_epilogue_rejects_what_it_does_not_take(gemm_precision):
+    """Row maps, the atomic flag, precisions other than the fp16 split and a short addend stride
+    are refused with an error code and nothing is written."""
+    from cxgnncomp_backend import _lib, _typed
+    lib = _lib.load()
+    M, K, N = 256, 64, 64
+    a = torch.randn(M, K).cuda()
+    w = torch.randn(1, K, N).cuda()
+    seg = torch.tensor([0, M], dtype=torch.int64).cuda()
+    idx = torch.arange(M, dtype=torch.int64).cuda()
+    bias = torch.randn(1, N).cuda()
+    out = torch.full((M, N), 7.0).cuda()
+
+    def call(flags, src=None, dst=None, addend=None, ldd=N):
+        return lib.cxg_typed_gemm_epilogue_f32(a.data_ptr(), K, w.data_ptr(), bias.data_ptr(), _lib.ptr(addend), ldd,
+                                               out.data_ptr(), N, _lib.ptr(src), _lib.ptr(dst), seg.data_ptr(),
+                                               M, K, N, 1, flags, _lib.current_stream(a.device))
+    if gemm_precision != "fp32":
+        pytest.skip("independent of the default precision: runs once")
+    announce("typed_gemm_epilogue argument checks")
+    assert call(_typed.GEMM_SPLIT_F16X3, src=idx) != 0
+    assert call(_typed.GEMM_SPLIT_F16X3, dst=idx) != 0
+    assert call(0) != 0
+    assert call(_typed.GEMM_SPLIT_F16X3 | 1) != 0
+    assert call(_typed.GEMM_SPLIT_F16X3 | 2) != 0
+    assert call(_typed.GEMM_SPLIT_F16X3, addend=out, ldd=N - 4) != 0
+    torch.cuda.synchronize()
+    assert bool((out == 7.0).all())
+    assert call(_typed.GEMM_SPLIT_F16X3) == 0
+
+
+@pytest.mark.parametrize("M,K,N", [(5000, 128, 256), (4096, 100, 64), (130000, 256, 256)])
+def test_dense_linear_helpers_match_library(M, K, N):
+    """dense_linear / dense_linear_add_ (what LinearOP, SageLayerOP and GatLayerOP call) against
+    float64 F.linear; shapes they do not take return None / False and write nothing."""
+    from cxgnncomp_backend import _typed
+    gen = torch.Generator().manual_seed(M + K)
+    x = (torch.randn(M, K, generator=gen) / K ** 0.5).cuda()
+    w = torch.randn(N, K, generator=gen).cuda()                    # nn.Linear layout [out, in]
+    b = torch.randn(N, generator=gen).cuda()
+    add = torch.randn(M, N, generator=gen).cuda()
+    announce("dense_linear M=%d K=%d N=%d" % (M, K, N))
+    want = x.double() @ w.double().t() + b.double()
+    got = _typed.dense_linear(x, w.t(), b)
+    if _typed.GEMM_PRECISION != "split_f16":             # only the default form has the epilogue
+        assert got is None and not _typed.dense_linear_add_(add.clone(), x, w.t())
+        return
+    assert got is not None
+    assert_close(_np(got), _np(want), RTOL, 2 * ATOL, "dense_linear bias")
+    if K <= 128:
+        got = _typed.dense_linear(x, w.t(), b, add)
+        assert_close(_np(got), _np(want + add.double()), RTOL, 2 * ATOL, "dense_linear bias addend")
+        acc = add.clone()
+        assert _typed.dense_linear_add_(acc, x, w.t())
+        assert_close(_np(acc), _np(want - b.double() + add.double()), RTOL, 2 * ATOL, "dense_linear_add_")
+    else:
+        assert _typed.dense_linear(x, w.t(), b, add) is None
+        acc = add.clone()
+        assert not _typed.dense_linear_add_(acc, x, w.t())
+        assert torch.equal(acc, add)
+    assert _typed.dense_linear(x[:100], w.t(), b) is None
+    assert _typed.dense_linear(x.double(), w.t().double(), b.double()) is None
+
+
+def test_linear_op_gradients_through_typed_gemm():
+    """LinearOP on a shape dense_linear takes: output and the three gradients against float64
+    autograd of F.linear."""
+    from cxgnncomp.graph_conv import LinearOP
+    gen = torch.Generator().manual_seed(5)
+    M, K, N = 6000, 128, 64
+    x = (torch.randn(M, K, generator=gen) / K ** 0.5).cuda().requires_grad_()
+    w = torch.randn(N, K, generator=gen).cuda().requires_grad_()
+    b = torch.randn(N, generator=gen).cuda().requires_grad_()
+    g = torch.randn(M, N, generator=gen).cuda()
+    announce("LinearOP fwd+bwd M=%d K=%d N=%d" % (M, K, N))
+    y = LinearOP.apply(x, w, b)
+    y.backward(g)
+    xd, wd, bd = (t.detach().double().requires_grad_() for t in (x, w, b))
+    yd = torch.nn.functional.linear(xd, wd, bd)
+    yd.backward(g.double())
+    assert_close(_np(y), _np(yd), RTOL, 2 * ATOL, "LinearOP forward")
+    for name, got, want in (("x", x.grad, xd.grad), ("w", w.grad, wd.grad), ("b", b.grad, bd.grad)):
+        scale = max(1.0, float(want.abs().max()))
+        assert_close(_np(got) / scale, _np(want) / scale, RTOL, 2 * ATOL, "LinearOP grad " + name)
