@@ -420,13 +420,19 @@ __global__ __launch_bounds__(64 * kReduceSlices) void wgrad_reduce_kernel(
   }
 }
 
+// Rows per chunk.  A CU runs one block (chunk x column tile) at a time and every block ends
+// with a K x 128 partial that the reduction reads again, so few long chunks beat many short
+// ones: the number of rounds of one block per CU that the longest chunks would need, then
+// the chunk length that fills those rounds evenly.
 int64_t chunk_rows(int64_t M, int N, bool mapped) {
-  int64_t rows = M * ceil_div(N, 128) / 4096;
-  rows = (rows + kMT - 1) / kMT * kMT;
-  const int64_t most = mapped ? kMappedRows : 256 * kMT;
-  if (rows < 8 * kMT) rows = 8 * kMT;
-  if (rows > most) rows = most;
-  return rows;
+  const int64_t g_max = (mapped ? kMappedRows : 256 * kMT) / kMT;
+  const int64_t tiles = ceil_div(M, (int64_t)kMT) * ceil_div(N, 128);
+  int64_t rounds = ceil_div(tiles, 256 * g_max);
+  if (rounds < 1) rounds = 1;
+  int64_t g = ceil_div(tiles, 256 * rounds);
+  if (g < 8) g = 8;
+  if (g > g_max) g = g_max;
+  return g * kMT;
 }
 
 }  // namespace
