@@ -75,41 +75,84 @@ __device__ __forceinline__ bool locate_tile(const int64_t* __restrict__ seg, int
 // four groups of four consecutive rows; the destination rows of a group are fetched from
 // LDS together (they are 32 contiguous bytes) and the four stores follow without waits.
 // MODE 0: store, 1: read-add-store, 2: fp32 atomic add.
-template <int BN, int MT, int MODE, bool EPI = false>
+template <int BN, int MT, int MODE, bool EPI = false, int QB = 1>
 __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&acc)[MT],
                                                 const int64_t* s_dst, int wm, int wn, int lane, int n0) {
   const int col = n0 + wn * 32 + (lane & 31);
   if (col >= g.N) return;
   float* const base = g.c + col;
   const int64_t ldc = g.ldc;
+  if constexpr (MODE != 1 && !EPI) {
+    // nothing is read: the rows of a group of four as soon as their indices are there
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int rl0 = (wm * MT + mt) * 32 + q * 8 + (lane >> 5) * 4;
+        int64_t d[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) d[j] = s_dst[rl0 + j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (d[j] < 0) continue;
+          float* p = base + d[j] * ldc;
+          if (MODE == 2) unsafeAtomicAdd(p, acc[mt][q * 4 + j]);
+          else *p = acc[mt][q * 4 + j];
+        }
+      }
+    }
+    return;
+  }
+  // What the rows are added to (the old row when accumulating, the addend) is requested for
+  // 4 * QB rows before their first store: a read-add-store per element in turn is one trip
+  // to memory after the other, since a store may alias the next load.
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int rl0 = (wm * MT + mt) * 32 + q * 8 + (lane >> 5) * 4;
-      int64_t d[4];
+    for (int q0 = 0; q0 < 4; q0 += QB) {
+      constexpr int NR = 4 * QB;
+      int64_t d[NR];
+      float v[NR];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) d[j] = s_dst[rl0 + j];
+      for (int q = 0; q < QB; ++q) {
+        const int rl0 = (wm * MT + mt) * 32 + (q0 + q) * 8 + (lane >> 5) * 4;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (d[j] < 0) continue;
-        float* p = base + d[j] * ldc;
-        float v = acc[mt][q * 4 + j];
-        if (EPI && g.addend) v += g.addend[d[j] * g.ldd + col];
-        if (MODE == 2) unsafeAtomicAdd(p, v);
-        else if (MODE == 1) *p += v;
-        else *p = v;
+        for (int j = 0; j < 4; ++j) {
+          d[q * 4 + j] = s_dst[rl0 + j];
+          v[q * 4 + j] = acc[mt][(q0 + q) * 4 + j];
+        }
+      }
+      if (MODE == 1) {
+        float o[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) o[i] = d[i] >= 0 ? base[d[i] * ldc] : 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) v[i] += o[i];
+      }
+      if (EPI && g.addend) {
+        float o[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) o[i] = d[i] >= 0 ? g.addend[d[i] * g.ldd + col] : 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) v[i] += o[i];
+      }
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        if (d[i] < 0) continue;
+        float* p = base + d[i] * ldc;
+        if (MODE == 2) unsafeAtomicAdd(p, v[i]);
+        else *p = v[i];
       }
     }
   }
 }
 
-template <int BN, int MT, bool EPI = false>
+template <int BN, int MT, bool EPI = false, int QB = 1>
 __device__ __forceinline__ void store_tile(const GemmArgs& g, const v16f (&acc)[MT],
                                            const int64_t* s_dst, int wm, int wn, int lane, int n0) {
-  if (g.atomic) store_tile_mode<BN, MT, 2, EPI>(g, acc, s_dst, wm, wn, lane, n0);
-  else if (g.accumulate) store_tile_mode<BN, MT, 1, EPI>(g, acc, s_dst, wm, wn, lane, n0);
-  else store_tile_mode<BN, MT, 0, EPI>(g, acc, s_dst, wm, wn, lane, n0);
+  if (g.atomic) store_tile_mode<BN, MT, 2, EPI, QB>(g, acc, s_dst, wm, wn, lane, n0);
+  else if (g.accumulate) store_tile_mode<BN, MT, 1, EPI, QB>(g, acc, s_dst, wm, wn, lane, n0);
+  else store_tile_mode<BN, MT, 0, EPI, QB>(g, acc, s_dst, wm, wn, lane, n0);
 }
 
 __device__ __forceinline__ void load_row_maps(const GemmArgs& g, int64_t row0, int64_t row_end,
@@ -744,7 +787,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
           for (int i = 0; i < 16; ++i)
             Cw[mt * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)][lane & 31] = acc[mt][i];
       } else {
-        store_tile<128, 2, EPI>(g, acc, s_dst[t % SLOTS], 0, wave, lane, n0);
+        store_tile<128, 2, EPI, 4>(g, acc, s_dst[t % SLOTS], 0, wave, lane, n0);
       }
     }
     if (wide_store) {

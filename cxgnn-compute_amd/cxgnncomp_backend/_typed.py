@@ -141,17 +141,16 @@ def dense_linear(x, w_kn, bias=None, addend=None):
     """x [M, K] @ w_kn [K, N] + bias [N] + addend [M, N] (either may be None) as a typed GEMM over
     one segment, bias and addend added to the accumulator before the rows are stored.  Returns
     None for inputs the split kernels do not take (the caller then uses the library GEMM):
-    other dtypes or layouts, few rows, K above 128 (256 when K >= 176, N >= 96, at least 10^5
-    rows and no addend), K not a multiple of 4, a default precision other than the fp16 split
-    form."""
+    other dtypes or layouts, few rows, K above 128 (256 when K >= 176, N >= 96 and at least
+    10^5 rows), K not a multiple of 4, a default precision other than the fp16 split form."""
     flags = _PRECISION_FLAGS.get(GEMM_PRECISION, 0)
     if flags != GEMM_SPLIT_F16X3 or not x.is_cuda or x.dim() != 2 or x.dtype != torch.float32 or w_kn.dtype != torch.float32:
         return None
     M, K = x.shape
     N = w_kn.shape[1]
     # the 256-wide form stores from the accumulators (no staged 16-byte stores): it beats the
-    # library from about 10^5 rows on and not with an addend (measured on 4 k - 2.4 M rows)
-    wide = 176 <= K <= 256 and N >= 96 and addend is None and M >= DENSE_WIDE_MIN_ROWS
+    # library from about 10^5 rows on (measured on 4 k - 2.4 M rows, with and without addend)
+    wide = 176 <= K <= 256 and N >= 96 and M >= DENSE_WIDE_MIN_ROWS
     if M < DENSE_MIN_ROWS or K % 4 or not (K <= 128 or wide) or w_kn.shape[0] != K:
         return None
     if not x.is_contiguous() or x.data_ptr() % 16:

@@ -454,14 +454,13 @@ def test_dense_linear_helpers_match_library(M, K, N):
         return
     assert got is not None
     assert_close(_np(got), _np(want), RTOL, 2 * ATOL, "dense_linear bias")
+    got = _typed.dense_linear(x, w.t(), b, add)
+    assert_close(_np(got), _np(want + add.double()), RTOL, 2 * ATOL, "dense_linear bias addend")
     if K <= 128:
-        got = _typed.dense_linear(x, w.t(), b, add)
-        assert_close(_np(got), _np(want + add.double()), RTOL, 2 * ATOL, "dense_linear bias addend")
         acc = add.clone()
         assert _typed.dense_linear_add_(acc, x, w.t())
         assert_close(_np(acc), _np(want - b.double() + add.double()), RTOL, 2 * ATOL, "dense_linear_add_")
     else:
-        assert _typed.dense_linear(x, w.t(), b, add) is None
         acc = add.clone()
         assert not _typed.dense_linear_add_(acc, x, w.t())
         assert torch.equal(acc, add)
