@@ -327,14 +327,19 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     """gw[r] = sum over the rows i of segment r of a[src(i)]^T (x) g[dst(i)] -> [num_rel, K, N]
     (see cxg_typed_gemm_wgrad_f32).  One launch takes K <= 128; a wider K runs as one launch per
     128 columns of ``a`` (a single relation writes its rows of gw in place, several relations go
-    through a [num_rel, 128, N] buffer per slice).  Returns None for shapes the kernel does not
-    take (K or N not multiples of 4)."""
+    through a [num_rel, 128, N] buffer per slice).  An N that is not a multiple of 4 (a class
+    count, say) runs on a copy of g padded with zero columns.  Returns None when K is not a
+    multiple of 4, which the kernel does not take."""
     lib = _lib.load()
     _req(a, "a", torch.float32, 2)
     _req(g, "g", torch.float32, 2)
     K, N = a.shape[1], g.shape[1]
-    if K % 4 or N % 4:
+    if K % 4:
         return None
+    if N % 4:
+        gw = typed_gemm_wgrad(a, torch.nn.functional.pad(g, (0, -N % 4)), seg_ptr, m_rows, num_rel,
+                              src_idx=src_idx, dst_idx=dst_idx, precision=precision)
+        return gw[:, :, :N].contiguous()
     precision = precision or GEMM_PRECISION
     flags = (GEMM_SPLIT_F16X3 if precision == "split_f16" else
              GEMM_SPLIT_BF16X3 if precision in ("split3", "bf16") else GEMM_SPLIT_BF16X6)

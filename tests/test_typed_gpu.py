@@ -216,12 +216,13 @@ def test_rgcn_fused_forward_backward(K, N, R, strategy, monkeypatch):
 
 
 @pytest.mark.parametrize("K,N,R,M", [(128, 128, 16, 5000), (64, 48, 3, 1000), (4, 256, 1, 3000), (128, 2048, 1, 700),
-                                     (32, 40, 4, 70000), (12, 20, 5, 1), (256, 128, 5, 3000), (200, 64, 1, 900)])
+                                     (32, 40, 4, 70000), (12, 20, 5, 1), (256, 128, 5, 3000), (200, 64, 1, 900),
+                                     (256, 47, 1, 1024), (64, 5, 3, 2000)])
 def test_typed_gemm_wgrad(K, N, R, M):
     """gw[r] = sum over the rows of relation r of a[src]^T (x) g[dst], against per-relation
     float64 products; covers several column tiles (N = 2048), K far below one tile (K = 4),
-    K above one launch's 128 (in slices, one and several relations), many row chunks (M = 70000)
-    and relations without rows."""
+    K above one launch's 128 (in slices, one and several relations), many row chunks (M = 70000),
+    N that is not a multiple of 4 (padded copy of g) and relations without rows."""
     from cxgnncomp_backend import _typed
     gen = torch.Generator().manual_seed(K + N + M)
     n_a, n_g = max(1, M // 2), max(1, M // 3)
