@@ -20,6 +20,8 @@
 // (cxgnncomp/codegen/triton_typed_matmul.py:146-215,364-430,529-592,691-749;
 // launcher :752-860) and, through the host wrappers, the per-row CUDA kernels
 // typed_linear_kernel / _s2e / _s2d (src/cpp/src/rel_spmm.cu:231-358).
+#include <type_traits>
+
 #include "cxg_common.hpp"
 
 namespace cxg {
@@ -482,9 +484,11 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
   // stores (or read-add-stores) of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
-  const bool wide_store = KS <= 8 && !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
-                          ((uintptr_t)g.c & 15) == 0 &&
-                          (!EPI || !g.addend || ((g.ldd & 3) == 0 && ((uintptr_t)g.addend & 15) == 0));
+  // (not with an addend: those rows leave from the accumulators, see store_tile_mode -- measured
+  // faster, 7.3 M x 128 x 128 3.52 -> 2.37 ms, while accumulation into C is faster this way, 3.08
+  // against 3.47 ms)
+  const bool wide_store = KS <= 8 && !g.atomic && !(EPI && g.addend) && n0 + wave * 32 + 32 <= N &&
+                          (g.ldc & 3) == 0 && ((uintptr_t)g.c & 15) == 0;
 
   // ---- producer state -------------------------------------------------------------
   const int ptid = tid & 255;
@@ -684,18 +688,11 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       return *reinterpret_cast<const float4*>(&Cw[it * 8 + (lane >> 3)][(lane & 7) * 4]);
     };
     auto piece_row = [&](int it, int t) -> int64_t { return s_dst[t % SLOTS][it * 8 + (lane >> 3)]; };
-    const bool add_old = g.accumulate != 0;
-    const bool add_row = EPI && g.addend != nullptr;
-    auto piece_store = [&](const float4& v, int64_t d) {
+    auto piece_store = [&](const float4& v, int64_t d, auto add_tag) {
       if (d < 0) return;
       float4* const p = reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wave * 32 + (lane & 7) * 4);
-      if (add_old || add_row) {
-        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (add_old) o = *p;
-        if (add_row) {
-          const float4 r = *reinterpret_cast<const float4*>(g.addend + d * g.ldd + n0 + wave * 32 + (lane & 7) * 4);
-          o = make_float4(o.x + r.x, o.y + r.y, o.z + r.z, o.w + r.w);
-        }
+      if constexpr (decltype(add_tag)::value) {
+        const float4 o = *p;
         *p = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
       } else {
         *p = v;
@@ -704,10 +701,20 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
     // this lane's accumulator column and its bias
     const int col_own = n0 + wave * 32 + (lane & 31);
     const float bias_own = (EPI && g.bias && col_own < N) ? g.bias[(int64_t)rel * N + col_own] : 0.f;
+    // The tile loop exists three times, chosen once per wave (WAY 0: plain stores through the
+    // LDS area, 1: the same with read-add-stores, 2: from the accumulators).  The first contains
+    // no load from global memory, so the compiler puts no wait for memory into it; with all
+    // kinds of store in one loop it waited at the loop's end for everything in flight, stores
+    // included, because the reading paths reuse registers (7.3 M x 64 x 64 rows: 0.85 -> 0.71 ms
+    // without that wait).
+    auto run_tiles = [&](auto way_tag) {
+    constexpr int WAY = decltype(way_tag)::value;
+    constexpr bool WIDE = WAY < 2;
+    constexpr std::integral_constant<bool, WAY == 1> add_tag{};
     for (int t = 0; t < n_tiles; ++t) {
       __syncthreads();
       const uint16_t (*src)[kBM][KP] = Ap[t & 1];
-      const bool drain = wide_store && t > 0;
+      const bool drain = WIDE && t > 0;
       float4 pv[PPS];
       int64_t pd[PPS];
       v16f acc[2];
@@ -732,7 +739,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
         if (drain) {
           if (s > 0) {
 #pragma unroll
-            for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u]);
+            for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u], add_tag);
           }
 #pragma unroll
           for (int u = 0; u < PPS; ++u) {
@@ -772,7 +779,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       }
       if (drain) {
 #pragma unroll
-        for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u]);
+        for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u], add_tag);
       }
       if (EPI && g.bias) {
 #pragma unroll
@@ -780,7 +787,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) acc[mt][i] += bias_own;
       }
-      if (wide_store) {
+      if constexpr (WIDE) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -790,9 +797,17 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
         store_tile<128, 2, EPI, 4>(g, acc, s_dst[t % SLOTS], 0, wave, lane, n0);
       }
     }
-    if (wide_store) {
+    if constexpr (WIDE) {
 #pragma unroll
-      for (int it = 0; it < 8; ++it) piece_store(piece_read(it), piece_row(it, n_tiles - 1));
+      for (int it = 0; it < 8; ++it) piece_store(piece_read(it), piece_row(it, n_tiles - 1), add_tag);
+    }
+    };
+    if constexpr (KS <= 8) {
+      if (wide_store && !g.accumulate) run_tiles(std::integral_constant<int, 0>{});
+      else if (wide_store) run_tiles(std::integral_constant<int, 1>{});
+      else run_tiles(std::integral_constant<int, 2>{});
+    } else {
+      run_tiles(std::integral_constant<int, 2>{});
     }
   } else {
     if (MAPPED) {
