@@ -105,6 +105,65 @@ __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&
     }
     return;
   }
+  if constexpr (QB == 4 && MODE == 1) {
+    // Accumulation: the old rows of the whole tile are requested first, then all sums are
+    // formed, then all rows are stored (with an addend only, 16 rows at a time as below
+    // measured faster: 2.45 M x 256 x 256 2.92 against 3.23 ms; accumulation 3.21 -> 2.73 ms).  Loads and stores of
+    // a wave share one in-order counter and a store may be acknowledged before an older load
+    // returns, so a load that is waited for after a store is waited for together with that
+    // store's acknowledgement; and a read-add-store per element in turn is one trip to memory
+    // after the other, since a store may alias the next load.  The loads carry no condition
+    // (rows that do not exist read a weight element instead); the row indices are read from
+    // LDS a second time for the stores rather than kept.
+    float o[MT][16];
+    const bool both = EPI && g.addend;
+    const float* const src = both ? g.addend + col : base;
+    const int64_t ld = both ? g.ldd : ldc;
+    const float* const safe = reinterpret_cast<const float*>(g.w) + col;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int rl0 = (wm * MT + mt) * 32 + q * 8 + (lane >> 5) * 4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int64_t d = s_dst[rl0 + j];
+          o[mt][q * 4 + j] = *(d >= 0 ? src + d * ld : safe);
+        }
+      }
+    if (both) {                              // accumulation and an addend: the old rows as well
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rl0 = (wm * MT + mt) * 32 + q * 8 + (lane >> 5) * 4;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int64_t d = s_dst[rl0 + j];
+            o[mt][q * 4 + j] += *(d >= 0 ? base + d * ldc : safe);
+          }
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        o[mt][i] += acc[mt][i];
+        asm volatile("" : "+v"(o[mt][i]));   // (an opaque use: otherwise each sum moves down to its store)
+      }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int rl0 = (wm * MT + mt) * 32 + q * 8 + (lane >> 5) * 4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int64_t d = s_dst[rl0 + j];
+          if (d >= 0) base[d * ldc] = o[mt][q * 4 + j];
+        }
+      }
+    return;
+  }
   // What the rows are added to (the old row when accumulating, the addend) is requested for
   // 4 * QB rows before their first store: a read-add-store per element in turn is one trip
   // to memory after the other, since a store may alias the next load.
@@ -484,11 +543,13 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
   // stores (or read-add-stores) of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
-  // (not with an addend: those rows leave from the accumulators, see store_tile_mode -- measured
-  // faster, 7.3 M x 128 x 128 3.52 -> 2.37 ms, while accumulation into C is faster this way, 3.08
-  // against 3.47 ms)
-  const bool wide_store = KS <= 8 && !g.atomic && !(EPI && g.addend) && n0 + wave * 32 + 32 <= N &&
-                          (g.ldc & 3) == 0 && ((uintptr_t)g.c & 15) == 0;
+  const bool wide_store = KS <= 8 && !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
+                          ((uintptr_t)g.c & 15) == 0 &&
+                          (!EPI || !g.addend || ((g.ldd & 3) == 0 && ((uintptr_t)g.addend & 15) == 0));
+  // what a stored row is added to, if anything: the addend (epilogue entry point, never together
+  // with accumulation) or the row of C itself
+  const float* const add_src = (EPI && g.addend) ? g.addend : g.accumulate ? g.c : nullptr;
+  const int64_t add_ld = (EPI && g.addend) ? g.ldd : g.ldc;
 
   // ---- producer state -------------------------------------------------------------
   const int ptid = tid & 255;
@@ -688,11 +749,16 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       return *reinterpret_cast<const float4*>(&Cw[it * 8 + (lane >> 3)][(lane & 7) * 4]);
     };
     auto piece_row = [&](int it, int t) -> int64_t { return s_dst[t % SLOTS][it * 8 + (lane >> 3)]; };
+    auto old_load = [&](int64_t d) -> float4 {
+      const int colq = n0 + wave * 32 + (lane & 7) * 4;
+      const float* q = d >= 0 ? add_src + d * add_ld + colq : reinterpret_cast<const float*>(g.w) + colq;
+      return *reinterpret_cast<const float4*>(q);
+    };
     auto piece_store = [&](const float4& v, int64_t d, auto add_tag) {
       if (d < 0) return;
       float4* const p = reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wave * 32 + (lane & 7) * 4);
       if constexpr (decltype(add_tag)::value) {
-        const float4 o = *p;
+        const float4 o = *reinterpret_cast<const float4*>(add_src + d * add_ld + n0 + wave * 32 + (lane & 7) * 4);
         *p = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
       } else {
         *p = v;
@@ -715,8 +781,10 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       __syncthreads();
       const uint16_t (*src)[kBM][KP] = Ap[t & 1];
       const bool drain = WIDE && t > 0;
+      const int tp = t > 0 ? t - 1 : 0;        // the tile whose pieces leave during this one
       float4 pv[PPS];
       int64_t pd[PPS];
+      float4 po[8];                            // WAY 1: the old rows of tile t-1's pieces
       v16f acc[2];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
@@ -736,7 +804,14 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         if (s + 1 < KS) read_ap(s + 1);
-        if (drain) {
+        if constexpr (WAY == 1) {
+          // read-add-stores: the old rows of the eight pieces of tile t-1 are requested here,
+          // at the start of tile t, and added and stored after its last k-step (below)
+          if (s == 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) po[i] = old_load(piece_row(i, tp));
+          }
+        } else if (drain) {
           if (s > 0) {
 #pragma unroll
             for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u], add_tag);
@@ -777,7 +852,28 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
             acc[mt][q * 4 + 3] *= ri.w * inv_w;
           }
       }
-      if (drain) {
+      if constexpr (WAY == 1) {
+        // Loads and stores of a wave share one in-order counter, and a store may be acknowledged
+        // before an older load returns: a load that is waited for after a store can only be
+        // waited for together with everything before it.  So all eight sums are formed first
+        // (one wait, for loads that have had the whole tile to return) and the eight stores
+        // follow with no wait between them.  The loads carry no condition (rows that do not
+        // exist read a weight row instead), so the compiler counts them exactly.  (One
+        // read-add-store per piece in turn, between the k-steps, made every piece a trip to
+        // memory: 7.3 M x 128 x 128 rows 3.08 ms.)
+        __builtin_amdgcn_sched_barrier(0);     // the sums stay behind the last k-step
+        if (drain) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float4 v = piece_read(i);
+            po[i] = make_float4(po[i].x + v.x, po[i].y + v.y, po[i].z + v.z, po[i].w + v.w);
+            // (an opaque use: otherwise each sum is moved down into the branch around its store)
+            asm volatile("" : "+v"(po[i].x), "+v"(po[i].y), "+v"(po[i].z), "+v"(po[i].w));
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) piece_store(po[i], piece_row(i, tp), std::false_type{});
+        }
+      } else if (drain) {
 #pragma unroll
         for (int u = 0; u < PPS; ++u) piece_store(pv[u], pd[u], add_tag);
       }
@@ -803,7 +899,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
     }
     };
     if constexpr (KS <= 8) {
-      if (wide_store && !g.accumulate) run_tiles(std::integral_constant<int, 0>{});
+      if (wide_store && !add_src) run_tiles(std::integral_constant<int, 0>{});
       else if (wide_store) run_tiles(std::integral_constant<int, 1>{});
       else run_tiles(std::integral_constant<int, 2>{});
     } else {
