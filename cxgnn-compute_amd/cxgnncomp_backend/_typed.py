@@ -179,7 +179,8 @@ def dense_linear_add_(out, x, w_kn):
         return False
     M, K = x.shape
     N = w_kn.shape[1]
-    if (M < DENSE_MIN_ROWS or K % 4 or K > 128 or tuple(out.shape) != (M, N)
+    wide = 176 <= K <= 256 and N >= 96 and M >= DENSE_WIDE_MIN_ROWS
+    if (M < DENSE_MIN_ROWS or K % 4 or not (K <= 128 or wide) or tuple(out.shape) != (M, N)
             or not x.is_contiguous() or not out.is_contiguous() or x.data_ptr() % 16):
         return False
     typed_gemm(x, w_kn.contiguous().unsqueeze(0), _one_segment(M, x.device), M, out=out, accumulate=True,

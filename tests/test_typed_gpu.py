@@ -457,14 +457,12 @@ def test_dense_linear_helpers_match_library(M, K, N):
     assert_close(_np(got), _np(want), RTOL, 2 * ATOL, "dense_linear bias")
     got = _typed.dense_linear(x, w.t(), b, add)
     assert_close(_np(got), _np(want + add.double()), RTOL, 2 * ATOL, "dense_linear bias addend")
-    if K <= 128:
-        acc = add.clone()
-        assert _typed.dense_linear_add_(acc, x, w.t())
-        assert_close(_np(acc), _np(want - b.double() + add.double()), RTOL, 2 * ATOL, "dense_linear_add_")
-    else:
-        acc = add.clone()
-        assert not _typed.dense_linear_add_(acc, x, w.t())
-        assert torch.equal(acc, add)
+    acc = add.clone()
+    assert _typed.dense_linear_add_(acc, x, w.t())
+    assert_close(_np(acc), _np(want - b.double() + add.double()), RTOL, 2 * ATOL, "dense_linear_add_")
+    acc = add[:100].clone()
+    assert not _typed.dense_linear_add_(acc, x[:100], w.t())         # too few rows: nothing written
+    assert torch.equal(acc, add[:100])
     assert _typed.dense_linear(x[:100], w.t(), b) is None
     assert _typed.dense_linear(x.double(), w.t().double(), b.double()) is None
 
