@@ -262,7 +262,7 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
 /* Typed (relation-segmented) GEMM -- the MFMA path                            */
 /* ------------------------------------------------------------------------- */
 
-#define CXG_GEMM_ACCUMULATE 1u /* C += A W instead of C = A W                      */
+#define CXG_GEMM_ACCUMULATE 1u /* C += A W instead of C = A W (read-add-store: every destination row at most once per call) */
 #define CXG_GEMM_ATOMIC 2u     /* add with fp32 atomics (several rows share a dst) */
 #define CXG_GEMM_SPLIT_BF16X6 4u /* fp32 products as 6 bf16 partial products (fp32-accurate) */
 #define CXG_GEMM_SPLIT_BF16X3 8u /* fp32 products as 3 bf16 partial products (2^-16 / product) */
