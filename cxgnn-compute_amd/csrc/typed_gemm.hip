@@ -421,7 +421,9 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_kernel(GemmArgs g) {
 // issued before it -- the stores of a tile then have to drain (microseconds under a
 // write-heavy load) before the next tile can be staged.  Consumer waves never wait on
 // memory: their stores (or atomics) stay in flight for as long as the hardware queue
-// allows.  Producer waves only ever wait for their own loads.  The conversion work of
+// allows (when rows are added to -- accumulation, an addend -- they wait once per tile,
+// for old rows requested a tile earlier; see the tile loops).  Producer waves only ever
+// wait for their own loads.  The conversion work of
 // the producers runs on the same SIMDs in the shadow of the consumers' MFMAs.
 template <int NS>
 __device__ __forceinline__ void split_bf16(float x, __bf16 (&p)[NS]) {
