@@ -439,9 +439,11 @@ class _PairGraph:
                                its backward pair row.
     For the aggregate-first order (built on first use, _pair_graph_aggregate):
       bp_ptr [Ub+1], bp_src [E]  CSR over the backward pairs: sources of a pair's edges;
-      dp_ptr [n+1], dp_rows [Ub] CSR over the destinations: the pair rows of a destination."""
+      dp_ptr [n+1], dp_rows [Ub] CSR over the destinations: the pair rows of a destination;
+      mean_fwd [E], mean_rev [E] 1 / in-degree of every edge's destination in bp and in reversed
+                               edge order (the mean layer, _pair_mean_weights)."""
     __slots__ = ("n_edges", "f_src", "f_seg", "f_row", "f_ptr", "f_dst", "b_dst", "b_seg", "ptr_src", "b_row_rev",
-                 "b_row", "bp_ptr", "bp_src", "dp_ptr", "dp_rows", "_keep")
+                 "b_row", "bp_ptr", "bp_src", "dp_ptr", "dp_rows", "mean_fwd", "mean_rev", "_keep")
 
 
 _PAIR_CACHE = collections.OrderedDict()
@@ -475,7 +477,7 @@ def _pair_graph(ptr, idx, rel, n, n_src, R):
     pg.ptr_src = tg.ptr_t
     pg.b_row_rev = b_row[tg.perm].contiguous()
     pg.b_row = b_row.contiguous()
-    pg.bp_ptr = pg.bp_src = pg.dp_ptr = pg.dp_rows = None
+    pg.bp_ptr = pg.bp_src = pg.dp_ptr = pg.dp_rows = pg.mean_fwd = pg.mean_rev = None
     pg._keep = (ptr, idx, rel)
     _PAIR_CACHE[key] = pg
     while len(_PAIR_CACHE) > _REL_CACHE_CAP:
@@ -493,26 +495,45 @@ def _pair_graph_aggregate(pg, idx, n):
     return pg
 
 
-def _pairs_aggregate_first(pg, x, weights, idx, n, precision=None):
+def _pair_mean_weights(pg, ptr, n):
+    """1 / in-degree of the destination of every edge, in the edge order of the pair rows
+    (bp) and of the reversed graph (ptr_src): with these as edge values the two gathers of
+    the aggregate-first order apply the division by the degree themselves, so neither the
+    output nor its gradient takes a pass of its own.  Kept with the pair graph."""
+    if pg.mean_fwd is None:
+        per_pair = _inv_degree(ptr, n)[pg.b_dst]
+        n_pairs = pg.b_dst.shape[0]
+        pg.mean_fwd = per_pair[_ops.csr_row_ids(pg.bp_ptr, n_pairs, pg.bp_src.shape[0])].contiguous()
+        pg.mean_rev = per_pair[pg.b_row_rev].contiguous()
+    return pg.mean_fwd, pg.mean_rev
+
+
+def _pairs_aggregate_first(pg, x, weights, idx, n, precision=None, mean_ptr=None):
     """out[d] = sum_r (sum of x over d's edges of relation r) @ W[r] on the (destination,
     relation) pairs that own an edge: one SpMM into the pair rows (gathering rows of x), one
     typed GEMM over the relation segments of pair rows, one SpMM that gives every destination
-    the sum of its pairs' product rows.  Returns (out, z) with z the aggregated pair rows."""
+    the sum of its pairs' product rows.  With ``mean_ptr`` (the row offsets of the graph) the
+    first SpMM weights every edge by 1 / in-degree of its destination, which divides out[d] by
+    the degree.  Returns (out, z)
+    with z the aggregated (and weighted) pair rows."""
     _pair_graph_aggregate(pg, idx, n)
     n_pairs = pg.b_dst.shape[0]
-    z = _ops.spmm(pg.bp_ptr, pg.bp_src, x, n_pairs)                       # [Ub, K]
+    val = _pair_mean_weights(pg, mean_ptr, n)[0] if mean_ptr is not None else None
+    z = _ops.spmm(pg.bp_ptr, pg.bp_src, x, n_pairs, val=val)              # [Ub, K]
     t = typed_gemm(z, weights, pg.b_seg, n_pairs, precision=precision)                         # [Ub, N]
     return _ops.spmm(pg.dp_ptr, pg.dp_rows, t, n), z
 
 
-def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w, precision=None):
-    """Gradients of _pairs_aggregate_first for x and the weights."""
+def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w, precision=None, mean=False):
+    """Gradients of _pairs_aggregate_first for x and the weights (``mean``: the forward pass
+    weighted the edges by 1 / degree; z holds the weighted rows, so only the gather of the
+    input gradient repeats the weights)."""
     n_pairs = pg.b_dst.shape[0]
     gx = gw = None
     if need_x:
         gz = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, n_pairs, src_idx=pg.b_dst,
                         precision=precision)
-        gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, gz, n_src)
+        gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, gz, n_src, val=pg.mean_rev if mean else None)
     if need_w:
         gw = _weight_grad(z, grad_out, _edge_positions(n_pairs, z.device), pg.b_dst, pg.b_seg, weights.shape,
                           precision)
@@ -561,9 +582,7 @@ class _RgcnFusedFunction(torch.autograd.Function):
             ctx.pairs = pg.f_src.shape[0] <= RGCN_PAIR_FILL_MAX * n_src * R
         ctx.aggregate_first = ctx.pairs and K <= N and not force_dense     # gather the narrower rows
         if ctx.aggregate_first:
-            out, z = _pairs_aggregate_first(pg, x, weights, idx, n, precision)
-            if mean:
-                out *= _inv_degree(ptr, n).unsqueeze(1)
+            out, z = _pairs_aggregate_first(pg, x, weights, idx, n, precision, ptr if mean else None)
             ctx.pg = pg
             ctx.save_for_backward(x, weights, ptr, z)
             return out
@@ -606,13 +625,14 @@ class _RgcnFusedFunction(torch.autograd.Function):
         R, K, N = weights.shape
         n, n_src = ctx.n, x.shape[0]
         precision = ctx.precision
-        if ctx.mean:
-            grad_out = grad_out * _inv_degree(ptr, n).unsqueeze(1)
         gx = gw = None
         if ctx.aggregate_first:
             gx, gw = _pairs_aggregate_first_bwd(ctx.pg, weights, ctx.saved_tensors[3], grad_out, n_src,
-                                                ctx.needs_input_grad[0], ctx.needs_input_grad[3], precision)
+                                                ctx.needs_input_grad[0], ctx.needs_input_grad[3], precision,
+                                                ctx.mean)
             return gx, None, None, gw, None, None, None, None, None
+        if ctx.mean:
+            grad_out = grad_out * _inv_degree(ptr, n).unsqueeze(1)
         if ctx.pairs:
             pg = ctx.pg
             if ctx.needs_input_grad[0]:
