@@ -84,7 +84,7 @@ __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&
   if (col >= g.N) return;
   float* const base = g.c + col;
   const int64_t ldc = g.ldc;
-  if constexpr (MODE != 1 && !EPI) {
+  if (MODE != 1 && !(EPI && g.addend)) {
     // nothing is read: the rows of a group of four as soon as their indices are there
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -559,7 +559,6 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const bool k_ok = 4 * c4 < K;
   const float* A = reinterpret_cast<const float*>(g.a);
   float4 areg0[NLD], areg1[NLD];             // rows of the next two tiles, in flight
-  unsigned live0 = 0, live1 = 0;             // bit i: row i of the set exists (its values are zeroed otherwise)
   // Row tables (source and destination row of every row of a tile; -1: no such row).
   // Given row maps (MAPPED) are fetched for ALL the block's tiles before the first tile,
   // beside the consumers' weight loads: the loads of a wave complete in order, so a map
@@ -574,45 +573,53 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
     }
   };
   // Loads are issued unconditionally (rows and columns that do not exist are redirected
-  // to an address that does and zeroed when the tile is staged): with no branch around a
+  // to an address that does; see the staging code for what happens to them): with no branch around a
   // load the compiler counts the loads in flight exactly and waits only for the older of
   // the two register sets.
-  // Which rows exist is noted here, as a bit mask that travels with the register set: the
-  // staging code then runs from the loaded registers alone, with no table look-up (an LDS
-  // read and a wait per row) between the conversions.
-  auto gload = [&](float4 (&areg)[NLD], unsigned& live_mask, int t) {
+  // The staging code runs from the loaded registers alone: no table look-up (an LDS read
+  // and a wait per row) between the conversions.
+  auto gload = [&](float4 (&areg)[NLD], int t) {
     const int tc = t < n_tiles ? t : n_tiles - 1;
-    unsigned mask = 0;
+    if constexpr (MAPPED) {
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      int64_t sidx;
-      if constexpr (MAPPED) {
-        sidx = s_src[tc % SLOTS][i * RPI + rsub];
-      } else {
-        sidx = row0 + (int64_t)tc * kBM + i * RPI + rsub;
-        if (sidx >= row_end) sidx = -1;
+      for (int i = 0; i < NLD; ++i) {
+        const int64_t sidx = s_src[tc % SLOTS][i * RPI + rsub];
+        areg[i] = *reinterpret_cast<const float4*>(A + (sidx >= 0 ? sidx : 0) * g.lda + (k_ok ? 4 * c4 : 0));
       }
-      mask |= (sidx >= 0 ? 1u : 0u) << i;
-      areg[i] = *reinterpret_cast<const float4*>(A + (sidx >= 0 ? sidx : 0) * g.lda + (k_ok ? 4 * c4 : 0));
+    } else {
+      // consecutive rows: one base address per tile (the same for every lane, so it lives in
+      // scalar registers) and a 32-bit offset per row instead of sixteen 64-bit addresses kept
+      // from tile to tile -- the widest form (K up to 256: sixteen 16-byte loads per lane and
+      // set) otherwise spills inside this loop, and a reload from scratch memory waits for
+      // every row load in flight before it.  (The launch sees to it that 64 * lda fits.)
+      const int64_t tile_row = row0 + (int64_t)tc * kBM;
+      const float* const base = A + tile_row * g.lda;
+      const int64_t left = row_end - tile_row;
+      const int rows_here = left < kBM ? (int)left : kBM;          // at least 1
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int rl = i * RPI + rsub;
+        const unsigned off = (unsigned)(rl < rows_here ? rl : 0) * (unsigned)g.lda + (unsigned)(k_ok ? 4 * c4 : 0);
+        areg[i] = *reinterpret_cast<const float4*>(base + off);
+      }
     }
-    live_mask = mask;
   };
   // split the rows held in areg and write the parts of tile t into its LDS half
-  auto stage = [&](const float4 (&areg)[NLD], unsigned live_mask, int t) {
+  // Rows that do not exist (past the segment's end, or skipped by a negative map entry) hold
+  // whatever the redirected load returned: an output row depends on its own A row only and
+  // theirs is never stored, so nothing is zeroed for them.  Only the lanes past K (K below
+  // the tile's 16 * KS columns) must contribute zeros, which costs one select per row.
+  auto stage = [&](const float4 (&areg)[NLD], int t) {
     uint16_t (*dst)[kBM][KP] = Ap[t & 1];
     unsigned row_max[NLD];                   // F16: largest magnitude of each row (bit pattern)
     if constexpr (F16) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const bool live = k_ok && ((live_mask >> i) & 1u) != 0;
-        unsigned m = 0;
-        const float v[4] = {areg[i].x, areg[i].y, areg[i].z, areg[i].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const unsigned b = live ? (__float_as_uint(v[j]) & 0x7fffffffu) : 0u;
-          m = b > m ? b : m;
-        }
-        row_max[i] = m;
+        const unsigned b0 = __float_as_uint(areg[i].x) & 0x7fffffffu, b1 = __float_as_uint(areg[i].y) & 0x7fffffffu;
+        const unsigned b2 = __float_as_uint(areg[i].z) & 0x7fffffffu, b3 = __float_as_uint(areg[i].w) & 0x7fffffffu;
+        const unsigned m01 = b0 > b1 ? b0 : b1, m23 = b2 > b3 ? b2 : b3;
+        const unsigned m = m01 > m23 ? m01 : m23;
+        row_max[i] = k_ok ? m : 0u;
       }
 #pragma unroll
       for (int i = 0; i < NLD; ++i) row_max[i] = group_max_u32<LPR>(row_max[i]);
@@ -620,16 +627,18 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int row = i * RPI + rsub;
-      const bool live = k_ok && ((live_mask >> i) & 1u) != 0;
-      const float v[4] = {live ? areg[i].x : 0.f, live ? areg[i].y : 0.f, live ? areg[i].z : 0.f,
-                          live ? areg[i].w : 0.f};
       if constexpr (F16) {
         float scale, inv;
         pow2_scales(row_max[i], scale, inv);
+        // (the widest form zeroes element by element instead: with the select per row its
+        // register allocation spills inside the tile loop, 4.3 -> 6.0 ms at 5 M x 256 x 256)
+        const float sc = (KS == 16 || k_ok) ? scale : 0.f;
+        const float v[4] = {(KS < 16 || k_ok) ? areg[i].x : 0.f, (KS < 16 || k_ok) ? areg[i].y : 0.f,
+                            (KS < 16 || k_ok) ? areg[i].z : 0.f, (KS < 16 || k_ok) ? areg[i].w : 0.f};
         v4h part[2];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float xs = v[j] * scale;
+          const float xs = v[j] * sc;
           const _Float16 h0 = (_Float16)xs;
           part[0][j] = h0;
           part[1][j] = (_Float16)(xs - (float)h0);
@@ -638,6 +647,8 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
         for (int q = 0; q < 2; ++q) *reinterpret_cast<v4h*>(&dst[q][row][4 * c4]) = part[q];
         if (c4 == 0) s_inv[t & 1][row] = inv;
       } else {
+        const float v[4] = {k_ok ? areg[i].x : 0.f, k_ok ? areg[i].y : 0.f, k_ok ? areg[i].z : 0.f,
+                            k_ok ? areg[i].w : 0.f};
         v4bf part[NS];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -927,10 +938,10 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       for (int t = 0; t < 4; ++t) maps_fill(t);
     }
     __syncthreads();                         // row tables visible
-    gload(areg0, live0, 0);
-    gload(areg1, live1, 1);
-    stage(areg0, live0, 0);
-    gload(areg0, live0, 2);
+    gload(areg0, 0);
+    gload(areg1, 1);
+    stage(areg0, 0);
+    gload(areg0, 2);
     // Two iterations per trip, so that each register set keeps a fixed role.  The loop is
     // left with `return`, never through a path that rejoins the loop head with the two
     // register sets in the other order: the compiler, which counts the loads in flight
@@ -940,13 +951,13 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
       if (t >= n_tiles) return;
       __syncthreads();
       maps_fill(t + 4);
-      stage(areg1, live1, t + 1);
-      gload(areg1, live1, t + 3);
+      stage(areg1, t + 1);
+      gload(areg1, t + 3);
       if (t + 1 >= n_tiles) return;
       __syncthreads();
       maps_fill(t + 5);
-      stage(areg0, live0, t + 2);
-      gload(areg0, live0, t + 4);
+      stage(areg0, t + 2);
+      gload(areg0, t + 4);
     }
   }
 }
@@ -1147,7 +1158,7 @@ static int typed_gemm_f32_impl(const float* a, int64_t lda, const float* w, cons
   // N = 256 10.6 -> 5.8 ms, N = 128 5.3 -> 3.3 ms; K = 160, N = 64 2.0 -> 2.5 ms).
   const bool wide_k = (flags & CXG_GEMM_SPLIT_F16X3) && K > 128 && K <= 256 && K >= 176 && N >= 96;
   if ((flags & (CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) && (K <= 128 || wide_k) && (K & 3) == 0 &&
-      (lda & 3) == 0 && ((uintptr_t)a & 15) == 0) {
+      (lda & 3) == 0 && lda < ((int64_t)1 << 24) && ((uintptr_t)a & 15) == 0) {
     // 64*G rows per block, up to 32 tiles (16 with row maps, which the block keeps in LDS).  A
     // CU runs one block at a time and a block first loads and splits its weight slab, so few
     // large blocks beat many small ones: the number of rounds of one block per CU that the
