@@ -351,6 +351,16 @@ def test_typed_gemm_small_shapes_and_skipped_rows(M, K, N):
         if not bool(skip[i]):
             want[dst[i]] = a[src[i]].double() @ w[types[i]].double()
     assert_close(_np(out), want.numpy(), RTOL, 2 * ATOL, "typed_gemm with skipped rows")
+    # the same rows added to what is there (the read-add-store paths), twice in a row
+    acc = torch.full((M + 5, N), 3.0).cuda()
+    for _ in range(2):
+        _typed.typed_gemm(a.cuda(), w.cuda(), seg.cuda(), M, src_idx=src_m.cuda(), dst_idx=dst_m.cuda(), out=acc,
+                          accumulate=True)
+    want_acc = torch.full((M + 5, N), 3.0, dtype=torch.float64)      # 3 + 2 * product on the rows that exist
+    for i in range(M):
+        if not bool(skip[i]):
+            want_acc[dst[i]] += 2 * want[dst[i]]
+    assert_close(_np(acc), want_acc.numpy(), RTOL, 4 * ATOL, "typed_gemm accumulate with skipped rows")
     g = torch.randn(M + 5, N, generator=gen)
     gw = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg.cuda(), M, R, src_idx=src_m.cuda(), dst_idx=dst_m.cuda())
     want_gw = torch.zeros(R, K, N, dtype=torch.float64)
