@@ -160,6 +160,14 @@ __global__ void transpose_prefix_fill_kernel(const int64_t* __restrict__ ptr_t_a
   if (k <= n_cols) ptr_t[k] = pos[ptr_t_all[k]];
 }
 
+// rocPRIM sorts up to 2^20 items by merge sort whatever the key width: one block sort and
+// log2(n / 4096) merge passes of two kernels each -- 22 launches of a few microseconds for
+// the 936 k edges of a sampled batch, whose keys have 20 significant bits.  Its radix sort
+// takes one pass per 8 key bits, so it is used from 2^16 items on (the reversed graph of the
+// largest layer of a sampled batch, sort and fills: 0.260 -> 0.225 ms).
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, (size_t)1 << 16>;
+
 int bits_for(int64_t n) {
   int b = 1;
   while (b < 63 && ((int64_t)1 << b) < n) ++b;
@@ -173,7 +181,7 @@ constexpr int64_t kNarrowLimit = (int64_t)1 << 32;
 size_t narrow_sort_temp_bytes(int64_t n_edges, int64_t n_cols) {
   size_t temp = 0;
   ColumnKeyIter keys(nullptr, ColumnKey());
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, keys, (uint32_t*)nullptr,
+  hipError_t e = rocprim::radix_sort_pairs<cxg::SortConfig>(nullptr, temp, keys, (uint32_t*)nullptr,
                                            (const uint64_t*)nullptr, (uint64_t*)nullptr,
                                            (size_t)n_edges, 0, bits_for(n_cols > 1 ? n_cols : 2),
                                            (hipStream_t)0);
@@ -189,7 +197,7 @@ size_t cxg_csr_transpose_workspace_bytes(int64_t n_edges, int64_t n_cols) {
   if (n_edges < 0 || n_cols < 0) return 0;
   size_t temp = 0;
   rocprim::counting_iterator<int64_t> iota(0);
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (const int64_t*)nullptr, (int64_t*)nullptr,
+  hipError_t e = rocprim::radix_sort_pairs<cxg::SortConfig>(nullptr, temp, (const int64_t*)nullptr, (int64_t*)nullptr,
                                            iota, (int64_t*)nullptr, (size_t)n_edges, 0,
                                            cxg::bits_for(n_cols > 1 ? n_cols : 2), (hipStream_t)0);
   if (e != hipSuccess) return 0;
@@ -228,7 +236,7 @@ int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows
                        (void*)packed);
     CXG_LAUNCH_CHECK("expand_rows_kernel");
     cxg::ColumnKeyIter keys(idx, cxg::ColumnKey());
-    CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, keys, sorted_key, packed,
+    CXG_HIP_CHECK(rocprim::radix_sort_pairs<cxg::SortConfig>(temp, temp_bytes, keys, sorted_key, packed,
                                             reinterpret_cast<uint64_t*>(perm), (size_t)n_edges, 0,
                                             cxg::bits_for(n_cols > 1 ? n_cols : 2), st));
     const int64_t work = (n_edges > n_cols + 1) ? n_edges : n_cols + 1;
@@ -239,7 +247,7 @@ int cxg_csr_transpose_i64(const int64_t* ptr, const int64_t* idx, int64_t n_rows
   }
   if (n_edges > 0) {
     rocprim::counting_iterator<int64_t> iota(0);
-    CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, idx, sorted_src, iota, perm,
+    CXG_HIP_CHECK(rocprim::radix_sort_pairs<cxg::SortConfig>(temp, temp_bytes, idx, sorted_src, iota, perm,
                                             (size_t)n_edges, 0, cxg::bits_for(n_cols > 1 ? n_cols : 2),
                                             st));
   }

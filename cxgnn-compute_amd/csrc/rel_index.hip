@@ -33,6 +33,12 @@ __global__ void seg_ptr_kernel(const T* __restrict__ sorted, int64_t n, int R,
   seg_ptr[r] = lo;
 }
 
+// rocPRIM sorts up to 2^20 items by merge sort whatever the key width (a block sort and
+// log2(n / 4096) merge passes of two kernels each); its radix sort takes one pass per 8
+// significant key bits, so it is used from 2^16 items on.
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, (size_t)1 << 16>;
+
 int bits_for(int64_t n) {
   int b = 1;
   while (b < 62 && ((int64_t)1 << b) < n) ++b;
@@ -44,7 +50,7 @@ template <typename T>
 size_t ws_bytes(int64_t n, int R) {
   size_t temp = 0;
   rocprim::counting_iterator<int64_t> iota(0);
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (const T*)nullptr, (T*)nullptr, iota,
+  hipError_t e = rocprim::radix_sort_pairs<cxg::SortConfig>(nullptr, temp, (const T*)nullptr, (T*)nullptr, iota,
                                            (int64_t*)nullptr, (size_t)n, 0, bits_for(R + 1),
                                            (hipStream_t)0);
   if (e != hipSuccess) return 0;
@@ -68,7 +74,7 @@ int rel_segment(const T* types, int64_t n, int R, int64_t* perm, int64_t* seg_pt
   size_t temp_bytes = workspace_bytes - off;
   if (n > 0) {
     rocprim::counting_iterator<int64_t> iota(0);
-    CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, types, sorted, iota, perm, (size_t)n, 0,
+    CXG_HIP_CHECK(rocprim::radix_sort_pairs<cxg::SortConfig>(temp, temp_bytes, types, sorted, iota, perm, (size_t)n, 0,
                                             bits_for(R + 1), st));
   }
   hipLaunchKernelGGL(seg_ptr_kernel<T>, dim3((unsigned)ceil_div(R + 1, kBlock)), dim3(kBlock), 0, st,

@@ -20,6 +20,13 @@
 namespace cxg {
 namespace {
 
+// rocPRIM sorts up to 2^20 items by merge sort whatever the key width (a block sort and
+// log2(n / 4096) merge passes of two kernels each); its radix sort takes one pass per 8
+// significant key bits, so it is used from 2^16 items on.
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, (size_t)1 << 16>;
+
+
 constexpr int kBlock = 256;
 
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
@@ -257,7 +264,7 @@ size_t cxg_coo_to_csr_workspace_bytes(int64_t n_edges, int64_t n_rows) {
   if (n_edges < 0 || n_rows < 0) return 0;
   size_t temp = 0;
   rocprim::counting_iterator<int64_t> iota(0);
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (const int64_t*)nullptr, (int64_t*)nullptr,
+  hipError_t e = rocprim::radix_sort_pairs<cxg::SortConfig>(nullptr, temp, (const int64_t*)nullptr, (int64_t*)nullptr,
                                            iota, (int64_t*)nullptr, (size_t)n_edges, 0,
                                            cxg::bits_for(n_rows > 1 ? n_rows : 2), (hipStream_t)0);
   if (e != hipSuccess) return 0;
@@ -281,7 +288,7 @@ int cxg_coo_to_csr_i64(const int64_t* src, const int64_t* dst, int64_t n_edges, 
   size_t temp_bytes = workspace_bytes - off;
   if (n_edges > 0) {
     rocprim::counting_iterator<int64_t> iota(0);
-    CXG_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, dst, sorted_dst, iota, perm, (size_t)n_edges,
+    CXG_HIP_CHECK(rocprim::radix_sort_pairs<cxg::SortConfig>(temp, temp_bytes, dst, sorted_dst, iota, perm, (size_t)n_edges,
                                             0, cxg::bits_for(n_rows > 1 ? n_rows : 2), st));
   }
   const int64_t work = (n_edges > n_rows + 1) ? n_edges : n_rows + 1;
