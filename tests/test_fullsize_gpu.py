@@ -500,3 +500,41 @@ def test_c5_sage_model_full_size(sampled):
     wg, wr = model.convs[2].lin_r.weight.grad.cpu().numpy(), ref.convs[2].lin_r.weight.grad.numpy()
     scw = float(np.abs(wr).max())
     assert_close(wg / scw, wr / scw, 2e-4, 2e-5, "SAGE grad lin_r of the last layer")
+
+
+@pytest.mark.parametrize("K,N", [(128, 256), (256, 128)])
+def test_dense_layers_full_size(K, N):
+    """The dense products of the layers at the headline node count (2,449,029 rows): the
+    epilogue entry point with bias and addend, and accumulation in place, through the shapes
+    the layers use (128 -> 256 staged stores, 256 -> 128 the wide form).  Checked on sampled
+    rows against float64, and through linearity on all rows: the product of a sum of two
+    inputs equals the sum of the products, to the products' rounding."""
+    from cxgnncomp_backend import _typed
+    M = N_NODES
+    gen = torch.Generator(device="cuda").manual_seed(K + N)
+    x = torch.randn(M, K, device="cuda", generator=gen) / K ** 0.5
+    w = torch.randn(N, K, device="cuda", generator=gen)               # nn.Linear layout
+    b = torch.randn(N, device="cuda", generator=gen)
+    add = torch.randn(M, N, device="cuda", generator=gen)
+    announce("dense_linear %d x %d -> %d with bias and addend" % (M, K, N))
+    got = _typed.dense_linear(x, w.t(), b, add)
+    assert got is not None
+    rows = torch.randint(0, M, (4096,), device="cuda", generator=gen)
+    rows[:2] = torch.tensor([0, M - 1], device="cuda")
+    want = x[rows].double() @ w.double().t() + b.double() + add[rows].double()
+    assert_close(got[rows].cpu().numpy(), want.cpu().numpy(), 1e-4, 2e-5, "dense_linear rows")
+    announce("dense_linear_add_ %d x %d -> %d" % (M, K, N))
+    acc = add.clone()
+    assert _typed.dense_linear_add_(acc, x, w.t())
+    want_acc = x[rows].double() @ w.double().t() + add[rows].double()
+    assert_close(acc[rows].cpu().numpy(), want_acc.cpu().numpy(), 1e-4, 2e-5, "dense_linear_add_ rows")
+    # all rows: bias + addend and accumulation agree with each other up to the bias
+    diff = (got - acc - b).abs().max()
+    assert float(diff) <= 2e-5, float(diff)
+    # linearity on all rows
+    x2 = torch.randn(M, K, device="cuda", generator=gen) / K ** 0.5
+    p1 = _typed.dense_linear(x, w.t())
+    p2 = _typed.dense_linear(x2, w.t())
+    p12 = _typed.dense_linear(x + x2, w.t())
+    scale = float(p12.abs().max())
+    assert float((p12 - p1 - p2).abs().max()) <= 4e-5 * max(1.0, scale)
