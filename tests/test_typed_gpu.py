@@ -497,3 +497,65 @@ def test_linear_op_gradients_through_typed_gemm():
     for name, got, want in (("x", x.grad, xd.grad), ("w", w.grad, wd.grad), ("b", b.grad, bd.grad)):
         scale = max(1.0, float(want.abs().max()))
         assert_close(_np(got) / scale, _np(want) / scale, RTOL, 2 * ATOL, "LinearOP grad " + name)
+
+
+def test_typed_gemm_random_shapes_all_store_paths(gemm_precision):
+    """120 seeded random shapes (M up to 5000, K up to 256, N up to 300, 1 - 5 relations) through
+    every way a row can leave the kernel: plain, accumulating, with row maps and skipped rows,
+    with bias and / or addend through the epilogue entry point; each against float64."""
+    import random
+    from cxgnncomp_backend import _lib, _typed
+    if gemm_precision != "split_f16":
+        pytest.skip("the store paths are those of the default form: runs once")
+    lib = _lib.load()
+    rnd = random.Random(1)
+    gen = torch.Generator().manual_seed(1)
+    announce("typed_gemm random shapes")
+    for case in range(120):
+        M = rnd.choice([1, 7, 63, 64, 65, 200, 1023, 1100, 2049, 5000])
+        K = rnd.choice([4, 8, 36, 64, 100, 128, 176, 200, 256])
+        N = rnd.choice([4, 32, 40, 64, 96, 100, 128, 132, 200, 256, 300])
+        R = rnd.choice([1, 1, 2, 5])
+        mode = rnd.choice(["plain", "acc", "bias", "addend", "bias+addend", "mapped", "mapped_acc"])
+        if mode in ("bias", "addend", "bias+addend") and K > 128 and not (K >= 176 and N >= 96):
+            continue
+        n_a = M + 3
+        a = (torch.randn(n_a, K, generator=gen) / K ** 0.5).cuda()
+        w = torch.randn(R, K, N, generator=gen).cuda()
+        cuts = sorted(rnd.randint(0, M) for _ in range(R - 1))
+        seg = torch.tensor([0] + cuts + [M], dtype=torch.int64).cuda()
+        rel = torch.bucketize(torch.arange(M, device="cuda"), seg[1:], right=True)
+        base = torch.randn(M + 2, N, generator=gen).cuda()
+        out = base.clone()
+        src = dst = None
+        if mode.startswith("mapped"):
+            src = torch.randint(0, n_a, (M,), generator=gen).cuda()
+            dst = torch.randperm(M + 2, generator=gen)[:M].cuda()
+            src = torch.where((torch.rand(M, generator=gen) < 0.15).cuda(), torch.full_like(src, -1), src)
+        s_eff = src if src is not None else torch.arange(M, device="cuda")
+        d_eff = dst if dst is not None else torch.arange(M, device="cuda")
+        live = s_eff >= 0
+        prod = torch.zeros(M, N, dtype=torch.float64, device="cuda")
+        prod[live] = torch.bmm(a[s_eff[live]].double().unsqueeze(1), w[rel[live]].double()).squeeze(1)
+        want = base.double().clone()
+        if mode in ("plain", "mapped"):
+            want[d_eff[live]] = prod[live]
+            _typed.typed_gemm(a, w, seg, M, src_idx=src, dst_idx=dst, out=out)
+        elif mode in ("acc", "mapped_acc"):
+            want[d_eff[live]] += prod[live]
+            _typed.typed_gemm(a, w, seg, M, src_idx=src, dst_idx=dst, out=out, accumulate=True)
+        else:
+            bias = torch.randn(R, N, generator=gen).cuda() if "bias" in mode else None
+            addend = torch.randn(M, N + 4, generator=gen).cuda() if "addend" in mode else None
+            want[:M] = prod
+            if bias is not None:
+                want[:M] += bias[rel].double()
+            if addend is not None:
+                want[:M] += addend[:, :N].double()
+            st = lib.cxg_typed_gemm_epilogue_f32(a.data_ptr(), K, w.data_ptr(), _lib.ptr(bias), _lib.ptr(addend), N + 4,
+                                                 out.data_ptr(), N, None, None, seg.data_ptr(), M, K, N, R,
+                                                 _typed.GEMM_SPLIT_F16X3, _lib.current_stream(a.device))
+            _lib.check(st)
+        torch.cuda.synchronize()
+        assert_close(_np(out), want.cpu().numpy(), RTOL, 2 * ATOL,
+                     "case %d: M=%d K=%d N=%d R=%d %s" % (case, M, K, N, R, mode))
