@@ -116,6 +116,7 @@ def test_gat_configuration_full_size(big):
     got = ev.detach()[torch.from_numpy(pos).cuda()].cpu().numpy()
     assert_close(got, ref, 2e-4, 1e-7, "softmax on sampled rows vs oracle")
     x = (torch.randn(N_NODES, H, C, device="cuda") / 8).requires_grad_(True)
+    ev.retain_grad()
     announce("SpMMValOP fwd+bwd full size")
     out = SpMMValOP.apply(x, ptr, idx, ev, N_NODES)
     g = torch.randn(N_NODES, H, C, device="cuda") / 8
@@ -129,6 +130,41 @@ def test_gat_configuration_full_size(big):
     assert abs(lhs - rhs) <= 1e-6 * max(1.0, abs(lhs))
     assert att_src.grad is not None and att_dst.grad is not None
     assert torch.isfinite(att_src.grad).all() and torch.isfinite(att_dst.grad).all()
+    # The edge-value gradient (left by the pass over the reversed graph that also computes grad_x)
+    # on the sampled rows' edges: gval[e,h] = <g[row(e),h,:], x[idx[e],h,:]>.
+    rows_d = torch.from_numpy(rows).cuda()
+    pos_d = torch.from_numpy(pos).cuda()
+    x_np = x.detach().cpu().numpy()
+    gval = ev.grad[pos_d].cpu().numpy()
+    ref_gval = oracle.edge_grad(sub_ptr, sub_idx, x_np, g[rows_d].cpu().numpy(), len(rows))
+    assert_close(gval, ref_gval, 1e-4, 1e-5, "edge-value gradient on sampled rows vs oracle")
+    # The softmax backward on the same rows, fed with the kernel's own forward output and edge-value
+    # gradient: grad_att_dst of a row needs that row's edges only.
+    gd_ref, _ = oracle.edge_softmax_bwd(sub_ptr, sub_idx, gval, mask, got, len(rows), N_NODES, 0.2)
+    assert_close(att_dst.grad[rows_d].cpu().numpy(), gd_ref, 1e-4, 1e-5, "grad att_dst on sampled rows vs oracle")
+    # grad_att_src of a source sums one term from every row that lists it, and each term needs its
+    # whole row: take sources of moderate out-degree, collect every row that gathers from them (the
+    # graph is symmetric as a multiset, so those rows are the sources' own neighbour lists) and run
+    # the oracle over all edges of those rows.
+    deg_np = deg.cpu().numpy()
+    p_np = ptr.cpu().numpy()
+    cand = np.nonzero((deg_np > 0) & (deg_np <= 48))[0]
+    srcs = np.unique(np.concatenate([rng.choice(cand, 48, replace=False),
+                                     np.nonzero((deg_np > 200) & (deg_np < 400))[0][:2]]))
+    nb = np.unique(np.concatenate([idx[int(p_np[s]):int(p_np[s + 1])].cpu().numpy() for s in srcs]))
+    sp2, si2, pos2 = _sub_csr(ptr, idx, nb)
+    assert len(si2) < 30_000_000
+    announce("oracle softmax backward over %d rows / %d edges for %d sources" % (len(nb), len(si2), len(srcs)))
+    pos2_d = torch.from_numpy(pos2).cuda()
+    ev2 = ev.detach()[pos2_d].cpu().numpy()
+    _, mask2 = oracle.edge_softmax_fwd(sp2, si2, att_dst.detach()[torch.from_numpy(nb).cuda()].cpu().numpy(),
+                                       att_src.detach().cpu().numpy(), len(si2), 0.2)
+    _, gs_ref = oracle.edge_softmax_bwd(sp2, si2, ev.grad[pos2_d].cpu().numpy(), mask2, ev2, len(nb), N_NODES, 0.2)
+    # every edge into a sampled source lies in a collected row
+    into = torch.isin(idx, torch.from_numpy(srcs).cuda())
+    assert int(into.sum()) == int(torch.isin(torch.from_numpy(si2), torch.from_numpy(srcs)).sum())
+    assert_close(att_src.grad[torch.from_numpy(srcs).cuda()].cpu().numpy(), gs_ref[srcs], 1e-4, 1e-5,
+                 "grad att_src on sampled sources vs oracle")
     # every edge term of the softmax gradient reaches exactly one source and one destination,
     # and a row whose activations share a sign contributes zero in total to both
     assert abs(float(att_src.grad.double().sum()) - float(att_dst.grad.double().sum())) < 1e-2
@@ -165,6 +201,160 @@ def test_gspmm_full_size(big):
     ref = oracle.gspmm(sp.astype(np.int32), si.astype(np.int32), x.cpu().numpy(), 2, 0,
                        val=val[torch.from_numpy(pos).cuda()].cpu().numpy())
     assert np.array_equal(got2[torch.from_numpy(rows).cuda()].cpu().numpy(), ref)
+
+
+# --------------------------------------------------------------------------- #
+# 3-layer GCN configuration at its stated size: 169,343 nodes / 1,166,243 directed edges
+# symmetrised to 2,332,486 CSR entries, features 128 -> 256 -> 256 -> 40
+# --------------------------------------------------------------------------- #
+C2_N, C2_DIRECTED = 169343, 1166243
+
+
+@pytest.fixture(scope="module")
+def citation():
+    from cxgnncomp import synthetic as S
+    announce("generate the 169,343-node / 2,332,486-entry graph")
+    ptr, idx = S.powerlaw_directed_symmetrised(C2_N, C2_DIRECTED, seed=0)
+    assert idx.shape[0] == 2 * C2_DIRECTED and ptr.shape[0] == C2_N + 1
+    return ptr, idx
+
+
+@pytest.mark.parametrize("feat", [128, 256])
+def test_c2_spmm_forward_backward_full_size(citation, feat):
+    """Sum and 1/deg-weighted aggregation, forward and over the reversed graph, at both row widths
+    of the configuration, every row against the oracle.  The edge multiset is symmetric, so the
+    sum's reversed pass alone could not tell A from A^T: the weighted form (weights depend on the
+    destination only) and a row-prefix call (rows [0, N/3) of the same CSR) are not symmetric."""
+    import cxgnncomp_backend as B
+    ptr, idx = citation
+    p_np, i_np = ptr.numpy(), idx.numpy()
+    n, E = C2_N, idx.shape[0]
+    deg = ptr[1:] - ptr[:-1]
+    sc = 1.0 / float(deg.max()) ** 0.5
+    torch.manual_seed(feat)
+    x = torch.randn(n, feat) * sc
+    g = torch.randn(n, feat) * sc
+    pc, ic = ptr.cuda(), idx.cuda()
+    z = (0,) * 9
+    announce("C2 sum SpMM forward F=%d" % feat)
+    out = B.run_spmm_configurable(pc, ic, x.cuda(), n, *z)
+    assert_close(out.cpu().numpy(), oracle.spmm(p_np, i_np, x.numpy(), n), 1e-4, 1e-5, "sum forward")
+    announce("C2 sum SpMM reversed-graph backward F=%d" % feat)
+    gx = B.run_spmm_configurable_bwd(pc, ic, x.cuda(), g.cuda(), n, *z)
+    assert_close(gx.cpu().numpy(), oracle.spmm_bwd(p_np, i_np, g.numpy(), n, n), 1e-4, 1e-5, "sum backward")
+    rows = n // 3
+    announce("C2 sum SpMM backward over the row prefix [0, %d) F=%d" % (rows, feat))
+    xg = x.cuda().requires_grad_(True)
+    o = B.sage_sum_forward(xg, pc, ic, rows)
+    o.backward(g[:rows].cuda())
+    assert_close(o.detach().cpu().numpy(), oracle.spmm(p_np, i_np, x.numpy(), rows), 1e-4, 1e-5, "prefix forward")
+    assert_close(xg.grad.cpu().numpy(), oracle.spmm_bwd(p_np, i_np, g[:rows].numpy(), rows, n), 1e-4, 1e-5,
+                 "prefix backward")
+    announce("C2 1/deg-weighted SpMM forward + backward F=%d" % feat)
+    val = B.edge_value_degree(pc, n, E)
+    v_np = oracle.edge_value_degree(p_np, n, E)
+    assert np.array_equal(val.cpu().numpy(), v_np)
+    xg = x.cuda().requires_grad_(True)
+    ow = B.sage_sum_forward_edge_value(xg, pc, ic, val, n)
+    ow.backward(g.cuda())
+    torch.cuda.synchronize()
+    assert_close(ow.detach().cpu().numpy(), oracle.spmm(p_np, i_np, x.numpy(), n, val=v_np), 1e-4, 1e-5,
+                 "weighted forward")
+    assert_close(xg.grad.cpu().numpy(), oracle.spmm_bwd(p_np, i_np, g.numpy(), n, n, val=v_np), 1e-4, 1e-5,
+                 "weighted backward")
+    # the weighted forward is the mean aggregation
+    m = B.sage_mean_forward(x.cuda(), pc, ic, n)
+    assert_close(m.cpu().numpy(), ow.detach().cpu().numpy(), 1e-5, 1e-7, "1/deg weights == mean")
+
+
+@pytest.mark.parametrize("normalize", [False, True])
+def test_c2_gcn_model_full_size(citation, normalize):
+    """3-layer GCN 128 -> 256 -> 256 -> 40 (BatchNorm + ReLU between the layers, model.py:58-71),
+    sum aggregation (AggrOP) and 1/deg-weighted aggregation (gcn_norm), logits, input gradient and
+    all weight gradients against a float64 restatement of the stack on the host.
+
+    A ReLU network is piecewise linear; which piece a point lies on is decided by the signs of
+    172 million pre-activations, and the few that float64 puts within rounding of zero may fall on
+    the other side in fp32.  The restatement therefore takes the activation pattern from the GPU
+    run (the positive entries of the layers' post-ReLU outputs), checks that it differs from its
+    own signs only where its pre-activation is within 1e-5 of zero, and compares values and
+    gradients on that same piece."""
+    import copy
+
+    import torch.nn.functional as F
+
+    import cxgnncomp
+    from oracle import pyref
+    ptr, idx = citation
+    n, E = C2_N, idx.shape[0]
+    cxgnncomp.set_timers()
+    torch.manual_seed(11)
+    x = torch.randn(n, 128)
+    model = cxgnncomp.GCN(128, 256, 40, 3, 0.0, "CSR")
+    with torch.no_grad():
+        for conv in model.convs:
+            conv.normalize = normalize
+            conv.bias.normal_(0, 0.1)
+    ref = copy.deepcopy(model).double()
+    g = torch.randn(n, 40, dtype=torch.float64) / 8
+
+    announce("GCN 128-256-256-40 on the full graph, normalize=%s" % normalize)
+    dev_model = model.cuda()
+    patterns = []
+    hooks = [bn.register_forward_hook(lambda mod, inp, out: patterns.append((out > 0).cpu())) for bn in dev_model.bns]
+    b = cxgnncomp.Batch(x.cuda().requires_grad_(True), ptr.cuda(), idx.cuda(), torch.tensor([n, n, n, n]))
+    got = dev_model(b)
+    got.backward(g.float().cuda())
+    torch.cuda.synchronize()
+    for h in hooks:
+        h.remove()
+    assert len(patterns) == 2
+
+    val = pyref.gcn_norm(ptr, idx).double() if normalize else torch.ones(E, dtype=torch.float64)
+    x64 = x.double().requires_grad_(True)
+    h = x64
+    for i, conv in enumerate(ref.convs):
+        before = conv.in_channels > conv.out_channels
+        t = conv.lin(h) if before else h
+        t = pyref.spmm_torch(t, ptr, idx, n, val)
+        if not before:
+            t = conv.lin(t)
+        h = t + conv.bias
+        if i < 2:
+            bn = ref.bns[i]
+            h = F.batch_norm(h, None, None, bn.weight, bn.bias, True, 0.0, bn.eps)
+            differ = (h.detach() > 0) != patterns[i]
+            assert int(differ.sum()) < 1000
+            # within fp32 rounding of zero, at the scale of the unit's own row (hub rows sum 13 k terms)
+            near = 2e-5 * h.detach().abs().amax(dim=1, keepdim=True).clamp(min=1.0)
+            assert bool((h.detach().abs() < near)[differ].all())
+            h = h * patterns[i].double()
+    want = h.log_softmax(-1)
+    want.backward(g)
+    assert got.shape == (n, 40)
+    # log_softmax subtracts numbers of the row's raw scale (hub rows of the sum aggregation reach
+    # several hundred): the absolute part of the tolerance follows that scale, 2e-6 of it (a few
+    # dozen fp32 roundings), on top of 2e-5 for rows of O(1)
+    raw = h.detach().abs().amax(dim=1, keepdim=True).clamp(min=1.0).numpy()
+    assert_close(got.detach().cpu().numpy() / raw, want.detach().numpy() / raw, 2e-4, 2e-6 + 2e-5 / raw.max(),
+                 "GCN logits at the rows' raw scale")
+    assert_close(got.detach().cpu().numpy(), want.detach().numpy(), 2e-4, 2e-5 + 2e-6 * float(raw.max()), "GCN logits")
+    sc = float(x64.grad.abs().max())
+    assert_close(b.x.grad.cpu().numpy() / sc, x64.grad.numpy() / sc, 2e-4, 4e-5, "GCN grad x")
+    # ... and every row at its own scale, in norm (rows far from the hubs carry tiny gradients)
+    row_err = (b.x.grad.cpu().double() - x64.grad).norm(dim=1)
+    row_ref = x64.grad.norm(dim=1)
+    assert bool((row_err <= 1e-3 * row_ref + 1e-7 * sc).all()), float((row_err / (row_ref + 1e-7 * sc)).max())
+    for (name, p_got), (_, p_ref) in zip(dev_model.named_parameters(), ref.named_parameters()):
+        assert p_got.grad is not None, name
+        if name in ("convs.0.bias", "convs.1.bias"):
+            # A bias in front of a training-mode BatchNorm has gradient zero (the layer subtracts the
+            # column mean): both sides hold only the rounding residue of a sum that cancels, which at
+            # the sum aggregation's gradient scale (hub rows multiply it by 10^4 per layer) is large
+            # in absolute terms and means nothing.
+            continue
+        scw = float(p_ref.grad.abs().max())
+        assert_close(p_got.grad.cpu().numpy() / scw, p_ref.grad.numpy() / scw, 2e-4, 4e-5, "GCN grad " + name)
 
 
 # --------------------------------------------------------------------------- #

@@ -3,7 +3,9 @@
 Tolerances: SDDMM is an fp32 dot product (1e-4 rel / 1e-5 abs at O(1) scale).
 The softmax uses the hardware exponential (__expf, as the reference does,
 src/cpp/src/edge_softmax.cu:25); its outputs lie in [0,1] and are compared at
-2e-4 relative / 1e-6 absolute against the double-precision oracle."""
+2e-4 relative / 1e-6 absolute against the double-precision oracle.  The softmax
+backward is plain fp32 arithmetic on the saved output: 1e-4 / 1e-5, the bar of
+every fp32 aggregation, against the oracle's backward of that same output."""
 import numpy as np
 import pytest
 import torch
@@ -13,6 +15,7 @@ from conftest import announce, assert_close
 from test_spmm_gpu import ATOL, RTOL, _graph
 
 pytestmark = pytest.mark.gpu
+SM_BWD_RTOL, SM_BWD_ATOL = 1e-4, 1e-5
 
 
 def _np(t):
@@ -89,10 +92,12 @@ def test_edge_softmax_forward_backward(kind, heads):
     ref, mask = oracle.edge_softmax_fwd(p, i, att_dst.numpy(), att_src.numpy(), E, slope)
     assert out.shape == (E, heads)
     assert_close(_np(out), ref, 2e-4, 1e-6, "softmax fwd")
-    # backward of the oracle on the oracle's own forward output
-    gd, gs = oracle.edge_softmax_bwd(p, i, g.numpy(), mask, ref, n, n, slope)
-    assert_close(_np(ad.grad), gd, 1e-3, 2e-5, "grad att_dst")
-    assert_close(_np(asr.grad), gs, 1e-3, 2e-5, "grad att_src")
+    # The backward consumes the saved forward output (edge_softmax.cu:134-177), so the oracle's
+    # backward is run on the kernel's own output: the hardware exp of the forward (2e-4) then does
+    # not enter, and both gradients are held to the fp32 aggregation bar, 1e-4 / 1e-5.
+    gd, gs = oracle.edge_softmax_bwd(p, i, g.numpy(), mask, _np(out), n, n, slope)
+    assert_close(_np(ad.grad), gd, SM_BWD_RTOL, SM_BWD_ATOL, "grad att_dst")
+    assert_close(_np(asr.grad), gs, SM_BWD_RTOL, SM_BWD_ATOL, "grad att_src")
     # rows sum to one
     if E:
         sums = oracle.spmv(p, np.arange(E), _np(out)[:, 0], n)
@@ -148,9 +153,9 @@ def test_edge_softmax_degrees_at_the_step_boundaries(heads):
     p, i = ptr.numpy(), idx.numpy()
     ref, mask = oracle.edge_softmax_fwd(p, i, att_dst.numpy(), att_src.numpy(), E, slope)
     assert_close(_np(out), ref, 2e-4, 1e-6, "softmax fwd")
-    gd, gs = oracle.edge_softmax_bwd(p, i, g.numpy(), mask, ref, n, n, slope)
-    assert_close(_np(ad.grad), gd, 1e-3, 2e-5, "grad att_dst")
-    assert_close(_np(asr.grad), gs, 1e-3, 2e-5, "grad att_src")
+    gd, gs = oracle.edge_softmax_bwd(p, i, g.numpy(), mask, _np(out), n, n, slope)
+    assert_close(_np(ad.grad), gd, SM_BWD_RTOL, SM_BWD_ATOL, "grad att_dst")
+    assert_close(_np(asr.grad), gs, SM_BWD_RTOL, SM_BWD_ATOL, "grad att_src")
     # a second run gives the same bits
     ad2 = att_dst.cuda().requires_grad_(True)
     out2 = B.edge_attention(ptr=ptr.cuda(), idx=idx.cuda(), att_dst=ad2, att_src=asr.detach(), num_edge=E, relu_l=slope)
