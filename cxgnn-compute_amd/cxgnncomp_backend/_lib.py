@@ -41,6 +41,8 @@ SIGNATURES = {
     "cxg_typed_gemm_epilogue_f32": (_I32, [_P, _I64, _P, _P, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I32, _I32, _I32,
                                             _U32, _P]),
     "cxg_typed_gemm_bf16": (_I32, [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I32, _I32, _I32, _U32, _P]),
+    "cxg_typed_gemm_wide_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "cxg_typed_gemm_wide_f32": (_I32, [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I32, _I32, _I32, _U32, _P, _SZ, _P]),
     "cxg_rel_segment_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "cxg_rel_segment_i64": (_I32, [_P, _I64, _I32, _P, _P, _P, _SZ, _P]),
     "cxg_rel_segment_i32": (_I32, [_P, _I64, _I32, _P, _P, _P, _SZ, _P]),

@@ -110,6 +110,13 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
             st = lib.cxg_typed_gemm_bf16(a16.data_ptr(), K, wt16.data_ptr(), out.data_ptr(), N,
                                          _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
                                          m_rows, K, N, R, flags, stream)
+        elif _takes_wide_form(K, N, flags):
+            # wide operands: the tiled kernel with both operand tiles in LDS (W split into the workspace)
+            _req(w, "weights", torch.float32, 3)
+            ws = _workspace(lib.cxg_typed_gemm_wide_workspace_bytes(K, N, R), a.device)
+            st = lib.cxg_typed_gemm_wide_f32(a.data_ptr(), K, w.data_ptr(), out.data_ptr(), N,
+                                             _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
+                                             m_rows, K, N, R, flags, ws.data_ptr(), ws.numel(), stream)
         else:
             _req(w, "weights", torch.float32, 3)
             st = lib.cxg_typed_gemm_f32(a.data_ptr(), K, w.data_ptr(), out.data_ptr(), N,
@@ -117,6 +124,14 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
                                         m_rows, K, N, R, flags, stream)
     _lib.check(st)
     return out
+
+
+def _takes_wide_form(K, N, flags):
+    """The fp16 split arithmetic on shapes the register-resident kernel does not take: K above
+    256, and 160 <= K <= 256 where that kernel's 256 x 128 tile would be mostly empty."""
+    if not (flags & GEMM_SPLIT_F16X3) or K % 4 or K < 160:
+        return False
+    return K > 256 or not (K >= 176 and N >= 96)
 
 
 # --------------------------------------------------------------------------- #

@@ -331,6 +331,27 @@ int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, flo
                         unsigned flags, void* stream);
 
 /*
+ * The same contraction for wide operands (K >= 160, any N; K and lda multiples of 4, A
+ * 16-byte aligned; otherwise CXG_ERR_UNSUPPORTED): a tiled GEMM -- block tile 128 rows x 256
+ * columns, K walked in chunks of 32 with both operand tiles in LDS -- in the
+ * CXG_GEMM_SPLIT_F16X3 arithmetic (three fp16 partial products of power-of-two-scaled
+ * operands, 2^-21 per product, fp32 accumulation; the flag may be passed or left out).  W is
+ * split once per call into the workspace (its two fp16 parts per relation, column tile and
+ * k-chunk, and the columns' inverse scales).  A row's scale follows the largest magnitude
+ * met so far along K with three bits of headroom; when a later value outgrows it the sums so
+ * far are multiplied by the power-of-two ratio, so the result does not depend on where along
+ * K the large values sit.  flags: CXG_GEMM_ACCUMULATE, CXG_GEMM_ATOMIC as above.  This is
+ * the shape class the reference benchmarks its typed_matmul on
+ * (cxgnncomp/codegen/triton_typed_matmul.py:752-860 with K = N = 512,
+ * test/ae/E3_ablation/test-batch.py:27-52).
+ */
+size_t cxg_typed_gemm_wide_workspace_bytes(int K, int N, int R);
+int cxg_typed_gemm_wide_f32(const float* a, int64_t lda, const float* w, float* c, int64_t ldc,
+                            const int64_t* src_idx, const int64_t* dst_idx, const int64_t* seg_ptr,
+                            int64_t M, int K, int N, int R, unsigned flags, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
+/*
  * Weight gradient of the typed GEMM: gw[r] (K x N, fp32, overwritten) = sum over
  * the rows i of segment r of A[src(i), :]^T (x) G[dst(i), :]; relations without
  * rows give zeros.  A is [*, K] (row stride lda), G is [*, N] (row stride ldg);
