@@ -58,6 +58,7 @@ constexpr int kWBlockHalfs = 2 * kWN * kWK;   // fp16 elements of one (relation,
 constexpr int kWMaxTiles = 8;              // row tiles per block
 constexpr int kWBlockBytes = kWBlockHalfs * 2;                       // 32 KB
 constexpr int kWAsBytes = 2 * 2 * kWM * kWP * 2;                     // both stages, both parts of the A tile
+constexpr int kWCP = 136;                  // floats per row of a consumer wave's store staging area
 
 struct WideArgs {
   const float* a;
@@ -190,6 +191,9 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
       for (int gc = 0; gc < total; ++gc) __syncthreads();
       return;
     }
+    // this wave's staging area for stores, 8 rows x (128 + 8) floats (rows 4 apart land 32 banks apart)
+    float (*Cw)[kWCP] = reinterpret_cast<float (*)[kWCP]>(reinterpret_cast<unsigned char*>(s_flag) + 16) + (size_t)wave * 8;
+    const bool wide_store = !g.atomic && n0 + wn * 128 + 128 <= N && (g.ldc & 3) == 0 && ((uintptr_t)g.c & 15) == 0;
     float invw[4];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt)
@@ -288,6 +292,33 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
           const int rl0 = wm * 64 + mt * 32 + q * 8 + (lane >> 5) * 4;
           const float4 ri = *reinterpret_cast<const float4*>(&s_inv[t & 1][rl0]);
           const float rinv[4] = {ri.x, ri.y, ri.z, ri.w};
+          if (wide_store) {
+            // Eight rows x this wave's 128 columns go through the wave's own LDS area and leave
+            // as 16 bytes per lane, 512 contiguous bytes per row: a quarter of the store
+            // instructions of 4-byte stores from the accumulators (128 per tile and wave, which
+            // cost the K = N = 512 product 1.5 of its 5.1 ms).  LDS operations of one wave
+            // execute in order, so the area needs no barrier.
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                Cw[(lane >> 5) * 4 + j][nt * 32 + (lane & 31)] = acc[nt][mt][q * 4 + j] * (rinv[j] * invw[nt]);
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+              const int rl = it * 2 + (lane >> 5);
+              const float4 v = *reinterpret_cast<const float4*>(&Cw[rl][(lane & 31) * 4]);
+              const int64_t d = drow[wm * 64 + mt * 32 + q * 8 + rl];
+              if (d < 0) continue;
+              float4* const p = reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wn * 128 + (lane & 31) * 4);
+              if (g.accumulate) {
+                const float4 o = *p;
+                *p = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
+              } else {
+                *p = v;
+              }
+            }
+            continue;
+          }
           int64_t d[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) d[j] = drow[rl0 + j];
@@ -504,7 +535,8 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
   __builtin_amdgcn_s_waitcnt(0x0F70);        // nothing of this wave is on its way into LDS when it ends
 }
 
-constexpr size_t kWideLds = kWAsBytes + 3 * kWBlockBytes + 4 * kWM * 4 + 4 * kWM * 8 + 16;
+constexpr size_t kWideLds = kWAsBytes + 3 * kWBlockBytes + 4 * kWM * 4 + 4 * kWM * 8 + 16 + 4 * 8 * kWCP * 4;
+static_assert(kWideLds <= 160 * 1024, "LDS of a CU");
 
 }  // namespace
 }  // namespace cxg
