@@ -267,24 +267,49 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
               }
             }
         }
-        // (the scheduling fences keep the LDS reads of the next k-step in front of this step's
-        // matrix instructions; left alone, the compiler sinks each read to just before its first
-        // use and the matrix pipe waits for an LDS round trip per operand)
+        // (the scheduling groups put the LDS reads of the next k-step between the first matrix
+        // instructions of this step; left alone, the compiler sinks each read to just before its
+        // first use and the matrix pipe waits for an LDS round trip per operand)
         read_ops(ya, yb, st, wst, 1);
-        __builtin_amdgcn_sched_barrier(0);
         mfmas(xa, xb);
+#pragma unroll
+        for (int i = 0; i < 12; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 12, 0);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();                     // chunk gc + 1 is staged; chunk gc has been read
         flag = s_flag[st ^ 1];
         wst = wst == 2 ? 0 : wst + 1;
         read_ops(xa, xb, st ^ 1, wst, 0);
-        __builtin_amdgcn_sched_barrier(0);
         mfmas(ya, yb);
+#pragma unroll
+        for (int i = 0; i < 13; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 11, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
       // undo the scales and store: accumulator element i of (nt, mt) is row
       // wm*64 + mt*32 + (i>>2)*8 + (lane>>5)*4 + (i&3), column n0 + wn*128 + nt*32 + (lane&31)
       const int64_t* drow = s_dst[t & 1];
+      float4 pv[4];                          // the group of rows read back last, not yet stored
+      int64_t pd[4];
+      auto store_group = [&](const float4 (&v)[4], const int64_t (&d)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          if (d[it] < 0) continue;
+          float4* const p = reinterpret_cast<float4*>(g.c + d[it] * g.ldc + n0 + wn * 128 + (lane & 31) * 4);
+          if (g.accumulate) {
+            const float4 o = *p;
+            *p = make_float4(o.x + v[it].x, o.y + v[it].y, o.z + v[it].z, o.w + v[it].w);
+          } else {
+            stream_store(reinterpret_cast<float*>(p), v[it]);   // written once: not kept in the L2, where W and the A rows live
+          }
+        }
+      };
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -297,26 +322,27 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
             // as 16 bytes per lane, 512 contiguous bytes per row: a quarter of the store
             // instructions of 4-byte stores from the accumulators (128 per tile and wave, which
             // cost the K = N = 512 product 1.5 of its 5.1 ms).  LDS operations of one wave
-            // execute in order, so the area needs no barrier.
+            // execute in order, so the area needs no barrier, and the rows of a group are stored
+            // only after the next group has been written and read back: its LDS round trip runs
+            // while the stores are issued (a group at a time, every store behind two LDS round
+            // trips of its own, took 1,200 cycles per group).
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
               for (int j = 0; j < 4; ++j)
                 Cw[(lane >> 5) * 4 + j][nt * 32 + (lane & 31)] = acc[nt][mt][q * 4 + j] * (rinv[j] * invw[nt]);
+            float4 cv[4];
+            int64_t cd[4];
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
               const int rl = it * 2 + (lane >> 5);
-              const float4 v = *reinterpret_cast<const float4*>(&Cw[rl][(lane & 31) * 4]);
-              const int64_t d = drow[wm * 64 + mt * 32 + q * 8 + rl];
-              if (d < 0) continue;
-              float4* const p = reinterpret_cast<float4*>(g.c + d * g.ldc + n0 + wn * 128 + (lane & 31) * 4);
-              if (g.accumulate) {
-                const float4 o = *p;
-                *p = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
-              } else {
-                *p = v;
-              }
+              cv[it] = *reinterpret_cast<const float4*>(&Cw[rl][(lane & 31) * 4]);
+              cd[it] = drow[wm * 64 + mt * 32 + q * 8 + rl];
             }
+            if (mt + q > 0) store_group(pv, pd);
+#pragma unroll
+            for (int it = 0; it < 4; ++it) { pv[it] = cv[it]; pd[it] = cd[it]; }
+            if (mt == 1 && q == 3) store_group(pv, pd);
             continue;
           }
           int64_t d[4];
@@ -498,17 +524,17 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
   stage(a0);
   dma_w();                                   // W of chunk 1
   gload(a0);                                 // chunk 2
-  // A wave's memory requests complete in order: the W block of chunk 0 has arrived when at
-  // most the 4 + 8 + 4 requests issued after it are outstanding.  vmcnt(16), no wait on the
-  // other counters:
+  // the W block of chunk 0 has arrived when at most the 4 + 8 + 4 requests issued after it are
+  // outstanding.  vmcnt(16), no wait on the other counters:
   __builtin_amdgcn_s_waitcnt(0x4F70);
   __syncthreads();                           // P
   // Iteration gc (between the barriers of chunks gc-1 and gc): split chunk gc+1 of A into its
   // LDS half, send chunk gc+2 of W on its way into the W area that chunk gc-1 has left, and
-  // request chunk gc+3 of A.  Two iterations per trip so that each register set keeps its
-  // role.  The row tables of tile t+1 are written during chunk 1 of tile t: the consumers are
-  // then done with the tables of tile t-1 (same slots), and the loads of tile t+1 start at the
-  // earliest in chunk NC-3 >= 2.
+  // request chunk gc+3 of A.  (With the W block requested first it would have half an iteration
+  // more to arrive; measured, that order is slower, 4.43 against 4.22 ms at K = N = 512.)  Two
+  // iterations per trip so that each register set keeps its role.  The row tables of tile t+1
+  // are written during chunk 1 of tile t: the consumers are then done with the tables of tile
+  // t-1 (same slots), and the loads of tile t+1 start at the earliest in chunk NC-3 >= 2.
   int it_c = 0, it_t = 0;                    // (tile, chunk) of iteration gc
   auto tables_due = [&]() __attribute__((always_inline)) {
     if (it_c == 1) fill_tables(it_t + 1);
