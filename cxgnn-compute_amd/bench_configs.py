@@ -578,6 +578,60 @@ def c5(iters):
         cpu_spmm("c5", ptr, idx, n_src, 128, nn[2])
 
 
+def e3(iters):
+    """The one typed-linear shape the reference stores timings for (test/ae/E3_ablation/test-batch.py:27-52,
+    output kept in process-batch-data.ipynb): the 169,343-node / 2,332,486-edge citation graph, 512 -> 512,
+    7 random relations; source -> edge typed linear.  The reference's stored numbers, hardware unstated:
+    Triton typed_matmul 18.76 - 27.92 ms, per-edge kernel typed_linear_s2e 417.36 ms."""
+    import cxgnncomp as cxgc
+    import cxgnncomp_backend as B
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _typed
+    ptr, idx = S.powerlaw_directed_symmetrised(169343, 1166243, seed=0, device="cuda")
+    n, E, K, R = ptr.shape[0] - 1, idx.shape[0], 512, 7
+    torch.manual_seed(0)
+    x = torch.randn(n, K, device="cuda")
+    rel = torch.randint(0, R, (E,), dtype=torch.int32, device="cuda")
+    rel64 = rel.long()
+    w = torch.randn(R, K, K, device="cuda")
+    flops = 2.0 * E * K * K
+    nbytes = E * (4 * K + 4 * K + 8) + 4 * R * K * K
+    pre = cxgc.TypedLinearS2EOP.preprocess(w, rel64, idx, thres=256)
+    report("e3", "TypedLinearS2EOP forward (typed_matmul, source -> edge), E=2,332,486 K=N=512 R=7",
+           timeit(lambda: cxgc.TypedLinearS2EOP.apply(x, w, rel64, idx, pre), iters), nbytes, flops,
+           note="reference's stored Triton typed_matmul: 18.76-27.92 ms (hardware unstated)")
+    out = torch.zeros(E, K, device="cuda")
+    report("e3", "typed_linear_s2e (accumulates into the caller's rows)",
+           timeit(lambda: B.typed_linear_s2e(x, w, out, idx, rel, 32), iters), nbytes + 4 * E * K, flops,
+           note="reference's stored per-edge kernel: 417.36 ms (hardware unstated)")
+    del out
+    perm, seg = _typed.rel_segment(rel, R)
+    xe = torch.randn(E, K, device="cuda")
+    oe = torch.empty(E, K, device="cuda")
+    report("e3", "typed GEMM over relation-sorted rows, plain (E x 512 x 512), 3 scaled fp16 products",
+           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="split_f16"), iters), nbytes, flops)
+    report("e3", "same, fp32 MFMA",
+           timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="fp32"), iters), nbytes, flops, MFMA_F32)
+    src = idx[perm].contiguous()
+    report("e3", "typed GEMM with gathered source rows, relation-sorted output",
+           timeit(lambda: _typed.typed_gemm(x, w, seg, E, src_idx=src, out=oe, precision="split_f16"), iters),
+           nbytes, flops)
+    g = torch.randn(E, K, device="cuda")
+    report("e3", "weight gradient over the edge rows (gathered sources), [7, 512, 512]",
+           timeit(lambda: _typed.typed_gemm_wgrad(x, g, seg, E, R, src_idx=src), iters), nbytes, flops)
+    global _last_spread
+    t_mm = timeit(lambda: torch.mm(xe, w[0], out=oe), iters)
+    report("e3", "torch.mm [E,512]x[512,512] (library fp32 GEMM of the same flops, one relation, for scale)",
+           t_mm, nbytes, flops, MFMA_F32)
+    xg = x.clone().requires_grad_(True)
+    wg = w.clone().requires_grad_(True)
+
+    def step():
+        xg.grad = wg.grad = None
+        cxgc.TypedLinearS2EOP.apply(xg, wg, rel64, idx, pre).backward(g)
+    report("e3", "TypedLinearS2EOP forward + backward (grad x and grad W)", timeit(step, iters), 3 * nbytes, 3 * flops)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
@@ -591,7 +645,7 @@ def main():
     global COLD, CPU_BASELINE, C5_STEPS, C5_FRESH
     COLD, CPU_BASELINE, C5_STEPS, C5_FRESH = args.cold, args.cpu_baseline, args.c5_steps, args.c5_fresh
     sys.path.insert(0, os.path.dirname(HERE))
-    table = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5}
+    table = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5, "e3": e3}
     for name in args.configs.split(","):
         table[name](args.iters)
         torch.cuda.empty_cache()

@@ -110,7 +110,7 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
             st = lib.cxg_typed_gemm_bf16(a16.data_ptr(), K, wt16.data_ptr(), out.data_ptr(), N,
                                          _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
                                          m_rows, K, N, R, flags, stream)
-        elif _takes_wide_form(K, N, flags):
+        elif _takes_wide_form(K, N, flags, src_idx is not None):
             # wide operands: the tiled kernel with both operand tiles in LDS (W split into the workspace)
             _req(w, "weights", torch.float32, 3)
             ws = _workspace(lib.cxg_typed_gemm_wide_workspace_bytes(K, N, R), a.device)
@@ -126,12 +126,14 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
     return out
 
 
-def _takes_wide_form(K, N, flags):
-    """The fp16 split arithmetic on shapes the register-resident kernel does not take: K above
-    256, and 160 <= K <= 256 where that kernel's 256 x 128 tile would be mostly empty."""
+def _takes_wide_form(K, N, flags, gathered=False):
+    """The fp16 split arithmetic on the tiled kernel: K above 256 (the register-resident kernel
+    holds at most 256 rows of W), and 160 <= K <= 256 where it measures faster -- more than one
+    128-column tile (5 M x 256 x 256: 2.8 against 3.9 ms), gathered rows (7.3 M x 256 x 128: 3.0
+    against 3.6 ms), or a 256 x 128 register tile that would be mostly empty."""
     if not (flags & GEMM_SPLIT_F16X3) or K % 4 or K < 160:
         return False
-    return K > 256 or not (K >= 176 and N >= 96)
+    return K > 256 or gathered or N > 128 or not (K >= 176 and N >= 96)
 
 
 # --------------------------------------------------------------------------- #

@@ -357,6 +357,50 @@ def test_c2_gcn_model_full_size(citation, normalize):
         assert_close(p_got.grad.cpu().numpy() / scw, p_ref.grad.numpy() / scw, 2e-4, 4e-5, "GCN grad " + name)
 
 
+def test_c2_typed_linear_512_full_size(citation):
+    """The shape of the reference's own typed-linear benchmark (test/ae/E3_ablation/test-batch.py:27-52):
+    the 2,332,486 edges of this graph, 512 -> 512, 7 random relations, source -> edge.  TypedLinearS2EOP
+    forward on every edge row against float64 (one relation at a time on the device), typed_linear_s2e
+    accumulating onto a pre-filled buffer, grad_x on every source row and grad_W on every element
+    against float64; 1e-4 / 1e-5 at the outputs' scale."""
+    import cxgnncomp
+    import cxgnncomp_backend as B
+    ptr, idx = citation
+    n, E, K, R = C2_N, idx.shape[0], 512, 7
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(n, K, device="cuda", generator=gen) / K ** 0.5
+    w = torch.randn(R, K, K, device="cuda", generator=gen)
+    rel = torch.randint(0, R, (E,), device="cuda", generator=gen)
+    g = torch.randn(E, K, device="cuda", generator=gen) / 16
+    ic = idx.cuda()
+    want = torch.empty(E, K, dtype=torch.float64, device="cuda")
+    want_gx = torch.zeros(n, K, dtype=torch.float64, device="cuda")
+    want_gw = torch.zeros(R, K, K, dtype=torch.float64, device="cuda")
+    for r in range(R):
+        e = torch.nonzero(rel == r).squeeze(1)
+        for chunk in torch.split(e, 1 << 19):
+            xs, gd = x[ic[chunk]].double(), g[chunk].double()
+            want[chunk] = xs @ w[r].double()
+            want_gx.index_add_(0, ic[chunk], gd @ w[r].double().t())
+            want_gw[r] += xs.t() @ gd
+    xg = x.clone().requires_grad_(True)
+    wg = w.clone().requires_grad_(True)
+    announce("TypedLinearS2EOP fwd+bwd at E=2,332,486, 512 -> 512, 7 relations")
+    pre = cxgnncomp.TypedLinearS2EOP.preprocess(wg, rel, ic, thres=256)
+    out = cxgnncomp.TypedLinearS2EOP.apply(xg, wg, rel, ic, pre)
+    out.backward(g)
+    torch.cuda.synchronize()
+    assert out.shape == (E, K)
+    _close_scaled(out.detach(), want, 1e-4, 1e-5, "typed linear forward, every edge row")
+    _close_scaled(xg.grad, want_gx, 1e-4, 1e-5, "typed linear grad x")
+    _close_scaled(wg.grad, want_gw, 1e-4, 1e-5, "typed linear grad W")
+    announce("typed_linear_s2e accumulating at the same size")
+    acc = torch.full((E, K), 0.25, device="cuda")
+    B.typed_linear_s2e(x, w, acc, ic, rel.int(), 32)
+    torch.cuda.synchronize()
+    _close_scaled(acc, want + 0.25, 1e-4, 1e-5, "typed_linear_s2e")
+
+
 # --------------------------------------------------------------------------- #
 # RGCN configuration at its stated size: 1,000,000 nodes / 20,000,000 edges / 16 relations
 # --------------------------------------------------------------------------- #
