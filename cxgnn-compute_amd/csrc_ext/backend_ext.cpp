@@ -25,6 +25,7 @@
 #include <list>
 #include <map>
 #include <memory>
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <tuple>
@@ -273,7 +274,8 @@ struct TransposedGraph {
   Tensor ptr_t, idx_t, perm;        // rows = source nodes, idx_t = destination ids, perm = original edge position
   int64_t n_edges = 0, n_src = 0, n_dst = 0;
   Tensor keep_ptr, keep_idx;        // the tensors the key was made from stay alive while cached
-  OptTensor inv_deg_t, rows32;      // filled on first use
+  OptTensor inv_deg_t, rows32;      // filled on first use, under fill_mu (a cached graph is shared between threads)
+  std::mutex fill_mu;
 };
 using GraphPtr = std::shared_ptr<TransposedGraph>;
 
@@ -290,8 +292,16 @@ struct LayerHint {
   c10::weak_intrusive_ptr<c10::TensorImpl> ptr, idx;   // a hint must not outlive its tensors
 };
 
+// Edge counts of row prefixes that the caller knows (a sampled batch carries num_edge_in_layer):
+// with them no transposition has to read ptr[n_rows] back from the device.
+struct EdgeCounts {
+  std::vector<std::pair<int64_t, int64_t>> rows_edges;
+  c10::weak_intrusive_ptr<c10::TensorImpl> ptr, idx;
+};
+
 struct GraphCache {
   std::mutex mu;
+  std::list<std::pair<GraphId, EdgeCounts>> edge_counts;
   size_t capacity = 8;
   std::list<std::pair<GraphKey, GraphPtr>> lru;                      // most recently used last
   std::map<GraphKey, std::list<std::pair<GraphKey, GraphPtr>>::iterator> index;
@@ -317,6 +327,22 @@ struct GraphCache {
     lru.clear();
     index.clear();
     hints.clear();
+    edge_counts.clear();
+  }
+  // number of edges of rows [0, n_rows) if the caller has announced it, else -1
+  int64_t known_edges(const GraphId& gid, const Tensor& ptr, const Tensor& idx, int64_t n_rows) {
+    for (auto it = edge_counts.begin(); it != edge_counts.end(); ++it) {
+      if (it->first != gid) continue;
+      auto p = it->second.ptr.lock(), i = it->second.idx.lock();
+      if (p.get() != ptr.unsafeGetTensorImpl() || i.get() != idx.unsafeGetTensorImpl()) {
+        edge_counts.erase(it);
+        return -1;
+      }
+      for (const auto& re : it->second.rows_edges)
+        if (re.first == n_rows) return re.second;
+      return -1;
+    }
+    return -1;
   }
   const LayerHint* hint(const GraphId& gid, const Tensor& ptr, const Tensor& idx) {
     for (auto it = hints.begin(); it != hints.end(); ++it) {
@@ -339,12 +365,20 @@ GraphCache& cache() {
   return *c;
 }
 
+std::atomic<int64_t> g_edge_count_readbacks{0};   // times a transposition had to fetch ptr[n_rows] from the device
+
 // Uncached transposition by a stable sort: (ptr_t, idx_t, perm, n_edges).
-std::tuple<Tensor, Tensor, Tensor, int64_t> csr_transpose(const Tensor& ptr, const Tensor& idx, int64_t n_rows, int64_t n_src) {
+// `known_edges` >= 0: the caller vouches for ptr[0] == 0 and ptr[n_rows] == known_edges, and nothing is read back.
+std::tuple<Tensor, Tensor, Tensor, int64_t> csr_transpose(const Tensor& ptr, const Tensor& idx, int64_t n_rows, int64_t n_src,
+                                                          int64_t known_edges = -1) {
   check_graph(ptr, idx, n_rows);
-  const Tensor ends = torch::stack({ptr[0], ptr[n_rows]}).cpu();          // one read-back for both
-  const int64_t first = ends[0].item<int64_t>(), n_edges = ends[1].item<int64_t>();
-  if (first != 0) bad("ptr[0] must be 0");
+  int64_t n_edges = known_edges;
+  if (n_edges < 0) {
+    ++g_edge_count_readbacks;
+    const Tensor ends = torch::stack({ptr[0], ptr[n_rows]}).cpu();          // one read-back for both
+    n_edges = ends[1].item<int64_t>();
+    if (ends[0].item<int64_t>() != 0) bad("ptr[0] must be 0");
+  }
   if (n_edges > idx.size(0))
     bad(fmt("ptr[num_node]=%lld exceeds idx length %lld", (long long)n_edges, (long long)idx.size(0)));
   Tensor ptr_t = torch::empty({n_src + 1}, ptr.options());
@@ -360,11 +394,13 @@ std::tuple<Tensor, Tensor, Tensor, int64_t> csr_transpose(const Tensor& ptr, con
 
 // The first n_rows rows of the graph `whole` was built from, as a stable compaction of its entries.
 std::tuple<Tensor, Tensor, Tensor, int64_t> csr_transpose_prefix(const TransposedGraph& whole, const Tensor& ptr,
-                                                                 int64_t n_rows, int64_t n_src) {
+                                                                 int64_t n_rows, int64_t n_src, int64_t known_edges = -1) {
   req(ptr, "ptr", at::kLong, {1});
   if (n_rows < 0 || n_rows + 1 > ptr.size(0)) bad("num_node does not fit ptr");
   if (n_src + 1 > whole.ptr_t.size(0)) bad("the whole graph has fewer sources than the prefix");
-  const int64_t n_edges = ptr[n_rows].item<int64_t>();
+  if (known_edges < 0) ++g_edge_count_readbacks;
+  const int64_t n_edges = known_edges >= 0 ? known_edges : ptr[n_rows].item<int64_t>();
+  if (n_edges > whole.n_edges) bad("the prefix has more edges than the whole graph");
   Tensor ptr_t = torch::empty({n_src + 1}, ptr.options());
   Tensor idx_t = torch::empty({n_edges}, ptr.options());
   Tensor perm = torch::empty({n_edges}, ptr.options());
@@ -393,14 +429,38 @@ void note_layer(const Tensor& ptr, const Tensor& idx, int64_t n_rows, int64_t n_
   while (c.hints.size() > 64) c.hints.pop_front();
 }
 
+// The caller knows how many edges the first rows[k] rows hold (Batch.num_node_in_layer /
+// num_edge_in_layer of a sampled batch, cxgnncomp/batch.py): transpositions of those row prefixes
+// then size their outputs from it instead of reading ptr[rows[k]] back, which made the host wait
+// for the GPU once per layer in the first backward pass of every new batch.
+void note_edge_counts(const Tensor& ptr, const Tensor& idx, const std::vector<int64_t>& rows,
+                      const std::vector<int64_t>& edges) {
+  if (rows.size() != edges.size()) bad("note_edge_counts: one edge count per row count");
+  std::vector<std::pair<int64_t, int64_t>> rows_edges;
+  for (size_t k = 0; k < rows.size(); ++k) {
+    if (rows[k] < 0 || rows[k] + 1 > ptr.size(0) || edges[k] < 0 || edges[k] > idx.size(0))
+      bad("note_edge_counts: counts do not fit ptr / idx");
+    rows_edges.emplace_back(rows[k], edges[k]);
+  }
+  EdgeCounts ec{std::move(rows_edges), c10::weak_intrusive_ptr<c10::TensorImpl>(ptr.getIntrusivePtr()),
+                c10::weak_intrusive_ptr<c10::TensorImpl>(idx.getIntrusivePtr())};
+  GraphCache& c = cache();
+  std::lock_guard<std::mutex> lock(c.mu);
+  const GraphId gid = graph_id(ptr, idx);
+  c.edge_counts.remove_if([&](const std::pair<GraphId, EdgeCounts>& h) { return h.first == gid; });
+  c.edge_counts.emplace_back(gid, std::move(ec));
+  while (c.edge_counts.size() > 64) c.edge_counts.pop_front();
+}
+
 GraphPtr transposed(const Tensor& ptr, const Tensor& idx, int64_t n_rows, int64_t n_src) {
   GraphCache& c = cache();
   const GraphId gid = graph_id(ptr, idx);
   const GraphKey key(gid, n_rows, n_src);
-  int64_t whole_rows = -1, whole_src = -1;
+  int64_t whole_rows = -1, whole_src = -1, known = -1;
   {
     std::lock_guard<std::mutex> lock(c.mu);
     if (GraphPtr g = c.find(key)) return g;
+    known = c.known_edges(gid, ptr, idx, n_rows);
     const LayerHint* h = c.hint(gid, ptr, idx);
     if (h && ptr.is_cuda() && h->n_rows > n_rows && h->n_src >= n_src && c.capacity > 1) {
       whole_rows = h->n_rows;
@@ -410,11 +470,11 @@ GraphPtr transposed(const Tensor& ptr, const Tensor& idx, int64_t n_rows, int64_
   auto g = std::make_shared<TransposedGraph>();
   if (whole_rows >= 0) {
     GraphPtr whole = transposed(ptr, idx, whole_rows, whole_src);
-    std::tie(g->ptr_t, g->idx_t, g->perm, g->n_edges) = csr_transpose_prefix(*whole, ptr, n_rows, n_src);
+    std::tie(g->ptr_t, g->idx_t, g->perm, g->n_edges) = csr_transpose_prefix(*whole, ptr, n_rows, n_src, known);
     std::lock_guard<std::mutex> lock(c.mu);
     ++c.cuts;
   } else {
-    std::tie(g->ptr_t, g->idx_t, g->perm, g->n_edges) = csr_transpose(ptr, idx, n_rows, n_src);
+    std::tie(g->ptr_t, g->idx_t, g->perm, g->n_edges) = csr_transpose(ptr, idx, n_rows, n_src, known);
     std::lock_guard<std::mutex> lock(c.mu);
     ++c.sorts;
   }
@@ -429,6 +489,7 @@ GraphPtr transposed(const Tensor& ptr, const Tensor& idx, int64_t n_rows, int64_
 
 // 1/deg(dst) per edge, in transposed edge order (kept with the graph).
 Tensor inv_degree_transposed(TransposedGraph& g, const Tensor& ptr, int64_t n_rows) {
+  std::lock_guard<std::mutex> lock(g.fill_mu);
   if (!g.inv_deg_t.has_value()) {
     Tensor inv = edge_value_degree(ptr, n_rows, g.n_edges);
     g.inv_deg_t = g.n_edges > 0 ? inv.index({g.perm}) : inv;
@@ -438,6 +499,7 @@ Tensor inv_degree_transposed(TransposedGraph& g, const Tensor& ptr, int64_t n_ro
 
 // Row (source) id of every edge of a transposed graph as int32 (kept with the graph).
 Tensor rows32_transposed(TransposedGraph& g) {
+  std::lock_guard<std::mutex> lock(g.fill_mu);
   if (!g.rows32.has_value()) {
     Tensor rows = torch::empty({g.n_edges}, g.ptr_t.options().dtype(at::kInt));
     c10::DeviceGuard guard(g.ptr_t.device());
@@ -830,11 +892,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("edge_softmax_bwd", &edge_softmax_bwd);
   m.def("narrow_gather_sum", &narrow_gather_sum, py::arg("ptr"), py::arg("sel"), py::arg("inp"), py::arg("n_rows"),
         py::arg("rows32") = py::none());
-  m.def("csr_transpose", &csr_transpose);
+  m.def("csr_transpose", &csr_transpose, py::arg("ptr"), py::arg("idx"), py::arg("n_rows"), py::arg("n_src"),
+        py::arg("known_edges") = -1);
   m.def("csr_transpose_prefix",
-        [](const GraphPtr& whole, const Tensor& ptr, int64_t n_rows, int64_t n_src) {
-          return csr_transpose_prefix(*whole, ptr, n_rows, n_src);
-        });
+        [](const GraphPtr& whole, const Tensor& ptr, int64_t n_rows, int64_t n_src, int64_t known_edges) {
+          return csr_transpose_prefix(*whole, ptr, n_rows, n_src, known_edges);
+        }, py::arg("whole"), py::arg("ptr"), py::arg("n_rows"), py::arg("n_src"), py::arg("known_edges") = -1);
+  m.def("note_edge_counts", &note_edge_counts);
   m.def("transposed", &transposed);
   m.def("note_layer", &note_layer);
   m.def("inv_degree_transposed", [](const GraphPtr& g, const Tensor& ptr, int64_t n) { return inv_degree_transposed(*g, ptr, n); });
@@ -875,7 +939,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("graph_cache_stats", []() {
     GraphCache& c = cache();
     std::lock_guard<std::mutex> lock(c.mu);
-    return py::dict(py::arg("graphs") = c.lru.size(), py::arg("sorts") = c.sorts, py::arg("cuts") = c.cuts);
+    return py::dict(py::arg("graphs") = c.lru.size(), py::arg("sorts") = c.sorts, py::arg("cuts") = c.cuts,
+                    py::arg("readbacks") = g_edge_count_readbacks.load());
   });
 
   // the reference's names (binding.cpp:15-25, 37-41, 58-78)

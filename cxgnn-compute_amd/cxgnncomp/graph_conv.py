@@ -350,8 +350,12 @@ class SageLayerOP(torch.autograd.Function):
     def forward(ctx, x, w_l, b_l, w_r, ptr, idx, num_node):
         n = int(num_node) if int(num_node) != 0 else ptr.shape[0] - 1
         x = x.contiguous()
-        _ops.note_layer(ptr, idx, n, x.shape[0])
         mm_first = w_l.shape[1] > w_l.shape[0]
+        if ctx.needs_input_grad[0] or mm_first:
+            # only a layer whose backward will ask for the reversed graph announces itself: the
+            # first layer of a batch with frozen input features does not, and the reversed graphs
+            # of the others are then cut out of the largest layer that does need one
+            _ops.note_layer(ptr, idx, n, x.shape[0])
         aggr = None
         if mm_first:
             out = _ops.spmm(ptr, idx, _mm(x, w_l.t(), b_l), n, mean=True)

@@ -72,6 +72,13 @@ class GNN(torch.nn.Module):
 
     def forward_cxg(self, batch, skip_first=False):
         x = batch.x
+        sizes = (getattr(batch, "num_node_in_layer", None), getattr(batch, "num_edge_in_layer", None))
+        if (self.graph_type == "CSR_Layer" and batch.ptr.is_cuda and sizes[0] is not None and sizes[1] is not None
+                and not any(getattr(v, "is_cuda", False) for v in sizes) and len(sizes[1]) + 1 == len(sizes[0])):
+            # the batch knows its layers' edge counts: the backward passes then build the reversed
+            # graphs without waiting for the device to report ptr[num_node] per layer
+            cxgnncomp_backend._ops.note_edge_counts(batch.ptr, batch.idx, batch.num_node_in_layer[:-1],
+                                                    batch.num_edge_in_layer)
         last = self.num_layer - 1
         for i, conv in enumerate(self.convs):
             if not (skip_first and i == 0 and i != last):

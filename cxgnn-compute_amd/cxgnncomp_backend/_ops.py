@@ -148,6 +148,14 @@ def note_layer(ptr, idx, n_rows, n_src):
     _C.note_layer(ptr, idx, int(n_rows), int(n_src))
 
 
+def note_edge_counts(ptr, idx, rows, edges):
+    """Tell the transposed-graph cache how many edges the first rows[k] rows of (ptr, idx) hold
+    (``num_node_in_layer`` / ``num_edge_in_layer`` of a sampled batch): the reversed graphs of
+    those row prefixes are then built without reading ptr[rows[k]] back from the device.  The
+    counts are trusted."""
+    _C.note_edge_counts(ptr, idx, [int(r) for r in rows], [int(e) for e in edges])
+
+
 def transposed(ptr, idx, n_rows, n_src):
     """Cached TransposedGraph of (ptr[:n_rows+1], idx) with n_src source nodes (LRU of
     ``set_graph_cache_capacity`` graphs, kept in the compiled host layer)."""

@@ -99,7 +99,7 @@ def test_compiled_host_layer_exports_the_reference_names():
     assert B.SPMM_MULTIHEAD_SCHEDULE.Optimal == B.Optimal
     assert "schedule" in B.spmm_multihead.__doc__ and "block_size" in B.spmm_multihead.__doc__
     assert _C.lib_version() == B._lib_version()
-    assert set(_C.graph_cache_stats()) == {"graphs", "sorts", "cuts"}
+    assert set(_C.graph_cache_stats()) == {"graphs", "sorts", "cuts", "readbacks"}
 
 
 def test_missing_host_layer_fails_loudly(monkeypatch):

@@ -253,3 +253,67 @@ def test_transposed_graphs_of_nested_layers_are_cut_from_the_largest():
     pt, it, pm, n_e = _ops.csr_transpose_prefix(whole, p, 0, 5)
     assert n_e == 0 and it.numel() == 0 and not pt.any()
     _ops.clear_graph_cache()
+
+
+def test_known_edge_counts_spare_the_read_back():
+    """A sampled batch carries its layers' edge counts.  Announced with note_edge_counts, they size
+    the reversed graphs, so no transposition reads ptr[num_node] back from the device (the host
+    then never waits for the GPU while it enqueues the first backward pass of a new batch); the
+    graphs are the same bit for bit."""
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    ptr, idx, nn, ne = S.sampled_batch(num_seeds=300, fanouts=(7, 5, 3), id_space=200000, seed=11)
+    p, i = ptr.cuda(), idx.cuda()
+    want = {k: _ops.csr_transpose(p, i, nn[k], nn[k + 1]) for k in (0, 1, 2)}
+    _ops.clear_graph_cache()
+    _ops.note_edge_counts(p, i, nn[:3], ne)
+    for k in (2, 1, 0):
+        _ops.note_layer(p, i, nn[k], nn[k + 1])
+    before = _ops._C.graph_cache_stats()
+    announce("transposed graphs of three nested layers with announced edge counts")
+    got = {k: _ops.transposed(p, i, nn[k], nn[k + 1]) for k in (0, 1, 2)}
+    after = _ops._C.graph_cache_stats()
+    assert after["readbacks"] == before["readbacks"]
+    assert after["sorts"] - before["sorts"] == 1 and after["cuts"] - before["cuts"] == 2
+    for k in (0, 1, 2):
+        pt, it, pm, n_e = want[k]
+        assert got[k].n_edges == n_e == ne[k]
+        assert torch.equal(got[k].ptr_t, pt) and torch.equal(got[k].idx_t, it) and torch.equal(got[k].perm, pm)
+    # without the announcement the counts come from the device
+    _ops.clear_graph_cache()
+    _ops.transposed(p, i, nn[0], nn[1])
+    assert _ops._C.graph_cache_stats()["readbacks"] == after["readbacks"] + 1
+    # counts that cannot be right are refused
+    with pytest.raises((ValueError, RuntimeError)):
+        _ops.note_edge_counts(p, i, [nn[0]], [idx.shape[0] + 1])
+    with pytest.raises((ValueError, RuntimeError)):
+        _ops.note_edge_counts(p, i, [ptr.shape[0]], [0])
+    _ops.clear_graph_cache()
+
+
+def test_sage_layer_with_frozen_input_announces_nothing():
+    """The first layer of a batch whose input features need no gradient (the normal training case)
+    does not ask for its reversed graph in the backward pass, so it does not announce itself: the
+    reversed graphs of the layers above it are cut from the largest layer that needs one, not from
+    the largest layer of the batch."""
+    import cxgnncomp
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    ptr, idx, nn, ne = S.sampled_batch(num_seeds=200, fanouts=(6, 4, 3), id_space=100000, seed=12)
+    p, i = ptr.cuda(), idx.cuda()
+    torch.manual_seed(0)
+    layers = [cxgnncomp.MySageConv(16, 32).cuda(), cxgnncomp.MySageConv(32, 32).cuda(), cxgnncomp.MySageConv(32, 8).cuda()]
+    x = torch.randn(nn[3], 16, device="cuda")                      # no gradient wanted
+    _ops.clear_graph_cache()
+    before = _ops._C.graph_cache_stats()
+    h = x
+    for li, layer in enumerate(layers):
+        h = torch.relu(layer(h, p, i, nn[2 - li]))
+    announce("3 SAGE layers, frozen input features")
+    h.sum().backward()
+    torch.cuda.synchronize()
+    after = _ops._C.graph_cache_stats()
+    # layers 2 and 3 need reversed graphs (rows nn[1] and nn[0]); the first layer's (rows nn[2]) is never built
+    assert after["sorts"] - before["sorts"] == 1 and after["cuts"] - before["cuts"] == 1
+    assert after["graphs"] == 2
+    _ops.clear_graph_cache()
