@@ -254,6 +254,13 @@ def c3(iters):
     g = torch.randn(N, H, C, device="cuda") / 8
     report("c3", "spmm_multihead_fwd H=4 C=64", timeit(lambda: _ops.spmm(ptr, idx, x, N, val=ev), iters),
            spmm_bytes(N, E, H * C, H), 2 * E * H * C)
+    import cxgnncomp_backend as B
+    report("c3", "spmm_multihead PreReduce H=4 C=64 (heads summed inside the kernel, out [N, 64])",
+           timeit(lambda: B.spmm_multihead(ptr, idx, ev, x, N, B.SPMM_MULTIHEAD_SCHEDULE.PreReduce), iters),
+           E * (4 * H * C + 8 + 4 * H) + 4 * N * C + 8 * (N + 1), 2 * E * H * C)
+    report("c3", "the same as two passes (Naive, then a sum over the heads)",
+           timeit(lambda: _ops._C.head_sum(B.spmm_multihead(ptr, idx, ev, x, N, B.SPMM_MULTIHEAD_SCHEDULE.Naive)), iters),
+           E * (4 * H * C + 8 + 4 * H) + 4 * N * C + 8 * (N + 1), 2 * E * H * C)
     report("c3", "spmm_multihead_bwd H=4 C=64",
            timeit(lambda: _ops.spmm(gt.ptr_t, gt.idx_t, g, N, val=ev, val_perm=gt.perm), iters),
            spmm_bytes(N, E, H * C, H) + 8 * E, 2 * E * H * C)

@@ -121,6 +121,15 @@ template <int G> __device__ __forceinline__ float lane_group_sum(float v) {
   for (int m = G / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, CXG_WAVE);
   return v;
 }
+__device__ __forceinline__ void vxor_add(float& a, int m) { a += __shfl_xor(a, m, CXG_WAVE); }
+__device__ __forceinline__ void vxor_add(float2& a, int m) {
+  a.x += __shfl_xor(a.x, m, CXG_WAVE); a.y += __shfl_xor(a.y, m, CXG_WAVE);
+}
+__device__ __forceinline__ void vxor_add(float4& a, int m) {
+  a.x += __shfl_xor(a.x, m, CXG_WAVE); a.y += __shfl_xor(a.y, m, CXG_WAVE);
+  a.z += __shfl_xor(a.z, m, CXG_WAVE); a.w += __shfl_xor(a.w, m, CXG_WAVE);
+}
+
 __device__ __forceinline__ float vdot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
 // DOTG > 0 (V == 4, whole column tiles, DOTG = channels / 4 lanes per head): the wave also
@@ -128,8 +137,15 @@ __device__ __forceinline__ float vdot4(float4 a, float4 b) { return a.x * b.x + 
 // stores the per-head sums at the edge's weight row -- the edge-value gradient of the
 // attention layer from the gathers of its input gradient.  The rows of dot_b are loaded
 // one output row ahead (a deeper ring measured the same).
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int U, int DOTG = 0>
+// PRE (WMODE 2, the whole row of heads x channels = 64 * V floats in one column tile): the
+// heads are summed before a row -- or a partial row on its way to the carry buffer -- is
+// stored: out[r, :] = sum_h sum_e val[e, h] x[idx[e], h, :].  A head occupies channels / V
+// consecutive lanes, so the sum over heads is a butterfly over the lane bits above that, and
+// the lanes of the first head store the channels floats of the row (out, bias, the carry rows
+// and the fix-up kernel then all work on rows of `channels` floats).
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int U, int DOTG = 0, bool PRE = false>
 __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
+  static_assert(!PRE || (WMODE == 2 && !GUARD && !EXT && DOTG == 0), "head pre-reduction: plain per-head weights only");
   using vec_t = typename Vec<V>::type;
   constexpr int kDotHeads = DOTG > 0 ? CXG_WAVE / DOTG : 1;       // heads of one 256-float column tile
   __shared__ __attribute__((aligned(16))) float s_dot[DOTG > 0 ? kWavesPerBlock : 1][DOTG > 0 ? CXG_WAVE * kDotHeads : 1];
@@ -150,7 +166,9 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   // column tile of this block (grid.y tiles rows wider than 64*V floats)
   const int col = blockIdx.y * (CXG_WAVE * V) + lane * V;
   const bool col_ok = GUARD ? (col < a.F) : true;
-  const int F = a.F;
+  const int F = PRE ? a.channels : a.F;      // floats of a stored row
+  const int lanes_per_head = PRE ? a.channels / V : CXG_WAVE;
+  const bool st_ok = PRE ? lane < lanes_per_head : col_ok;   // this lane stores (its column of the stored row is `col`)
 
   const int64_t r_lo = wave_lower_bound(a.ptr, n_rows, e0);
   bool is_head = (r_lo == n_rows) || ((int64_t)a.ptr[r_lo] > e0);
@@ -185,11 +203,17 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   }
 
   auto store_vec = [&](float* dst, vec_t v) {
-    if (col_ok) stream_store(dst + col, v);
+    if (st_ok) stream_store(dst + col, v);
+  };
+  // PRE: sum over the heads, left in every lane (the lanes of head 0 store it)
+  auto head_reduce = [&](vec_t& v) {
+    if constexpr (PRE) {
+      for (int m = lanes_per_head; m < CXG_WAVE; m <<= 1) vxor_add(v, m);
+    }
   };
   // What finish_row leaves in a row without edges.
   auto store_empty_row = [&](int64_t row) {
-    if ((EXT && a.targets) || (a.accumulate && !a.bias) || !col_ok) return;
+    if ((EXT && a.targets) || (a.accumulate && !a.bias) || !st_ok) return;
     float* dst = a.out + row * a.ldo;
     vec_t z = vzero<V>();
     if (a.bias) vadd(z, *reinterpret_cast<const vec_t*>(a.bias + col));
@@ -262,6 +286,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   }
   // Row r is complete inside this span: write it (or its head partial).
   auto finish_row = [&]() {
+    head_reduce(acc);
     if (is_head) {
       store_vec(carry_head, acc);
     } else if (EXT && a.targets) {
@@ -273,10 +298,10 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
         if (deg > 0) vscale(acc, 1.0f / (float)deg);
       }
       if (a.bias) {
-        if (col_ok) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
+        if (st_ok) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
       }
       if (a.accumulate) {
-        if (col_ok) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
+        if (st_ok) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
       }
       store_vec(dst, acc);
     }
@@ -365,6 +390,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
   int64_t tail = -1;
   while (r < n_rows) {
     if (cur_end > n) {
+      head_reduce(acc);
       if (is_head) {
         store_vec(carry_head, acc);
       } else if (cur_start < n) {
@@ -399,15 +425,6 @@ __device__ __forceinline__ int64_t shfl_i64(int64_t v, int src_lane) {
   const int hi = __shfl((int)(v >> 32), src_lane, CXG_WAVE);
   return ((int64_t)hi << 32) | (uint32_t)lo;
 }
-__device__ __forceinline__ void vxor_add(float& a, int m) { a += __shfl_xor(a, m, CXG_WAVE); }
-__device__ __forceinline__ void vxor_add(float2& a, int m) {
-  a.x += __shfl_xor(a.x, m, CXG_WAVE); a.y += __shfl_xor(a.y, m, CXG_WAVE);
-}
-__device__ __forceinline__ void vxor_add(float4& a, int m) {
-  a.x += __shfl_xor(a.x, m, CXG_WAVE); a.y += __shfl_xor(a.y, m, CXG_WAVE);
-  a.z += __shfl_xor(a.z, m, CXG_WAVE); a.w += __shfl_xor(a.w, m, CXG_WAVE);
-}
-
 template <typename IdxT, int V, int L, int WMODE, bool PERM>
 __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   using vec_t = typename Vec<V>::type;
@@ -731,7 +748,7 @@ Plan make_plan(int64_t n_edges_cap, int64_t row_floats) {
   return p;
 }
 
-template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0>
+template <typename IdxT, int V, bool GUARD, int WMODE, bool PERM, bool EXT, int DOTG = 0, bool PRE = false>
 int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t stream) {
   // Gathers in flight per wave.  Measured on MI355X (61.9M-edge power-law graph):
   // with 32 waves per CU the memory system is already saturated, and issuing more
@@ -760,7 +777,7 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
           hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n_cu > 0)
         cus = n_cu;
       if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-              &blocks, spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U, DOTG>, kBlock, 0) != hipSuccess || blocks < 1)
+              &blocks, spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U, DOTG, PRE>, kBlock, 0) != hipSuccess || blocks < 1)
         blocks = 4;
       return (int64_t)blocks * kWavesPerBlock * cus;
     }();
@@ -773,9 +790,21 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   }
   dim3 grid((unsigned)ceil_div(n_spans_cap, kWavesPerBlock), (unsigned)n_ct, 1);
   dim3 block(kBlock, 1, 1);
-  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U, DOTG>), grid, block, 0, stream, a);
+  hipLaunchKernelGGL((spmm_span_kernel<IdxT, V, GUARD, WMODE, PERM, EXT, U, DOTG, PRE>), grid, block, 0, stream, a);
   CXG_LAUNCH_CHECK("spmm_span_kernel");
-  hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, V, GUARD>), grid, block, 0, stream, a);
+  if constexpr (PRE) {
+    // the stored rows (and the carry rows) hold `channels` floats
+    SpmmArgs<IdxT> f = a;
+    f.F = a.channels;
+    if (f.F % 128 == 0) {
+      hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 2, false>), dim3(grid.x, (unsigned)(f.F / 128), 1), block, 0, stream, f);
+    } else {
+      hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 1, true>), dim3(grid.x, (unsigned)ceil_div(f.F, CXG_WAVE), 1), block, 0,
+                         stream, f);
+    }
+  } else {
+    hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, V, GUARD>), grid, block, 0, stream, a);
+  }
   CXG_LAUNCH_CHECK("spmm_fixup_kernel");
   return CXG_OK;
 }
@@ -869,7 +898,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
                 const float* x, int64_t ldx, float* out, int64_t ldo, int64_t n_rows,
                 int64_t n_edges_cap, int heads, int channels, unsigned flags, void* workspace,
                 size_t workspace_bytes, void* stream, const SpmmExt* ext = nullptr,
-                const SpmmDot* dot = nullptr, const float* bias = nullptr) {
+                const SpmmDot* dot = nullptr, const float* bias = nullptr, bool prereduce = false) {
   CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
   CXG_REQUIRE(heads >= 1 && channels >= 1, CXG_ERR_ARG, "heads/channels must be >= 1");
   CXG_REQUIRE((int64_t)heads * channels <= (1 << 20), CXG_ERR_UNSUPPORTED, "row too wide");
@@ -879,7 +908,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   CXG_REQUIRE(ptr && out, CXG_ERR_ARG, "null ptr/out");
   CXG_REQUIRE(n_edges_cap == 0 || (idx && x), CXG_ERR_ARG, "null idx/x");
   const int F = heads * channels;
-  CXG_REQUIRE(ldx >= F && ldo >= F, CXG_ERR_ARG, "row stride smaller than row");
+  CXG_REQUIRE(ldx >= F && ldo >= (prereduce ? channels : F), CXG_ERR_ARG, "row stride smaller than row");
   CXG_REQUIRE(!perm || val, CXG_ERR_ARG, "val_perm without val");
   const Plan plan = make_plan(n_edges_cap, F);
   CXG_REQUIRE(workspace && workspace_bytes >= plan.tail_bytes + plan.carry_bytes, CXG_ERR_WORKSPACE,
@@ -932,6 +961,28 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
 #undef CXG_DOT
     }
     return set_error(CXG_ERR_UNSUPPORTED, "spmm with dot products needs int64 indices");
+  }
+  if (prereduce) {
+    if constexpr (sizeof(IdxT) == 8) {
+      CXG_REQUIRE(val && heads > 1, CXG_ERR_ARG, "head pre-reduction needs per-head weights and more than one head");
+      CXG_REQUIRE(!a.mean, CXG_ERR_ARG, "head pre-reduction cannot be combined with mean");
+      // the row of heads x channels floats must be exactly one column tile of 64 lanes x V floats
+      int v = 0;
+      for (int t = 4; t >= 1; t /= 2)
+        if (F == CXG_WAVE * t && channels % t == 0) { v = t; break; }
+      const uintptr_t align_bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)a.carry | (uintptr_t)a.bias |
+                                   (uintptr_t)(ldx * 4) | (uintptr_t)(ldo * 4) | (uintptr_t)(channels * 4);
+      CXG_REQUIRE(v > 0 && (align_bits & (uintptr_t)(4 * v - 1)) == 0 && (heads & (heads - 1)) == 0, CXG_ERR_UNSUPPORTED,
+                  "head pre-reduction in the kernel needs heads * channels in {64, 128, 256}, a power-of-two head "
+                  "count and aligned rows");
+#define CXG_PRE(VV)                                                                                       \
+  if (v == VV)                                                                                            \
+    return perm ? launch_spmm<IdxT, VV, false, 2, true, false, 0, true>(a, plan.n_spans_cap, st)           \
+                : launch_spmm<IdxT, VV, false, 2, false, false, 0, true>(a, plan.n_spans_cap, st)
+      CXG_PRE(4); CXG_PRE(2); CXG_PRE(1);
+#undef CXG_PRE
+    }
+    return set_error(CXG_ERR_UNSUPPORTED, "head pre-reduction needs int64 indices");
   }
   if (!val) return dispatch_shape<IdxT, 0, false>(a, plan.n_spans_cap, st);
   if constexpr (sizeof(IdxT) == 8) {
@@ -1012,6 +1063,15 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx, const float* v
   if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
   return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
                                    heads, channels, flags, workspace, workspace_bytes, stream);
+}
+
+int cxg_spmm_prereduce_f32(const int64_t* ptr, const int64_t* idx, const float* val, const int64_t* val_perm,
+                           const float* x, int64_t ldx, float* out, int64_t ldo, int64_t n_rows, int64_t n_edges_cap,
+                           int heads, int channels, unsigned flags, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+  if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
+  return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap, heads, channels,
+                                   flags, workspace, workspace_bytes, stream, nullptr, nullptr, nullptr, true);
 }
 
 int cxg_spmm_weighted_bias_f32(const int64_t* ptr, const int64_t* idx, const float* val,

@@ -853,7 +853,31 @@ Tensor spmm_multihead(const Tensor& ptr, const Tensor& idx, const Tensor& val, c
   if (vin.dim() != 3) bad("vin must be 3D, [num_node, num_head, feat_len]");
   if (val.dim() != 2) bad("val must be 2D, [num_edge, num_head]");
   if (val.size(1) != vin.size(1)) bad(fmt("num_head mismatch %lld %lld", (long long)vin.size(1), (long long)val.size(1)));
-  Tensor out = spmm(ptr, idx, vin, as_int(num_node), false, val, c10::nullopt, c10::nullopt, false, c10::nullopt);
+  const int64_t n = as_int(num_node);
+  if (schedule != MultiheadSchedule::Naive) {
+    // PreReduce / Optimal: out[N, F], summed over the heads inside the aggregation kernel where the
+    // row of heads x channels floats is one 64-lane gather; other shapes aggregate per head and sum after
+    const int64_t heads = vin.size(1), channels = vin.size(2), row = heads * channels;
+    const bool one_gather = heads > 1 && (heads & (heads - 1)) == 0 && (row == 64 || row == 128 || row == 256);
+    if (one_gather && n > 0) {
+      check_graph(ptr, idx, n);
+      req(vin, "vin", at::kFloat, {3});
+      req(val, "val", at::kFloat, {2});
+      if (vin.device() != ptr.device()) bad("vin and ptr are on different devices");
+      if (val.size(0) < idx.size(0)) bad(fmt("val has %lld rows, idx has %lld", (long long)val.size(0), (long long)idx.size(0)));
+      Tensor out = torch::empty({n, channels}, vin.options());
+      Tensor ws = workspace(cxg_spmm_workspace_bytes(idx.size(0), row), vin);
+      c10::DeviceGuard guard(vin.device());
+      const int rc = cxg_spmm_prereduce_f32((const int64_t*)ptr.data_ptr(), (const int64_t*)ptr_or_null(idx),
+                                            (const float*)val.data_ptr(), nullptr, (const float*)ptr_or_null(vin), row,
+                                            (float*)out.data_ptr(), channels, n, idx.size(0), (int)heads, (int)channels,
+                                            n == ptr.size(0) - 1 ? kSpmmExactEdges : 0u, ws.data_ptr(), (size_t)ws.numel(),
+                                            stream_of(vin));
+      if (rc == 0) return out;
+      if (rc != CXG_ERR_UNSUPPORTED) check(rc);
+    }
+  }
+  Tensor out = spmm(ptr, idx, vin, n, false, val, c10::nullopt, c10::nullopt, false, c10::nullopt);
   return schedule == MultiheadSchedule::Naive ? out : head_sum(out);
 }
 

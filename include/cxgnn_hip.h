@@ -117,6 +117,24 @@ int cxg_spmm_weighted_f32(const int64_t* ptr, const int64_t* idx,
                           size_t workspace_bytes, void* stream);
 
 /*
+ * Multi-head edge-weighted aggregation summed over the heads inside the kernel:
+ *   out[r, c] = sum_h sum_e val[vrow(e), h] * x[idx[e], h, c]     (out is [n_rows, channels]).
+ * The wave that gathers a row of heads x channels floats adds its head groups with
+ * xor-shuffles when the row ends and stores channels floats: no [n_rows, heads, channels]
+ * intermediate is written and read back.  Takes heads * channels in {64, 128, 256} with a
+ * power-of-two head count (the whole row in one 64-lane gather), otherwise
+ * CXG_ERR_UNSUPPORTED (run cxg_spmm_weighted_f32 and cxg_head_sum_f32 instead).  Workspace
+ * as for cxg_spmm_weighted_f32 (cxg_spmm_workspace_bytes(n_edges_cap, heads * channels)).
+ * Replaces spmm_multihead(..., PreReduce / Optimal) and run_spmm_multihead_configurable
+ * (src/cpp/src/spmm_host.cu:158-256, kernels spmm_multihead_kernel.cu:38-207).
+ */
+int cxg_spmm_prereduce_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                           const int64_t* val_perm, const float* x, int64_t ldx, float* out,
+                           int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int heads,
+                           int channels, unsigned flags, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/*
  * cxg_spmm_weighted_f32 with bias[heads*channels] added to every output row as it is
  * stored (NULL: none; not with CXG_SPMM_MEAN): the `out + self.bias` that follows the
  * aggregation in MyGATConv.forward_many (cxgnncomp/graph_conv.py:488-494) without a second

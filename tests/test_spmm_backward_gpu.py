@@ -191,3 +191,52 @@ def test_bad_arguments_raise_instead_of_exiting():
         B.run_spmm_configurable(ptr.cuda(), idx.cuda(), x.cuda(), n + 5)  # more rows than ptr holds
     with pytest.raises(ValueError):
         B.run_spmm_configurable(ptr.cuda(), idx.cuda(), x.cuda().unsqueeze(0), n)  # vin must be 2D
+
+
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
+@pytest.mark.parametrize("shape", [(4, 64), (8, 32), (2, 128), (2, 64), (4, 32), (2, 32), (8, 8), (16, 16), (4, 40), (3, 64), (4, 128)])
+def test_spmm_multihead_head_sum_inside_the_kernel(kind, shape):
+    """spmm_multihead(PreReduce / Optimal): out[N, C] summed over the heads.  Rows of heads x channels
+    = 64, 128 or 256 floats with a power-of-two head count are summed by the gathering wave itself
+    (cxg_spmm_prereduce_f32: rows inside a span, rows completed by the fix-up kernel in 'one_hub' and
+    'powerlaw', rows without edges); the other shapes aggregate per head and sum afterwards.  Both
+    against the oracle, deterministic, and a row prefix."""
+    import cxgnncomp_backend as B
+    H, C = shape
+    ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    torch.manual_seed(H * 100 + C)
+    x = torch.randn(n, H, C) * _scale(ptr)
+    val = torch.rand(E, H) - 0.3
+    p, i = ptr.numpy(), idx.numpy()
+    announce("spmm_multihead PreReduce kind=%s H=%d C=%d" % (kind, H, C))
+    pc, ic, vc, xc = ptr.cuda(), idx.cuda(), val.cuda(), x.cuda()
+    pre = B.spmm_multihead(pc, ic, vc, xc, n, B.SPMM_MULTIHEAD_SCHEDULE.PreReduce)
+    assert pre.shape == (n, C)
+    want = oracle.spmm_prereduce(p, i, val.numpy(), x.numpy(), n)
+    assert_close(_np(pre), want, RTOL, ATOL, "prereduce")
+    assert torch.equal(pre, B.spmm_multihead(pc, ic, vc, xc, n, B.SPMM_MULTIHEAD_SCHEDULE.Optimal))
+    rows = n // 3
+    part = B.spmm_multihead(pc, ic, vc, xc, rows, B.SPMM_MULTIHEAD_SCHEDULE.PreReduce)
+    assert_close(_np(part), oracle.spmm_prereduce(p, i, val.numpy(), x.numpy(), rows), RTOL, ATOL, "prereduce prefix")
+
+
+def test_prereduce_entry_point_rejects_other_shapes():
+    from cxgnncomp_backend import _lib
+    lib = _lib.load()
+    ptr = torch.tensor([0, 2, 3], device="cuda")
+    idx = torch.tensor([0, 1, 1], device="cuda")
+    ws = torch.empty(lib.cxg_spmm_workspace_bytes(3, 512), dtype=torch.uint8, device="cuda")
+    st = _lib.current_stream(ptr.device)
+
+    def call(H, C):
+        x = torch.zeros(2, H, C, device="cuda")
+        val = torch.zeros(3, H, device="cuda")
+        out = torch.zeros(2, C, device="cuda")
+        return lib.cxg_spmm_prereduce_f32(ptr.data_ptr(), idx.data_ptr(), val.data_ptr(), None, x.data_ptr(), H * C,
+                                          out.data_ptr(), C, 2, 3, H, C, 0, ws.data_ptr(), ws.numel(), st)
+    assert call(4, 64) == 0 and call(2, 32) == 0
+    assert call(3, 64) == -2 and call(4, 128) == -2 and call(4, 40) == -2      # CXG_ERR_UNSUPPORTED
+    assert call(1, 64) == -1                                                   # one head: nothing to sum
+    torch.cuda.synchronize()
