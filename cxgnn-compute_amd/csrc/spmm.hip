@@ -102,6 +102,7 @@ struct SpmmArgs {
   int64_t ld_dot_b;
   float* dot_out;
   const float* bias;       // [F] added to every output row, or null
+  int out_bf16;            // the rows of `out` are bf16 (grouped-lane kernel with IO & 2, and its fix-up launch)
 };
 
 __device__ __forceinline__ void atomic_add_vec(float* p, float v) { unsafeAtomicAdd(p, v); }
@@ -425,8 +426,26 @@ __device__ __forceinline__ int64_t shfl_i64(int64_t v, int src_lane) {
   const int hi = __shfl((int)(v >> 32), src_lane, CXG_WAVE);
   return ((int64_t)hi << 32) | (uint32_t)lo;
 }
-template <typename IdxT, int V, int L, int WMODE, bool PERM>
+// bf16 rows: four values are 8 bytes; widened by a shift, narrowed with round-to-nearest-even
+__device__ __forceinline__ float4 load_bf16x4(const uint16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                     __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  v2bf t = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(unsigned, t);
+}
+__device__ __forceinline__ void store_bf16x4(uint16_t* p, float4 v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v.x, v.y), pack_bf16x2(v.z, v.w));
+}
+
+// IO & 1: the rows of x are bf16 (ldx in elements); IO & 2: the rows of out are bf16 (ldo in
+// elements) -- sums and carried partial rows stay fp32.  V == 4 only.
+template <typename IdxT, int V, int L, int WMODE, bool PERM, int IO = 0>
 __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
+  static_assert(IO == 0 || V == 4, "bf16 rows are handled four values at a time");
   using vec_t = typename Vec<V>::type;
   constexpr int G = CXG_WAVE / L;
   constexpr int UF = CXG_SPMM_GROUP_UF;       // steps issued together inside long rows
@@ -473,6 +492,10 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   // What finish_row leaves in a row without edges.
   auto store_empty_row = [&](int64_t row) {
     if ((a.accumulate && !a.bias) || !col_ok) return;
+    if constexpr ((IO & 2) != 0) {
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + row * a.ldo + col) = make_uint2(0u, 0u);
+      return;
+    }
     float* dst = a.out + row * a.ldo;
     vec_t z = vzero<V>();
     if (a.bias) vadd(z, *reinterpret_cast<const vec_t*>(a.bias + col));
@@ -543,6 +566,14 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     reduce_groups();
     if (is_head) {
       store_vec(carry_head, acc);
+    } else if constexpr ((IO & 2) != 0) {
+      if (a.mean) {
+        const int deg = cur_end - cur_start;
+        if (deg > 0) vscale(acc, 1.0f / (float)deg);
+      }
+      if constexpr (V == 4) {
+        if (writer) store_bf16x4(reinterpret_cast<uint16_t*>(a.out) + r * a.ldo + col, acc);
+      }
     } else {
       float* dst = a.out + r * a.ldo;
       if (a.mean) {
@@ -573,7 +604,11 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     }
     auto gather = [&](int e_idx, bool act, vec_t& v, float& w) {
       const int64_t src = shfl_i64(my_src, e_idx & 63);
-      v = (act && col_ok) ? *reinterpret_cast<const vec_t*>(a.x + src * a.ldx + col) : vzero<V>();
+      if constexpr ((IO & 1) != 0 && V == 4) {
+        v = (act && col_ok) ? load_bf16x4(reinterpret_cast<const uint16_t*>(a.x) + src * a.ldx + col) : vzero<V>();
+      } else {
+        v = (act && col_ok) ? *reinterpret_cast<const vec_t*>(a.x + src * a.ldx + col) : vzero<V>();
+      }
       if (WMODE == 1) {
         if (PERM) {
           const int64_t vrow = shfl_i64(my_vrow, e_idx & 63);
@@ -675,6 +710,11 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
       const int64_t row_b = shfl_i64(rb, j), row_e = shfl_i64(re, j);
       for (int64_t row = row_b + j; row < row_e; row += J) {
         if (!col_ok) continue;
+        if (a.out_bf16) {
+          uint16_t* d16 = reinterpret_cast<uint16_t*>(a.out) + row * a.ldo + col;
+          for (int k = 0; k < V; ++k) d16[k] = 0;
+          continue;
+        }
         float* dst = a.out + row * a.ldo;
         vec_t z = vzero<V>();
         if (a.bias) vadd(z, *reinterpret_cast<const vec_t*>(a.bias + col));
@@ -716,6 +756,12 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(SpmmArgs<IdxT> a) {
     return;
   }
   if (a.mean) vscale(acc, 1.0f / (float)(row_end - row_begin));
+  if (a.out_bf16) {
+    uint16_t* d16 = reinterpret_cast<uint16_t*>(a.out) + t * a.ldo + col;
+    const float* av = reinterpret_cast<const float*>(&acc);
+    for (int k = 0; k < V; ++k) d16[k] = (uint16_t)(pack_bf16x2(av[k], 0.f) & 0xffffu);
+    return;
+  }
   float* dst = a.out + t * a.ldo;
   if (a.bias) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
   if (a.accumulate) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
@@ -929,6 +975,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   a.src_map = nullptr; a.targets = nullptr;
   a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr;
   a.bias = bias;
+  a.out_bf16 = 0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (ext) {
     CXG_REQUIRE(!val, CXG_ERR_UNSUPPORTED, "extended gather takes no edge weights");
@@ -1072,6 +1119,62 @@ int cxg_spmm_prereduce_f32(const int64_t* ptr, const int64_t* idx, const float* 
   if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
   return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap, heads, channels,
                                    flags, workspace, workspace_bytes, stream, nullptr, nullptr, nullptr, true);
+}
+
+// single-head aggregation of rows of at most 128 values with bf16 rows on either side
+int cxg_spmm_bf16_rows(const int64_t* ptr, const int64_t* idx, const float* val, const int64_t* val_perm, const void* x,
+                       int64_t ldx, int x_bf16, void* out, int64_t ldo, int out_bf16, int64_t n_rows, int64_t n_edges_cap,
+                       int feat, unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace cxg;
+  CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
+  CXG_REQUIRE((flags & ~(CXG_SPMM_MEAN | CXG_SPMM_HINT_EXACT_EDGES)) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE(x_bf16 || out_bf16, CXG_ERR_ARG, "fp32 rows on both sides: use cxg_spmm_sum_f32 / cxg_spmm_weighted_f32");
+  CXG_REQUIRE(feat >= 4 && feat <= 128 && feat % 4 == 0, CXG_ERR_UNSUPPORTED, "bf16 rows: 4 <= feat <= 128, a multiple of 4");
+  if (n_rows == 0) return CXG_OK;
+  CXG_REQUIRE(ptr && out && (n_edges_cap == 0 || (idx && x)), CXG_ERR_ARG, "null pointer");
+  CXG_REQUIRE(ldx >= feat && ldo >= feat && ldx % 4 == 0 && ldo % 4 == 0, CXG_ERR_ARG, "row strides: at least feat, multiples of 4");
+  CXG_REQUIRE((((uintptr_t)x | (uintptr_t)out) & 15) == 0, CXG_ERR_ARG, "rows must be 16-byte aligned");
+  CXG_REQUIRE(!val_perm || val, CXG_ERR_ARG, "val_perm without val");
+  const Plan plan = make_plan(n_edges_cap, feat);
+  CXG_REQUIRE(workspace && workspace_bytes >= plan.tail_bytes + plan.carry_bytes && ((uintptr_t)workspace & 255) == 0,
+              CXG_ERR_WORKSPACE, "workspace of %zu bytes (256-byte aligned) needed", plan.tail_bytes + plan.carry_bytes);
+  SpmmArgs<int64_t> a;
+  a.ptr = ptr; a.idx = idx; a.x = reinterpret_cast<const float*>(x); a.out = reinterpret_cast<float*>(out);
+  a.val = val; a.perm = val_perm; a.ldx = ldx; a.ldo = ldo; a.n_rows = n_rows; a.F = feat; a.heads = 1; a.channels = feat;
+  a.T = plan.T; a.exact_edges = 0; a.mean = (flags & CXG_SPMM_MEAN) ? 1 : 0; a.accumulate = 0;
+  a.tail_row = reinterpret_cast<int64_t*>(workspace);
+  a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
+  a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0; a.src_map = nullptr; a.targets = nullptr;
+  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr; a.bias = nullptr; a.out_bf16 = out_bf16 ? 1 : 0;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int lanes = feat / 4;
+  int L = 4;
+  while (L < lanes) L <<= 1;
+  const dim3 grid((unsigned)ceil_div(plan.n_spans_cap, kWavesPerBlock), 1, 1), block(kBlock, 1, 1);
+  const int io = (x_bf16 ? 1 : 0) | (out_bf16 ? 2 : 0);
+  const int wmode = val ? 1 : 0;
+  bool done = false;
+#define CXG_IO(LL, WM, PM, IOV)                                                                              \
+  if (!done && L == LL && wmode == WM && (val_perm != nullptr) == PM && io == IOV) {                          \
+    hipLaunchKernelGGL((spmm_group_kernel<int64_t, 4, LL, WM, PM, IOV>), grid, block, 0, st, a);               \
+    done = true;                                                                                             \
+  }
+#define CXG_IO_L(LL)                                                                                          \
+  CXG_IO(LL, 0, false, 1) CXG_IO(LL, 0, false, 2) CXG_IO(LL, 0, false, 3)                                       \
+  CXG_IO(LL, 1, false, 1) CXG_IO(LL, 1, false, 2) CXG_IO(LL, 1, false, 3)                                       \
+  CXG_IO(LL, 1, true, 1) CXG_IO(LL, 1, true, 2) CXG_IO(LL, 1, true, 3)
+  CXG_IO_L(4) CXG_IO_L(8) CXG_IO_L(16) CXG_IO_L(32)
+#undef CXG_IO_L
+#undef CXG_IO
+  CXG_REQUIRE(done, CXG_ERR_UNSUPPORTED, "no kernel for this combination");
+  CXG_LAUNCH_CHECK("spmm_group_kernel");
+  if (feat % 128 == 0) {
+    hipLaunchKernelGGL((spmm_fixup_kernel<int64_t, 2, false>), dim3(grid.x, (unsigned)(feat / 128), 1), block, 0, st, a);
+  } else {
+    hipLaunchKernelGGL((spmm_fixup_kernel<int64_t, 1, true>), dim3(grid.x, (unsigned)ceil_div(feat, CXG_WAVE), 1), block, 0, st, a);
+  }
+  CXG_LAUNCH_CHECK("spmm_fixup_kernel");
+  return CXG_OK;
 }
 
 int cxg_spmm_weighted_bias_f32(const int64_t* ptr, const int64_t* idx, const float* val,

@@ -52,6 +52,7 @@ struct GemmArgs {
   const float* bias;
   const float* addend;
   int64_t ldd;
+  int c_bf16;             // the rows of C are bf16 (ldc in elements): the bf16-operand kernels, plain stores only
 };
 
 // Tile number -> (relation, first row, end of the relation's rows).  Every thread
@@ -203,6 +204,38 @@ __device__ __forceinline__ void store_tile_mode(const GemmArgs& g, const v16f (&
         float* p = base + d[i] * ldc;
         if (MODE == 2) unsafeAtomicAdd(p, v[i]);
         else *p = v[i];
+      }
+    }
+  }
+}
+
+// bf16 rows of C (N and ldc even, plain stores).  A lane holds four consecutive rows of ONE
+// column; it swaps values with the lane of the neighbouring column (lane ^ 1) so that the even
+// lane stores rows 0 and 1 and the odd lane rows 2 and 3 of each group as pairs of columns:
+// 4-byte stores instead of 2-byte ones.
+template <int MT>
+__device__ __forceinline__ void store_tile_bf16(const GemmArgs& g, const v16f (&acc)[MT], const int64_t* s_dst, int wn,
+                                                int lane, int n0) {
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  const int col = n0 + wn * 32 + (lane & 31);
+  const bool odd = lane & 1;
+  uint16_t* const base = reinterpret_cast<uint16_t*>(g.c) + (col & ~1);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int rl0 = mt * 32 + q * 8 + (lane >> 5) * 4;
+      float other[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        other[j] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc[mt][q * 4 + j]), 0xB1, 0xf, 0xf, false));
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int j = odd ? 2 + h : h;
+        const float mine = acc[mt][q * 4 + j], theirs = other[j];
+        const v2bf pr = {(__bf16)(odd ? theirs : mine), (__bf16)(odd ? mine : theirs)};
+        const int64_t d = s_dst[rl0 + j];
+        if (d >= 0 && col < g.N) *reinterpret_cast<unsigned*>(base + d * g.ldc) = __builtin_bit_cast(unsigned, pr);
       }
     }
   }
@@ -1091,7 +1124,8 @@ __global__ __launch_bounds__(kThreads) void typed_gemm_bf16_resident_kernel(Gemm
         acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bw[s], acc[mt], 0, 0, 0);
       }
     }
-    store_tile<128, 2>(g, acc, s_dst[t % 3], 0, wave, lane, n0);
+    if (g.c_bf16) store_tile_bf16<2>(g, acc, s_dst[t % 3], wave, lane, n0);
+    else store_tile<128, 2>(g, acc, s_dst[t % 3], 0, wave, lane, n0);
     __syncthreads();
   };
   uint4 areg0[NREG], areg1[NREG];
@@ -1117,7 +1151,7 @@ hipError_t allow_lds(KernelT kernel, size_t bytes) {
 int check_args(const void* a, const void* w, float* c, const int64_t* seg, int64_t M, int K, int N,
                int R, unsigned flags) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
-  CXG_REQUIRE((flags & ~63u) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE((flags & ~127u) == 0, CXG_ERR_ARG, "unknown flag");
   if (M == 0) return CXG_OK;
   CXG_REQUIRE(a && w && c && seg, CXG_ERR_ARG, "null pointer");
   return CXG_OK;
@@ -1135,8 +1169,14 @@ static int typed_gemm_f32_impl(const float* a, int64_t lda, const float* w, cons
   if (rc || M == 0) return rc;
   CXG_REQUIRE(lda >= K && ldc >= N, CXG_ERR_ARG, "row stride smaller than row");
   cxg::GemmArgs g{a, lda, w, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
-                  (int)(flags & 1u), (int)((flags >> 1) & 1u), bias, addend, ldd};
+                  (int)(flags & 1u), (int)((flags >> 1) & 1u), bias, addend, ldd, (int)((flags & CXG_GEMM_OUT_BF16) != 0)};
   const bool epilogue = bias || addend;
+  if (g.c_bf16) {
+    CXG_REQUIRE((flags & CXG_GEMM_ROUND_BF16) && !epilogue && !(flags & 3u) && K <= 128 && (K & 7) == 0 && (lda & 7) == 0 &&
+                    ((uintptr_t)a & 15) == 0 && (N & 1) == 0 && (ldc & 1) == 0 && ((uintptr_t)c & 3) == 0,
+                CXG_ERR_UNSUPPORTED,
+                "bf16 rows of C: with CXG_GEMM_ROUND_BF16 (K <= 128, K and lda multiples of 8), even N and ldc, plain stores");
+  }
   CXG_REQUIRE(!epilogue || ((flags & CXG_GEMM_SPLIT_F16X3) && !src_idx && !dst_idx), CXG_ERR_UNSUPPORTED,
               "bias / addend are taken by the fp16 split form without row maps");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -1252,7 +1292,11 @@ int cxg_typed_gemm_bf16(const uint16_t* a, int64_t lda, const uint16_t* w_t, flo
   CXG_REQUIRE(((uintptr_t)a & 15) == 0 && ((uintptr_t)w_t & 15) == 0, CXG_ERR_ARG,
               "bf16 operands must be 16-byte aligned");
   cxg::GemmArgs g{a, lda, w_t, c, ldc, src_idx, dst_idx, seg_ptr, M, K, N, R,
-                  (int)(flags & 1u), (int)((flags >> 1) & 1u)};
+                  (int)(flags & 1u), (int)((flags >> 1) & 1u), nullptr, nullptr, 0, (int)((flags & CXG_GEMM_OUT_BF16) != 0)};
+  if (g.c_bf16) {
+    CXG_REQUIRE(K <= 128 && !(flags & 3u) && (N & 1) == 0 && (ldc & 1) == 0 && ((uintptr_t)c & 3) == 0, CXG_ERR_UNSUPPORTED,
+                "bf16 rows of C: K <= 128, even N and ldc, plain stores");
+  }
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (K <= 128) {
     int G = (int)(M * cxg::ceil_div(N, 128) / ((int64_t)cxg::kBM * 4096));

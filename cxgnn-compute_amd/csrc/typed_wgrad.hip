@@ -22,6 +22,8 @@
 // Replaces the weight-gradient half of TypedLinearE2EOP.backward /
 // TypedLinearS2DMMAggrOP.backward (cxgnncomp/typed_linear.py:114-137,205-221),
 // which the reference computes with one torch.mm per relation.
+#include <type_traits>
+
 #include "cxg_common.hpp"
 
 namespace cxg {
@@ -50,6 +52,7 @@ struct WgradArgs {
   int64_t M;
   int K, N, R;
   int64_t rows_per_chunk;
+  int a_bf16;              // the rows of A are bf16 (lda in elements)
 };
 
 template <int NS>
@@ -125,7 +128,10 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned m) {
   return ab > cd ? ab : cd;
 }
 
-template <int NS, bool MAPPED, bool F16>
+// ABF16: the rows of A are bf16 in memory (a compile-time choice: a run-time branch around the
+// two kinds of load made the compiler wait for every load in flight, 1.6 -> 2.6 ms on the pair
+// rows of the relational layer).
+template <int NS, bool MAPPED, bool F16, bool ABF16 = false>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(3)))
 void typed_wgrad_split_kernel(WgradArgs g) {
   static_assert(!F16 || NS == 2, "the fp16 form has two parts");
@@ -165,6 +171,7 @@ void typed_wgrad_split_kernel(WgradArgs g) {
     const bool col_ok = operand ? (n0 + 4 * c4 < N) : (4 * c4 < K);      // N % 4 == 0 is required
     const float* const base = operand ? g.g + (col_ok ? n0 + 4 * c4 : 0) : g.a + (col_ok ? 4 * c4 : 0);
     const int64_t ld = operand ? g.ldg : g.lda;
+    const uint16_t* const base16 = reinterpret_cast<const uint16_t*>(g.a) + (col_ok ? 4 * c4 : 0);
     // row of this operand behind row r of tile t (-1: no such row)
     auto row_index = [&](int t, int r) -> int64_t {
       if constexpr (MAPPED) {
@@ -187,6 +194,10 @@ void typed_wgrad_split_kernel(WgradArgs g) {
         s_map[kMappedRows + i] = didx;
       }
     }
+    // (a generic lambda: with bf16 rows of A the A producers run their own copy of the loop, whose
+    // loads are all of one kind -- the compiler counts the loads in flight statically)
+    auto produce = [&](auto a16_tag) {
+    constexpr bool A16 = decltype(a16_tag)::value;
     // Loads are issued unconditionally: rows and columns that do not exist are redirected
     // to an address that does and zeroed when the tile is staged (a select between a
     // loaded vector and a zero vector made the compiler route the load through scratch).
@@ -199,7 +210,13 @@ void typed_wgrad_split_kernel(WgradArgs g) {
       for (int i = 0; i < 4; ++i) {
         const int64_t ridx = row_index(tc, mg * 4 + i);
         mask |= (ridx >= 0 ? 1u : 0u) << i;
-        r4[i] = *reinterpret_cast<const float4*>(base + (ridx >= 0 ? ridx : 0) * ld);
+        if constexpr (A16) {
+          // four bf16 values in two registers of the set, widened when the tile is staged
+          const uint2 u = *reinterpret_cast<const uint2*>(base16 + (ridx >= 0 ? ridx : 0) * ld);
+          r4[i] = make_float4(__uint_as_float(u.x), __uint_as_float(u.y), 0.f, 0.f);
+        } else {
+          r4[i] = *reinterpret_cast<const float4*>(base + (ridx >= 0 ? ridx : 0) * ld);
+        }
       }
       live_mask = mask;
     };
@@ -212,10 +229,16 @@ void typed_wgrad_split_kernel(WgradArgs g) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const bool live = col_ok && ((live_mask >> i) & 1u) != 0;
-        v[i][0] = live ? r4[i].x : 0.f;
-        v[i][1] = live ? r4[i].y : 0.f;
-        v[i][2] = live ? r4[i].z : 0.f;
-        v[i][3] = live ? r4[i].w : 0.f;
+        float4 w4 = r4[i];
+        if constexpr (A16) {                           // two registers of four bf16 values (exact)
+          const unsigned lo = __float_as_uint(r4[i].x), hi = __float_as_uint(r4[i].y);
+          w4 = make_float4(__uint_as_float(lo << 16), __uint_as_float(lo & 0xffff0000u), __uint_as_float(hi << 16),
+                           __uint_as_float(hi & 0xffff0000u));
+        }
+        v[i][0] = live ? w4.x : 0.f;
+        v[i][1] = live ? w4.y : 0.f;
+        v[i][2] = live ? w4.z : 0.f;
+        v[i][3] = live ? w4.w : 0.f;
       }
       if constexpr (F16) {
         unsigned m = 0;
@@ -283,6 +306,10 @@ void typed_wgrad_split_kernel(WgradArgs g) {
       gload(r0, live0, t + 4);
       if (t + 2 >= n_tiles) return;
     }
+      };
+    if (ABF16 && operand == 0) produce(std::true_type{});
+    else produce(std::false_type{});
+    return;
   }
 
   // ---- consumers --------------------------------------------------------------------
@@ -452,8 +479,8 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
                              int64_t M, int K, int N, int R, float* gw, unsigned flags, void* workspace,
                              size_t workspace_bytes, void* stream) {
   CXG_REQUIRE(M >= 0 && K >= 1 && N >= 1 && R >= 1, CXG_ERR_ARG, "bad M/K/N/R");
-  CXG_REQUIRE((flags & ~(CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3)) == 0, CXG_ERR_ARG,
-              "unknown flag");
+  CXG_REQUIRE((flags & ~(CXG_GEMM_SPLIT_BF16X6 | CXG_GEMM_SPLIT_BF16X3 | CXG_GEMM_SPLIT_F16X3 | CXG_WGRAD_A_BF16)) == 0,
+              CXG_ERR_ARG, "unknown flag");
   CXG_REQUIRE(gw && seg_ptr, CXG_ERR_ARG, "null gw/seg_ptr");
   CXG_REQUIRE(M == 0 || (a && g), CXG_ERR_ARG, "null a/g");
   CXG_REQUIRE(K <= 128 && (K & 3) == 0 && (N & 3) == 0 && (lda & 3) == 0 && (ldg & 3) == 0 &&
@@ -471,12 +498,17 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
   const int n_ct = (int)cxg::ceil_div(N, 128);
   CXG_REQUIRE(chunks * n_ct < ((int64_t)1 << 31), CXG_ERR_UNSUPPORTED, "too many chunks for one launch");
   cxg::WgradArgs wa{a, lda, g, ldg, src_idx, dst_idx, seg_ptr, reinterpret_cast<float*>(workspace),
-                    M, K, N, R, rows};
+                    M, K, N, R, rows, (int)((flags & CXG_WGRAD_A_BF16) != 0)};
   const dim3 grid((unsigned)(chunks * n_ct)), block(cxg::kWgThreads);
+#define CXG_WGRAD_LAUNCH_T(NSV, MAP, HALF, AH)                                                             \
+  do {                                                                                                    \
+    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_wgrad_split_kernel<NSV, MAP, HALF, AH>, cxg::wgrad_lds_bytes<NSV>(MAP))); \
+    hipLaunchKernelGGL((cxg::typed_wgrad_split_kernel<NSV, MAP, HALF, AH>), grid, block, cxg::wgrad_lds_bytes<NSV>(MAP), st, wa); \
+  } while (0)
 #define CXG_WGRAD_LAUNCH(NSV, MAP, HALF)                                                                  \
   do {                                                                                                    \
-    CXG_HIP_CHECK(cxg::allow_lds(cxg::typed_wgrad_split_kernel<NSV, MAP, HALF>, cxg::wgrad_lds_bytes<NSV>(MAP))); \
-    hipLaunchKernelGGL((cxg::typed_wgrad_split_kernel<NSV, MAP, HALF>), grid, block, cxg::wgrad_lds_bytes<NSV>(MAP), st, wa); \
+    if (wa.a_bf16) CXG_WGRAD_LAUNCH_T(NSV, MAP, HALF, true);                                              \
+    else CXG_WGRAD_LAUNCH_T(NSV, MAP, HALF, false);                                                       \
   } while (0)
   if (flags & CXG_GEMM_SPLIT_F16X3) {
     if (mapped) CXG_WGRAD_LAUNCH(2, true, true);
@@ -489,6 +521,7 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
     else CXG_WGRAD_LAUNCH(3, false, false);
   }
 #undef CXG_WGRAD_LAUNCH
+#undef CXG_WGRAD_LAUNCH_T
   CXG_LAUNCH_CHECK("typed_wgrad_split_kernel");
   const int64_t kn = (int64_t)K * N;
   hipLaunchKernelGGL(cxg::wgrad_reduce_kernel, dim3((unsigned)cxg::ceil_div(kn, 64), (unsigned)R),

@@ -117,6 +117,34 @@ TransposedGraph = _C.TransposedGraph      # ptr_t, idx_t, perm, n_edges, n_src, 
 _GRAPH_CACHE_CAP = 8
 
 
+def spmm_bf16_rows(ptr, idx, x, n_rows, val=None, val_perm=None, out_bf16=False, mean=False):
+    """Single-head aggregation whose gathered rows (x of dtype bfloat16) and / or stored rows
+    (``out_bf16``) are bf16, summed in fp32 (cxg_spmm_bf16_rows; rows of 4 .. 128 values, a
+    multiple of 4)."""
+    lib = _lib.load()
+    _check_graph(ptr, idx, n_rows)
+    if x.dim() != 2 or not x.is_contiguous() or x.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("x must be a contiguous [N, F] float32 or bfloat16 tensor")
+    x_bf16 = x.dtype == torch.bfloat16
+    if not (x_bf16 or out_bf16):
+        raise ValueError("fp32 rows on both sides: use spmm")
+    feat = x.shape[1]
+    out = torch.empty((n_rows, feat), dtype=torch.bfloat16 if out_bf16 else torch.float32, device=x.device)
+    if n_rows == 0:
+        return out
+    if val is not None:
+        _req(val, "val", torch.float32, 1)
+    if val_perm is not None:
+        _req(val_perm, "val_perm", torch.int64, 1)
+    ws = _workspace(lib.cxg_spmm_workspace_bytes(idx.shape[0], feat), x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_spmm_bf16_rows(ptr.data_ptr(), _lib.ptr(idx), _lib.ptr(val), _lib.ptr(val_perm), _lib.ptr(x), feat,
+                                    int(x_bf16), out.data_ptr(), feat, int(out_bf16), n_rows, idx.shape[0], feat,
+                                    SPMM_MEAN if mean else 0, ws.data_ptr(), ws.numel(), _lib.current_stream(x.device))
+    _lib.check(st)
+    return out
+
+
 def clear_graph_cache():
     _C.clear_graph_cache()
 

@@ -15,6 +15,8 @@ GEMM_SPLIT_BF16X6 = 4
 GEMM_SPLIT_BF16X3 = 8
 GEMM_SPLIT_F16X3 = 16
 GEMM_ROUND_BF16 = 32
+GEMM_OUT_BF16 = 64
+WGRAD_A_BF16 = 128
 
 # How fp32 typed GEMMs multiply: "split_f16" (the default: rows of A and columns of W scaled by
 # powers of two and split into two fp16 parts, three fp16 MFMA products per fp32 product, 2^-21
@@ -50,7 +52,7 @@ def rel_segment(types, num_rel):
 
 
 def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n_out=None,
-               accumulate=False, atomic=False, bf16=False, precision=None):
+               accumulate=False, atomic=False, bf16=False, precision=None, out_bf16=False):
     """out[dst(i)] (=|+=) a[src(i)] @ w[r] for rows i of segment r (see cxg_typed_gemm_f32).
 
     a [*, K] fp32, w [R, K, N] fp32.  precision "split_f16" (the default, see
@@ -78,7 +80,12 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
                 raise ValueError("%s shorter than the number of rows" % name)
     if src_idx is None and a.shape[0] < m_rows:
         raise ValueError("a has fewer rows than M")
-    if out is None:
+    if out_bf16:
+        # bf16 rows of the result (the bf16-operand kernels only: K <= 128, even N, plain stores)
+        if out is not None or accumulate or atomic or not bf16 or K > 128 or K % 8 or N % 2:
+            raise ValueError("out_bf16 goes with bf16 operands, K <= 128 (a multiple of 8), even N and a fresh output")
+        out = torch.empty((m_rows if n_out is None else n_out, N), dtype=torch.bfloat16, device=a.device)
+    elif out is None:
         if n_out is None:
             n_out = m_rows
         out = torch.empty((n_out, N), dtype=torch.float32, device=a.device)
@@ -88,7 +95,7 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
             raise ValueError("output has %d columns, weights N=%d" % (out.shape[1], N))
     if dst_idx is None and out.shape[0] < m_rows:
         raise ValueError("output has fewer rows than M")
-    flags = (GEMM_ACCUMULATE if accumulate else 0) | (GEMM_ATOMIC if atomic else 0)
+    flags = (GEMM_ACCUMULATE if accumulate else 0) | (GEMM_ATOMIC if atomic else 0) | (GEMM_OUT_BF16 if out_bf16 else 0)
     precision = precision or GEMM_PRECISION
     if precision == "bf16":
         bf16 = True
@@ -103,7 +110,8 @@ def typed_gemm(a, w, seg_ptr, m_rows, *, src_idx=None, dst_idx=None, out=None, n
             _req(w, "weights", torch.float32, 3)
             st = lib.cxg_typed_gemm_f32(a.data_ptr(), K, w.data_ptr(), out.data_ptr(), N,
                                         _lib.ptr(src_idx), _lib.ptr(dst_idx), seg_ptr.data_ptr(),
-                                        m_rows, K, N, R, (flags & (GEMM_ACCUMULATE | GEMM_ATOMIC)) | GEMM_ROUND_BF16, stream)
+                                        m_rows, K, N, R,
+                                        (flags & (GEMM_ACCUMULATE | GEMM_ATOMIC | GEMM_OUT_BF16)) | GEMM_ROUND_BF16, stream)
         elif bf16:
             a16 = a if a.dtype == torch.bfloat16 else a.to(torch.bfloat16)
             wt16 = w.detach().transpose(1, 2).contiguous().to(torch.bfloat16)
@@ -349,7 +357,8 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     count, say) runs on a copy of g padded with zero columns.  Returns None when K is not a
     multiple of 4, which the kernel does not take."""
     lib = _lib.load()
-    _req(a, "a", torch.float32, 2)
+    a_bf16 = a.dtype == torch.bfloat16                      # rows of a in bf16 (widened exactly as they are staged)
+    _req(a, "a", torch.bfloat16 if a_bf16 else torch.float32, 2)
     _req(g, "g", torch.float32, 2)
     K, N = a.shape[1], g.shape[1]
     if K % 4:
@@ -361,6 +370,8 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     precision = precision or GEMM_PRECISION
     flags = (GEMM_SPLIT_F16X3 if precision == "split_f16" else
              GEMM_SPLIT_BF16X3 if precision in ("split3", "bf16") else GEMM_SPLIT_BF16X6)
+    flags |= WGRAD_A_BF16 if a_bf16 else 0
+    esz = 2 if a_bf16 else 4
     gw = torch.empty((num_rel, K, N), dtype=torch.float32, device=a.device)
     with torch.cuda.device(a.device):
         for k0 in range(0, K, 128):
@@ -368,7 +379,7 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
             direct = num_rel == 1 or kb == K
             part = gw if direct else torch.empty((num_rel, kb, N), dtype=torch.float32, device=a.device)
             ws = _workspace(lib.cxg_typed_gemm_wgrad_workspace_bytes(m_rows, kb, N, num_rel), a.device)
-            st = lib.cxg_typed_gemm_wgrad_f32(a.data_ptr() + 4 * k0, K, g.data_ptr(), N, _lib.ptr(src_idx),
+            st = lib.cxg_typed_gemm_wgrad_f32(a.data_ptr() + esz * k0, K, g.data_ptr(), N, _lib.ptr(src_idx),
                                               _lib.ptr(dst_idx), seg_ptr.data_ptr(), m_rows, kb, N, num_rel,
                                               part.data_ptr() + (4 * k0 * N if direct else 0), flags, ws.data_ptr(),
                                               ws.numel(), _lib.current_stream(a.device))
@@ -536,9 +547,22 @@ def _pairs_aggregate_first(pg, x, weights, idx, n, precision=None, mean_ptr=None
     _pair_graph_aggregate(pg, idx, n)
     n_pairs = pg.b_dst.shape[0]
     val = _pair_mean_weights(pg, mean_ptr, n)[0] if mean_ptr is not None else None
+    K, N = weights.shape[1], weights.shape[2]
+    if _bf16_tables(precision, K, N):
+        # the bf16 variant keeps its pair-row tables in bf16: the aggregation into the pair rows
+        # rounds as it stores, the typed GEMM reads and writes bf16 rows, the sum per destination
+        # gathers bf16 rows and adds in fp32 -- half the bytes on every pass over the tables
+        # (x itself is rounded once, 1 M rows, so that the 20 M row gathers move bf16 rows too)
+        z = _ops.spmm_bf16_rows(pg.bp_ptr, pg.bp_src, x.to(torch.bfloat16), n_pairs, val=val, out_bf16=True)   # [Ub, K] bf16
+        t = typed_gemm(z, weights, pg.b_seg, n_pairs, bf16=True, out_bf16=True)                  # [Ub, N] bf16
+        return _ops.spmm_bf16_rows(pg.dp_ptr, pg.dp_rows, t, n), z
     z = _ops.spmm(pg.bp_ptr, pg.bp_src, x, n_pairs, val=val)              # [Ub, K]
     t = typed_gemm(z, weights, pg.b_seg, n_pairs, precision=precision)                         # [Ub, N]
     return _ops.spmm(pg.dp_ptr, pg.dp_rows, t, n), z
+
+
+def _bf16_tables(precision, K, N):
+    return precision == "bf16" and K <= 128 and N <= 128 and K % 8 == 0 and N % 8 == 0
 
 
 def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w, precision=None, mean=False):
@@ -547,7 +571,12 @@ def _pairs_aggregate_first_bwd(pg, weights, z, grad_out, n_src, need_x, need_w, 
     input gradient repeats the weights)."""
     n_pairs = pg.b_dst.shape[0]
     gx = gw = None
-    if need_x:
+    if need_x and z.dtype == torch.bfloat16:
+        # bf16 tables (see _pairs_aggregate_first): the per-pair gradient rows are stored and gathered in bf16
+        gz = typed_gemm(grad_out.to(torch.bfloat16), weights.transpose(1, 2).contiguous(), pg.b_seg, n_pairs,
+                        src_idx=pg.b_dst, bf16=True, out_bf16=True)
+        gx = _ops.spmm_bf16_rows(pg.ptr_src, pg.b_row_rev, gz, n_src, val=pg.mean_rev if mean else None)
+    elif need_x:
         gz = typed_gemm(grad_out, weights.transpose(1, 2).contiguous(), pg.b_seg, n_pairs, src_idx=pg.b_dst,
                         precision=precision)
         gx = _ops.spmm(pg.ptr_src, pg.b_row_rev, gz, n_src, val=pg.mean_rev if mean else None)

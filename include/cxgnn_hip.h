@@ -135,6 +135,20 @@ int cxg_spmm_prereduce_f32(const int64_t* ptr, const int64_t* idx, const float* 
                            void* stream);
 
 /*
+ * Single-head aggregation (sum, CXG_SPMM_MEAN, or one weight per edge, optionally read through
+ * val_perm) of rows of 4 .. 128 values (a multiple of 4) whose rows are bf16 on the gathered
+ * side (x_bf16), on the stored side (out_bf16), or both; sums are formed in fp32 and rounded to
+ * nearest even when stored.  ldx / ldo count elements of the respective type.  Serves the bf16
+ * variant of the relational layer (MyRGCNConv(precision="bf16"), cxgnncomp/graph_conv.py:329-378,
+ * where the reference has an fp32 layer only): its pair-row tables are written and gathered at
+ * half the bytes.  Workspace: cxg_spmm_workspace_bytes(n_edges_cap, feat).
+ */
+int cxg_spmm_bf16_rows(const int64_t* ptr, const int64_t* idx, const float* val, const int64_t* val_perm,
+                       const void* x, int64_t ldx, int x_bf16, void* out, int64_t ldo, int out_bf16,
+                       int64_t n_rows, int64_t n_edges_cap, int feat, unsigned flags, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
  * cxg_spmm_weighted_f32 with bias[heads*channels] added to every output row as it is
  * stored (NULL: none; not with CXG_SPMM_MEAN): the `out + self.bias` that follows the
  * aggregation in MyGATConv.forward_many (cxgnncomp/graph_conv.py:488-494) without a second
@@ -286,6 +300,7 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
 #define CXG_GEMM_SPLIT_BF16X3 8u /* fp32 products as 3 bf16 partial products (2^-16 / product) */
 #define CXG_GEMM_SPLIT_F16X3 16u /* fp32 products as 3 fp16 partial products of row- / column-scaled operands (2^-21 / product) */
 #define CXG_GEMM_ROUND_BF16 32u /* fp32 operands rounded to bf16 as they are staged, one bf16 MFMA product, fp32 accumulation */
+#define CXG_GEMM_OUT_BF16 64u  /* the rows of C are bf16 (ldc in elements; `c` points to them): bf16-operand forms with K <= 128, even N and ldc, plain stores */
 
 /*
  * C[dst(i), :] = A[src(i), :] @ W[r] for the rows i in [seg_ptr[r], seg_ptr[r+1]),
@@ -385,6 +400,7 @@ int cxg_typed_gemm_wide_f32(const float* a, int64_t lda, const float* w, float* 
  * Replaces the per-relation torch.mm of TypedLinearE2EOP.backward and
  * TypedLinearS2DMMAggrOP.backward (cxgnncomp/typed_linear.py:114-137,205-221).
  */
+#define CXG_WGRAD_A_BF16 128u   /* the rows of A are bf16 (`a` points to them, lda in elements, 8-byte aligned rows) */
 size_t cxg_typed_gemm_wgrad_workspace_bytes(int64_t M, int K, int N, int R);
 int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_t ldg,
                              const int64_t* src_idx, const int64_t* dst_idx,
