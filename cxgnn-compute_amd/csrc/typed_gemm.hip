@@ -578,8 +578,9 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
   const int n_tiles = (int)((rows_here + kBM - 1) / kBM);
 
   // stores (or read-add-stores) of whole 16-byte pieces: this wave's 32 columns exist, rows are aligned
+  // (W too: the read-add-store loads of rows that do not exist are pointed at a 16-byte piece of W)
   const bool wide_store = KS <= 8 && !g.atomic && n0 + wave * 32 + 32 <= N && (g.ldc & 3) == 0 &&
-                          ((uintptr_t)g.c & 15) == 0 &&
+                          ((uintptr_t)g.c & 15) == 0 && ((uintptr_t)g.w & 15) == 0 &&
                           (!EPI || !g.addend || ((g.ldd & 3) == 0 && ((uintptr_t)g.addend & 15) == 0));
   // what a stored row is added to, if anything: the addend (epilogue entry point, never together
   // with accumulation) or the row of C itself

@@ -320,7 +320,9 @@ int cxg_csr_row_ids_i32(const int64_t* ptr, int64_t n_rows, int64_t n_edges, int
  * a*b is accumulated on v_mfma_f32_32x32x16_f16 from three partial products and the
  * scales are undone when the row is stored: 2^-21 per product, half the matrix
  * instructions and two thirds of the LDS traffic of X6; this form also takes
- * 176 <= K <= 256 when N >= 96.  Rows or columns whose largest
+ * 176 <= K <= 256 when N >= 96.  C (and the addend of the epilogue entry point) is
+ * written and re-read in 16-byte pieces when c, w and the addend are 16-byte aligned
+ * and ldc (ldd) is a multiple of 4, element by element otherwise.  Rows or columns whose largest
  * magnitude is below 2^-112 count as zero; a row holding an infinity or NaN comes out
  * non-finite.  With CXG_GEMM_ROUND_BF16 (K <= 128, K and lda multiples of 8) the fp32
  * operands are rounded to bf16 (nearest even) on their way into the LDS and the

@@ -322,6 +322,36 @@ def test_typed_gemm_wgrad_scaled_fp16_dynamic_range(K, N, M):
         assert ok.all(), "relation %d: worst error / sum|a||g| = %.3e" % (r, float((err / mag.clamp_min(1e-300))[~ok].max()))
 
 
+def test_typed_gemm_wgrad_scaled_fp16_columns_of_different_scale():
+    """The weight gradient's fp16 parts share one power-of-two scale per group of 32 columns, so a
+    column far below the largest column of its group keeps fewer significant bits: the two parts
+    of a scaled value resolve 2^-24 absolute, i.e. 2^-37 of the group's largest magnitude with the
+    three bits of headroom.  Columns at 1, 2^-10, 2^-20 and 2^-30 of their group's scale, in
+    either operand: down to 2^-20 every gw element stays within 4e-6 of sum_i |a||g| of its own
+    reduction (measured 1.5e-7); at 2^-30 the bound is 2^-37 / 2^-30 = 8e-3 per product and 5e-4
+    is asserted on the sum (measured 1.4e-4).  The six-product bf16 form carries no shared scale
+    and stays at 2e-8 for every column (asserted at 4e-7)."""
+    from cxgnncomp_backend import _typed
+    K, N, M, R = 128, 128, 30000, 2
+    gen = torch.Generator().manual_seed(1)
+    ea = torch.tensor([0, 10, 20, 30])[torch.arange(K) % 4]
+    eg = torch.tensor([0, 10, 20, 30])[(torch.arange(N) // 2) % 4]
+    a = torch.randn(M, K, generator=gen) * torch.exp2(-ea.float())
+    g = torch.randn(M, N, generator=gen) * torch.exp2(-eg.float())
+    seg = torch.tensor([0, M // 2, M], dtype=torch.int64)
+    low = torch.maximum(ea[:, None], eg[None, :])
+    for precision, bound_near, bound_far in (("split_f16", 4e-6, 5e-4), ("split6", 4e-7, 4e-7)):
+        announce("typed_gemm_wgrad %s, columns at 2^0..2^-30 of their group's scale" % precision)
+        gw = _typed.typed_gemm_wgrad(a.cuda(), g.cuda(), seg.cuda(), M, R, precision=precision).cpu().double()
+        for r in range(R):
+            b, e = int(seg[r]), int(seg[r + 1])
+            want = a[b:e].double().t() @ g[b:e].double()
+            mag = a[b:e].double().abs().t() @ g[b:e].double().abs()
+            rel = (gw[r] - want).abs() / mag
+            assert float(rel[low <= 20].max()) <= bound_near, (precision, float(rel[low <= 20].max()))
+            assert float(rel[low == 30].max()) <= bound_far, (precision, float(rel[low == 30].max()))
+
+
 @pytest.mark.parametrize("M", [1, 63, 64, 65, 1100])
 @pytest.mark.parametrize("K,N", [(128, 128), (4, 4), (36, 72), (256, 96)])
 def test_typed_gemm_small_shapes_and_skipped_rows(M, K, N):

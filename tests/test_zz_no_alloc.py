@@ -59,6 +59,54 @@ def test_noalloc_matches_workspace_entry_point_twice():
         assert_close(got.cpu().numpy(), ref, 1e-4, 1e-5, "noalloc %s vs oracle" % name)
 
 
+def test_noalloc_allocates_nothing_and_runs_on_the_callers_stream():
+    """A call leaves the device's free memory and torch's allocator counters where they were
+    (the property the entry point exists for), and its kernels run on the stream it is given:
+    on a side stream the input rows are written behind a long spin kernel, the call follows on
+    the same stream and a dependent copy after it; had the kernels run on any other stream
+    they would have gathered the zeros the rows held before."""
+    from cxgnncomp_backend import _lib as L
+    from cxgnncomp import synthetic as S
+    lib = L.load()
+    dev = torch.device("cuda:0")
+    ptr, idx = S.powerlaw_directed_symmetrised(30000, 300000, max_degree=5000, seed=9)
+    n, feat = ptr.shape[0] - 1, 128
+    torch.manual_seed(3)
+    x = torch.randn(n, feat) / 30
+    ptr_d, idx_d, x_d = ptr.to(dev), idx.to(dev), x.to(dev)
+    out = torch.full((n, feat), float("nan"), device=dev)
+    args = (ptr_d.data_ptr(), idx_d.data_ptr(), x_d.data_ptr(), feat, out.data_ptr(), feat, n, idx.shape[0], feat, 0)
+    announce("noalloc memory counters around a call, n=%d E=%d" % (n, idx.shape[0]))
+    L.check(lib.cxg_spmm_sum_f32_noalloc(*args, L.current_stream(dev)))          # first call: symbol lookup
+    torch.cuda.synchronize()
+
+    def counters():
+        st = torch.cuda.memory_stats(dev)
+        return (st["allocation.all.allocated"], st["allocation.all.freed"], st["segment.all.allocated"],
+                st["segment.all.freed"], torch.cuda.mem_get_info(dev)[0])
+    before = counters()
+    L.check(lib.cxg_spmm_sum_f32_noalloc(*args, L.current_stream(dev)))
+    torch.cuda.synchronize()
+    assert counters() == before, "the call changed the allocator's counters or the device's free memory"
+    want = out.clone()
+
+    announce("noalloc on a side stream behind a spin kernel")
+    stale = torch.zeros_like(x_d)
+    out2 = torch.full((n, feat), float("nan"), device=dev)
+    side = torch.cuda.Stream(device=dev)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(50_000_000)                 # tens of milliseconds of spinning on `side`
+        stale.copy_(x_d)                              # the rows arrive behind it
+        L.check(lib.cxg_spmm_sum_f32_noalloc(ptr_d.data_ptr(), idx_d.data_ptr(), stale.data_ptr(), feat,
+                                             out2.data_ptr(), feat, n, idx.shape[0], feat, 0,
+                                             L.current_stream(dev)))
+        got = out2.clone()                            # dependent read on the same stream
+    side.synchronize()
+    assert torch.equal(got, want), "the call did not run in order on the stream it was given"
+    torch.cuda.synchronize()
+
+
 def test_noalloc_rejects_shapes_beyond_the_scratch():
     from cxgnncomp_backend import _lib as L
     lib = L.load()
