@@ -624,8 +624,8 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_fwd_walk_kernel(
 template <int H>
 __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
     const int64_t* __restrict__ ptr, const float* __restrict__ out, const uint8_t* __restrict__ mask,
-    const float* __restrict__ grad, float* __restrict__ g_dst, float* __restrict__ t_edge,
-    int64_t n_rows, int heads, float slope) {
+    const float* __restrict__ grad, const int64_t* __restrict__ gpos, float* __restrict__ g_dst,
+    float* __restrict__ t_edge, int64_t n_rows, int heads, float slope) {
   const int nh = H > 0 ? H : heads;
   constexpr int HB = H > 0 ? H : 1;
   for (int h0 = 0; h0 < nh; h0 += HB) {
@@ -640,7 +640,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
           kk[u] = k + u * stride;
           const int64_t c = kk[u] < e ? kk[u] : first;
           load_f<HB>(out + c * nh + h0, o[u]);
-          load_f<HB>(grad + c * nh + h0, g[u]);
+          load_f<HB>(grad + (gpos ? gpos[c] : c) * nh + h0, g[u]);
         }
 #pragma unroll
         for (int u = 0; u < kU; ++u)
@@ -662,7 +662,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
           kk[u] = k + u * stride;
           const int64_t c = kk[u] < e ? kk[u] : first;
           load_f<HB>(out + c * nh + h0, o[u]);
-          load_f<HB>(grad + c * nh + h0, g[u]);
+          load_f<HB>(grad + (gpos ? gpos[c] : c) * nh + h0, g[u]);
           load_b<HB>(mask + c * nh + h0, mk[u]);
         }
 #pragma unroll
@@ -712,11 +712,12 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_kernel(
 // Backward as an edge-parallel walk (see SegmentWalk): s = sum_row out*g, then
 // t = out*(g-s)*(mask ? 1 : slope) per edge and g_dst = sum_row t where the row has both
 // signs.
-template <int H>
+// AT: the gradient row of edge k sits at grad[gpos[k]] (the producer wrote it in another edge order).
+template <int H, bool AT>
 __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_walk_kernel(
     const int64_t* __restrict__ ptr, const float* __restrict__ out, const uint8_t* __restrict__ mask,
-    const float* __restrict__ grad, float* __restrict__ g_dst, float* __restrict__ t_edge,
-    int64_t n_rows, float slope) {
+    const float* __restrict__ grad, const int64_t* __restrict__ gpos, float* __restrict__ g_dst,
+    float* __restrict__ t_edge, int64_t n_rows, float slope) {
   const int lane = lane_id();
   const int64_t block_row0 = (int64_t)blockIdx.x * kBlock;
   const int64_t first_row = block_row0 + (int64_t)uniform_i32(threadIdx.x >> 6) * CXG_WAVE;
@@ -736,7 +737,10 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_walk_kernel(
     const int64_t k = w.eb + (rel < w.total ? rel : w.total - 1);
     float o[H], g[H], v[H];
     load_f<H>(out + k * H, o);
-    load_f<H>(grad + k * H, g);
+    load_f<H>(grad + (AT ? gpos[k] : k) * H, g);
+    // AT: one gather per edge -- the row is left at the edge's own place in t_edge, where the
+    // same lane finds it in sweep 2 before it overwrites it
+    if (AT && rel < w.total) store_f<H>(t_edge + k * H, g);
 #pragma unroll
     for (int h = 0; h < H; ++h) v[h] = o[h] * g[h];
     segment_scan(v, lane, lo, OpSum());
@@ -758,7 +762,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_walk_kernel(
     float o[H], g[H], t[H];
     bool mk[H];
     load_f<H>(out + k * H, o);
-    load_f<H>(grad + k * H, g);
+    load_f<H>((AT ? t_edge : grad) + k * H, g);
     load_b<H>(mask + k * H, mk);
     w.own_segment(at, first, last);
     const uint64_t own = last < 0 ? 0ull : ((~0ull >> (CXG_WAVE - 1 - last)) & (~0ull << first));
@@ -799,13 +803,15 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_walk_kernel(
         kk[u] = k + u * sc.nl;
         const int64_t c = kk[u] < e ? kk[u] : b + sc.li;
         load_f<H>(out + c * H, o[u]);
-        load_f<H>(grad + c * H, g[u]);
+        load_f<H>(grad + (AT ? gpos[c] : c) * H, g[u]);
       }
 #pragma unroll
       for (int u = 0; u < kU; ++u)
-        if (kk[u] < e)
+        if (kk[u] < e) {
+          if (AT) store_f<H>(t_edge + kk[u] * H, g[u]);
 #pragma unroll
           for (int h = 0; h < H; ++h) bs[h] += o[u][h] * g[u][h];
+        }
     }
     sc.template sum_n<H>(bs);
     for (int64_t k = b + sc.li; k < e; k += kU * sc.nl) {
@@ -817,7 +823,7 @@ __global__ __launch_bounds__(kBlock) void edge_softmax_bwd_walk_kernel(
         kk[u] = k + u * sc.nl;
         const int64_t c = kk[u] < e ? kk[u] : b + sc.li;
         load_f<H>(out + c * H, o[u]);
-        load_f<H>(grad + c * H, g[u]);
+        load_f<H>((AT ? t_edge : grad) + c * H, g[u]);
         load_b<H>(mask + c * H, mk[u]);
       }
 #pragma unroll
@@ -917,28 +923,40 @@ int cxg_edge_softmax_fwd_f32(const int64_t* ptr, const int64_t* idx, const float
   return CXG_OK;
 }
 
-int cxg_edge_softmax_bwd_f32(const int64_t* ptr, const float* out, const uint8_t* mask,
-                             const float* grad, float* g_dst, float* t_edge, int64_t n_dst, int heads,
-                             float slope, void* stream) {
+int cxg_edge_softmax_bwd_at_f32(const int64_t* ptr, const float* out, const uint8_t* mask,
+                                const float* grad, const int64_t* grad_pos, float* g_dst, float* t_edge,
+                                int64_t n_dst, int heads, float slope, void* stream) {
   CXG_REQUIRE(n_dst >= 0 && heads >= 1, CXG_ERR_ARG, "bad n_dst/heads");
   if (n_dst == 0) return CXG_OK;
   CXG_REQUIRE(ptr && g_dst, CXG_ERR_ARG, "null ptr/g_dst");
   CXG_REQUIRE(out && mask && grad && t_edge, CXG_ERR_ARG, "null out/mask/grad/t_edge");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   dim3 grid = cxg::row_grid(n_dst), block(cxg::kBlock);
-#define CXG_BWD(HH)                                                                              \
-  hipLaunchKernelGGL(cxg::edge_softmax_bwd_walk_kernel<HH>, grid, block, 0, st, ptr, out, mask, grad, \
-                     g_dst, t_edge, n_dst, slope)
+#define CXG_BWD(HH)                                                                                  \
+  do {                                                                                               \
+    if (grad_pos)                                                                                    \
+      hipLaunchKernelGGL((cxg::edge_softmax_bwd_walk_kernel<HH, true>), grid, block, 0, st, ptr, out, mask, \
+                         grad, grad_pos, g_dst, t_edge, n_dst, slope);                               \
+    else                                                                                             \
+      hipLaunchKernelGGL((cxg::edge_softmax_bwd_walk_kernel<HH, false>), grid, block, 0, st, ptr, out, mask, \
+                         grad, grad_pos, g_dst, t_edge, n_dst, slope);                               \
+  } while (0)
   if (heads == 1) CXG_BWD(1);
   else if (heads == 2) CXG_BWD(2);
   else if (heads == 4) CXG_BWD(4);
   else if (heads == 8) CXG_BWD(8);
   else
-    hipLaunchKernelGGL(cxg::edge_softmax_bwd_kernel<0>, grid, block, 0, st, ptr, out, mask, grad, g_dst,
-                       t_edge, n_dst, heads, slope);
+    hipLaunchKernelGGL(cxg::edge_softmax_bwd_kernel<0>, grid, block, 0, st, ptr, out, mask, grad, grad_pos,
+                       g_dst, t_edge, n_dst, heads, slope);
 #undef CXG_BWD
   CXG_LAUNCH_CHECK("edge_softmax_bwd_kernel");
   return CXG_OK;
+}
+
+int cxg_edge_softmax_bwd_f32(const int64_t* ptr, const float* out, const uint8_t* mask,
+                             const float* grad, float* g_dst, float* t_edge, int64_t n_dst, int heads,
+                             float slope, void* stream) {
+  return cxg_edge_softmax_bwd_at_f32(ptr, out, mask, grad, nullptr, g_dst, t_edge, n_dst, heads, slope, stream);
 }
 
 int cxg_narrow_gather_sum_f32(const int64_t* ptr, const int64_t* sel, const float* in, float* out,

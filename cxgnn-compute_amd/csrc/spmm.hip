@@ -101,6 +101,7 @@ struct SpmmArgs {
   const float* dot_b;
   int64_t ld_dot_b;
   float* dot_out;
+  int dot_at_edge;         // dot_out rows at the edge's own position although val is read through perm
   const float* bias;       // [F] added to every output row, or null
   int out_bf16;            // the rows of `out` are bf16 (grouped-lane kernel with IO & 2, and its fix-up launch)
 };
@@ -369,7 +370,7 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
       // complete in order, so every scattered store held up the next gathers)
       __builtin_amdgcn_wave_barrier();
       if (lane < cn) {
-        const int64_t vrow = PERM ? my_vrow : (e0 + c0 + lane);
+        const int64_t vrow = (PERM && !a.dot_at_edge) ? my_vrow : (e0 + c0 + lane);
         float* dst = a.dot_out + vrow * a.heads + blockIdx.y * kDotHeads;
         const float* src = &s_dot[wave][lane * kDotHeads];
         if constexpr (kDotHeads == 8) {
@@ -937,6 +938,7 @@ struct SpmmDot {
   const float* b = nullptr;     // [n_rows, heads, channels], row stride ld_b
   int64_t ld_b = 0;
   float* out = nullptr;         // [n_val_rows, heads]
+  bool at_edge = false;         // rows of `out` at the edge's position in idx, not at perm[position]
 };
 
 template <typename IdxT>
@@ -973,7 +975,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
   a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
   a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0;
   a.src_map = nullptr; a.targets = nullptr;
-  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr;
+  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr; a.dot_at_edge = 0;
   a.bias = bias;
   a.out_bf16 = 0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -996,7 +998,7 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
                       (channels == 32 || channels == 64 || channels == 128 || channels == 256),
                   CXG_ERR_UNSUPPORTED, "spmm with dot products needs heads*channels %% 256 == 0, channels in "
                   "{32, 64, 128, 256} and 16-byte aligned rows");
-      a.dot_b = dot->b; a.ld_dot_b = dot->ld_b; a.dot_out = dot->out;
+      a.dot_b = dot->b; a.ld_dot_b = dot->ld_b; a.dot_out = dot->out; a.dot_at_edge = dot->at_edge ? 1 : 0;
 #define CXG_DOT(WM, GG)                                                                          \
   return perm ? launch_spmm<IdxT, 4, false, WM, true, false, GG>(a, plan.n_spans_cap, st)          \
               : launch_spmm<IdxT, 4, false, WM, false, false, GG>(a, plan.n_spans_cap, st)
@@ -1145,7 +1147,7 @@ int cxg_spmm_bf16_rows(const int64_t* ptr, const int64_t* idx, const float* val,
   a.tail_row = reinterpret_cast<int64_t*>(workspace);
   a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
   a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0; a.src_map = nullptr; a.targets = nullptr;
-  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr; a.bias = nullptr; a.out_bf16 = out_bf16 ? 1 : 0;
+  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr; a.dot_at_edge = 0; a.bias = nullptr; a.out_bf16 = out_bf16 ? 1 : 0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int lanes = feat / 4;
   int L = 4;
@@ -1197,8 +1199,9 @@ int cxg_spmm_weighted_dot_f32(const int64_t* ptr, const int64_t* idx, const floa
   if (!val) return cxg::set_error(CXG_ERR_ARG, "val is null");
   cxg::SpmmDot dot;
   dot.b = dot_b; dot.ld_b = ld_dot_b; dot.out = dot_out;
+  dot.at_edge = (flags & CXG_SPMM_DOT_AT_EDGE) != 0;
   return cxg::spmm_common<int64_t>(ptr, idx, val, val_perm, x, ldx, out, ldo, n_rows, n_edges_cap,
-                                   heads, channels, flags, workspace, workspace_bytes, stream, nullptr, &dot);
+                                   heads, channels, flags & ~CXG_SPMM_DOT_AT_EDGE, workspace, workspace_bytes, stream, nullptr, &dot);
 }
 
 int cxg_spmm_ext_f32(const int64_t* ptr, const int64_t* idx, const float* x, int64_t ldx, float* out,

@@ -274,7 +274,7 @@ struct TransposedGraph {
   Tensor ptr_t, idx_t, perm;        // rows = source nodes, idx_t = destination ids, perm = original edge position
   int64_t n_edges = 0, n_src = 0, n_dst = 0;
   Tensor keep_ptr, keep_idx;        // the tensors the key was made from stay alive while cached
-  OptTensor inv_deg_t, rows32;      // filled on first use, under fill_mu (a cached graph is shared between threads)
+  OptTensor inv_deg_t, rows32, inv_perm;   // filled on first use, under fill_mu (a cached graph is shared between threads)
   std::mutex fill_mu;
 };
 using GraphPtr = std::shared_ptr<TransposedGraph>;
@@ -593,20 +593,40 @@ std::tuple<Tensor, Tensor> edge_softmax_fwd(const Tensor& ptr, const Tensor& idx
 }
 
 // (g_dst [n_dst, H], t_edge [E, H]); rows of t_edge at or past ptr[n_dst] are not written.
+// grad_pos (optional, int64 per edge): the gradient row of edge k is grad[grad_pos[k]].
 std::tuple<Tensor, Tensor> edge_softmax_bwd(const Tensor& ptr, const Tensor& out, const Tensor& mask, const Tensor& grad,
-                                            int64_t n_dst, double slope) {
+                                            int64_t n_dst, double slope, const OptTensor& grad_pos = c10::nullopt) {
   req(out, "out", at::kFloat, {2});
   req(grad, "grad", at::kFloat, {2});
   req(mask, "mask", at::kBool, {2});
   const int64_t heads = out.size(1);
   Tensor g_dst = torch::empty({n_dst, heads}, out.options());
   Tensor t_edge = torch::empty_like(out);
+  if (grad_pos.has_value()) {
+    req(*grad_pos, "grad_pos", at::kLong, {1});
+    if (n_dst + 1 > ptr.size(0)) bad("num rows does not fit ptr");
+  }
   c10::DeviceGuard guard(out.device());
-  check(cxg_edge_softmax_bwd_f32((const int64_t*)ptr.data_ptr(), (const float*)ptr_or_null(out),
-                                 (const uint8_t*)ptr_or_null(mask), (const float*)ptr_or_null(grad),
-                                 (float*)ptr_or_null(g_dst), (float*)ptr_or_null(t_edge), n_dst, (int)heads, (float)slope,
-                                 stream_of(out)));
+  check(cxg_edge_softmax_bwd_at_f32((const int64_t*)ptr.data_ptr(), (const float*)ptr_or_null(out),
+                                    (const uint8_t*)ptr_or_null(mask), (const float*)ptr_or_null(grad),
+                                    grad_pos.has_value() ? (const int64_t*)ptr_or_null(*grad_pos) : nullptr,
+                                    (float*)ptr_or_null(g_dst), (float*)ptr_or_null(t_edge), n_dst, (int)heads,
+                                    (float)slope, stream_of(out)));
   return std::make_tuple(g_dst, t_edge);
+}
+
+// Position in the transposed order of every original edge position (the inverse of perm; kept
+// with the graph): what a consumer walking the original order needs to read rows that were stored
+// in the transposed order.
+Tensor inverse_perm_transposed(TransposedGraph& g) {
+  std::lock_guard<std::mutex> lock(g.fill_mu);
+  if (!g.inv_perm.has_value()) {
+    c10::DeviceGuard guard(g.perm.device());
+    Tensor inv = torch::empty({g.n_edges}, g.perm.options());
+    if (g.n_edges > 0) inv.index_put_({g.perm}, torch::arange(g.n_edges, g.perm.options()));
+    g.inv_perm = inv;
+  }
+  return *g.inv_perm;
 }
 
 // out[r,:] = sum_{k in row r} inp[sel[k],:] (sel undefined: inp[k,:]); inp [M] or [M, W].  With
@@ -913,7 +933,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("n_rows"), py::arg("out") = py::none());
   m.def("sddmm_coo", &sddmm_coo);
   m.def("edge_softmax_fwd", &edge_softmax_fwd);
-  m.def("edge_softmax_bwd", &edge_softmax_bwd);
+  m.def("edge_softmax_bwd", &edge_softmax_bwd, py::arg("ptr"), py::arg("out"), py::arg("mask"), py::arg("grad"),
+        py::arg("n_dst"), py::arg("slope"), py::arg("grad_pos") = py::none());
+  m.def("inverse_perm_transposed", [](const GraphPtr& g) { return inverse_perm_transposed(*g); });
   m.def("narrow_gather_sum", &narrow_gather_sum, py::arg("ptr"), py::arg("sel"), py::arg("inp"), py::arg("n_rows"),
         py::arg("rows32") = py::none());
   m.def("csr_transpose", &csr_transpose, py::arg("ptr"), py::arg("idx"), py::arg("n_rows"), py::arg("n_src"),

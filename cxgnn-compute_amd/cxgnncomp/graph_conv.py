@@ -515,12 +515,16 @@ class GatLayerOP(torch.autograd.Function):
         if tg.n_edges < ev.shape[0]:
             g_ev[tg.n_edges:].zero_()
         if _ops.spmm_dot_supported(H, C):
-            # one pass over the reversed graph gathers the rows of g once for both results
-            g_xs, g_ev = _ops.spmm_dot(tg.ptr_t, tg.idx_t, g3, xs.shape[0], ev, tg.perm, xs, g_ev)
+            # one pass over the reversed graph gathers the rows of g once for both results; the
+            # edge-value gradient stays in that pass's edge order (contiguous stores) and the
+            # softmax backward reads it through the inverse permutation
+            g_xs, g_ev = _ops.spmm_dot(tg.ptr_t, tg.idx_t, g3, xs.shape[0], ev, tg.perm, xs, g_ev, dot_at_edge=True)
+            g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope,
+                                                   grad_pos=_ops.inverse_perm_transposed(tg))
         else:
             g_xs = _ops.spmm(tg.ptr_t, tg.idx_t, g3, xs.shape[0], val=ev, val_perm=tg.perm)
             g_ev = _ops.sddmm_csr(ptr, idx, xs, g3, num_dst, out=g_ev)
-        g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope)
+            g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope)
         g_asrc = _ops.narrow_gather_sum(tg.ptr_t, tg.perm, t_edge, xs.shape[0], rows32=_ops.rows32_transposed(tg))
         _, g_att_src, g_att_dst = _ops.attention_logits_bwd(xs, att_src, att_dst, g_asrc, g_adst, add_to=g_xs)
         g_xs2 = g_xs.view(-1, H * C)

@@ -53,6 +53,7 @@ SIGNATURES = {
     "cxg_sddmm_coo_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "cxg_edge_softmax_fwd_f32": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I32, _F32, _P]),
     "cxg_edge_softmax_bwd_f32": (_I32, [_P, _P, _P, _P, _P, _P, _I64, _I32, _F32, _P]),
+    "cxg_edge_softmax_bwd_at_f32": (_I32, [_P, _P, _P, _P, _P, _P, _P, _I64, _I32, _F32, _P]),
     "cxg_narrow_gather_sum_f32": (_I32, [_P, _P, _P, _P, _I64, _I32, _P]),
     "cxg_scatter_add_rows_f32": (_I32, [_P, _P, _P, _I64, _I32, _P]),
     "cxg_gather_rows_f32": (_I32, [_P, _P, _P, _I64, _I32, _P]),

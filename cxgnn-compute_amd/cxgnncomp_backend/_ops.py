@@ -16,6 +16,7 @@ _C = _native()
 SPMM_MEAN = 1
 SPMM_ACCUMULATE = 2
 SPMM_HINT_EXACT_EDGES = 4
+SPMM_DOT_AT_EDGE = 8
 
 
 def as_int(v):
@@ -67,9 +68,10 @@ def spmm_dot_supported(heads, channels):
     return (heads * channels) % 256 == 0 and channels in (32, 64, 128, 256)
 
 
-def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out):
+def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out, dot_at_edge=False):
     """Weighted multi-head SpMM that also stores, for every edge e of output row r,
-    dot_out[vrow(e), h] = <x[idx[e], h, :], dot_b[r, h, :]> (vrow(e) = val_perm[e], or e):
+    dot_out[vrow(e), h] = <x[idx[e], h, :], dot_b[r, h, :]> (vrow(e) = val_perm[e], or e; with
+    ``dot_at_edge`` always e, the position in idx: contiguous stores):
     (out [n_rows, H, C], dot_out).  x [n_src, H, C], val [*, H], dot_b [>= n_rows, H, C],
     dot_out [*, H] (the entries of the edges of the first n_rows rows are written)."""
     lib = _lib.load()
@@ -100,6 +102,8 @@ def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out):
         return out, dot_out
     ws = _workspace(lib.cxg_spmm_workspace_bytes(idx.shape[0], row), x.device)
     flags = SPMM_HINT_EXACT_EDGES if n_rows == ptr.shape[0] - 1 else 0
+    if dot_at_edge:
+        flags |= SPMM_DOT_AT_EDGE
     with torch.cuda.device(x.device):
         st = lib.cxg_spmm_weighted_dot_f32(ptr.data_ptr(), _lib.ptr(idx), val.data_ptr(), _lib.ptr(val_perm),
                                            _lib.ptr(x), row, out.data_ptr(), row, _lib.ptr(dot_b), row,
@@ -246,10 +250,12 @@ def edge_softmax_fwd(ptr, idx, att_dst, att_src, n_edges, slope):
     return _C.edge_softmax_fwd(ptr, idx, att_dst, att_src, int(n_edges), float(slope))
 
 
-def edge_softmax_bwd(ptr, out, mask, grad, n_dst, slope):
+def edge_softmax_bwd(ptr, out, mask, grad, n_dst, slope, grad_pos=None):
     """Returns (g_dst [n_dst,H], t_edge [E,H]); rows of t_edge at or past ptr[n_dst] are not
-    written (the transposed gather that consumes t_edge never reads them)."""
-    return _C.edge_softmax_bwd(ptr, out, mask, grad, int(n_dst), float(slope))
+    written (the transposed gather that consumes t_edge never reads them).  With ``grad_pos``
+    (int64 per edge) the gradient row of edge k is grad[grad_pos[k]]: a gradient that was stored
+    in the transposed graph's edge order is read through ``inverse_perm_transposed``."""
+    return _C.edge_softmax_bwd(ptr, out, mask, grad, int(n_dst), float(slope), grad_pos)
 
 
 def attention_logits(x, att_src, att_dst, n_dst):
@@ -407,6 +413,12 @@ def csr_row_ids32(ptr, n_rows, n_edges):
 def rows32_transposed(g):
     """Row (source) id of every edge of a TransposedGraph, built once and kept with it."""
     return _C.rows32_transposed(g)
+
+
+def inverse_perm_transposed(g):
+    """Position in the transposed edge order of every original edge position of a
+    TransposedGraph (the inverse of ``g.perm``), built once and kept with it."""
+    return _C.inverse_perm_transposed(g)
 
 
 def narrow_gather_sum(ptr, sel, inp, n_rows, rows32=None):

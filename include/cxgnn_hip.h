@@ -51,6 +51,7 @@ const char* cxg_last_error(void);
 #define CXG_SPMM_MEAN 1u       /* divide each row by its degree; empty rows stay 0 */
 #define CXG_SPMM_ACCUMULATE 2u /* out += result instead of out = result           */
 #define CXG_SPMM_HINT_EXACT_EDGES 4u /* n_edges_cap is the real edge count of the rows (tuning hint only) */
+#define CXG_SPMM_DOT_AT_EDGE 8u /* cxg_spmm_weighted_dot_f32 only: dot_out rows at the edge's position in idx although val is read through val_perm */
 
 /* Bytes of workspace needed by cxg_spmm_* for a graph whose idx array has
  * n_edges_cap entries and rows of `row_floats` floats (heads*channels). */
@@ -170,6 +171,10 @@ int cxg_spmm_weighted_bias_f32(const int64_t* ptr, const int64_t* idx, const flo
  * spmm_multihead_bwd + run_sddmm of SpMMValOP.backward (cxgnncomp/graph_kernel.py:20-37,
  * src/cpp/src/spmm_host.cu:198-214, src/cpp/src/sddmm_host.cu:4-14).  dot_b is
  * [n_rows, heads, channels] with row stride ld_dot_b, dot_out [n_val_rows, heads].
+ * With CXG_SPMM_DOT_AT_EDGE the row of edge position k (in idx) is dot_out[k] whether or
+ * not val is read through val_perm: contiguous stores instead of one scattered 16-byte
+ * store per edge (a consumer then reads row e of the original order at the inverse
+ * permutation's position, see cxg_edge_softmax_bwd_at_f32).
  * Shapes: heads*channels a multiple of 256, channels in {32, 64, 128, 256}, 16-byte
  * aligned rows (CXG_ERR_UNSUPPORTED otherwise: use the two separate calls).
  */
@@ -264,6 +269,18 @@ int cxg_edge_softmax_fwd_f32(const int64_t* ptr, const int64_t* idx,
 int cxg_edge_softmax_bwd_f32(const int64_t* ptr, const float* out, const uint8_t* mask,
                              const float* grad, float* g_dst, float* t_edge,
                              int64_t n_dst, int heads, float slope, void* stream);
+
+/*
+ * The same backward (src/cpp/src/edge_softmax.cu:44-95) when the incoming gradient was
+ * written in another edge order: the row of edge k is grad[grad_pos[k]] (grad_pos NULL:
+ * grad[k], i.e. cxg_edge_softmax_bwd_f32).  With grad_pos = the inverse of a transposed
+ * CSR's edge permutation it consumes what cxg_spmm_weighted_dot_f32 stored with
+ * CXG_SPMM_DOT_AT_EDGE: one 16-byte gather per edge here instead of one scattered store
+ * per edge there.  out, mask, t_edge and g_dst are in the order of ptr as before.
+ */
+int cxg_edge_softmax_bwd_at_f32(const int64_t* ptr, const float* out, const uint8_t* mask,
+                                const float* grad, const int64_t* grad_pos, float* g_dst,
+                                float* t_edge, int64_t n_dst, int heads, float slope, void* stream);
 
 /* out[r, 0..width) = sum_{k in [ptr[r], ptr[r+1])} in[sel ? sel[k] : k, 0..width)
  * for narrow rows (a few floats).  With width 1 and sel = idx this is spmv

@@ -315,6 +315,41 @@ def test_spmm_with_edge_dot_products(kind, shape):
     out2, dot2 = _ops.spmm_dot(pc, ic, xs.cuda(), n, ev.cuda(), None, g.cuda(), dot2)
     assert torch.equal(out2, _ops.spmm(pc, ic, xs.cuda(), n, val=ev.cuda()))
     assert_close(_np(dot2), ref.reshape(E, H), RTOL, ATOL, "edge dot products, CSR order")
+    # products left in the transposed graph's edge order (contiguous stores): the same values,
+    # row k of this result is row perm[k] of the first
+    dot3 = torch.full((E, H), float("nan"), device="cuda")
+    gx3, dot3 = _ops.spmm_dot(tg.ptr_t, tg.idx_t, g.cuda(), n, ev.cuda(), tg.perm, xs.cuda(), dot3, dot_at_edge=True)
+    assert torch.equal(gx3, want_gx)
+    assert torch.equal(dot3, dot[tg.perm])
+    inv = _ops.inverse_perm_transposed(tg)
+    assert torch.equal(inv[tg.perm], torch.arange(E, device="cuda"))
+    assert torch.equal(dot3[inv], dot)
+
+
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
+@pytest.mark.parametrize("heads", [1, 2, 4, 8, 3])
+def test_edge_softmax_backward_reads_the_gradient_through_positions(kind, heads):
+    """cxg_edge_softmax_bwd_at_f32: with the gradient rows stored in another edge order and the
+    position of every edge's row handed over, the result is bit for bit that of
+    cxg_edge_softmax_bwd_f32 on the gradient in CSR order (the walk kernels of 1, 2, 4, 8 heads
+    and the row kernel for other head counts)."""
+    from cxgnncomp_backend import _ops
+    ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    gen = torch.Generator().manual_seed(heads + 17)
+    pc, ic = ptr.cuda(), idx.cuda()
+    out, mask = _ops.edge_softmax_fwd(pc, ic, torch.randn(n, heads, generator=gen).cuda(),
+                                      torch.randn(n, heads, generator=gen).cuda(), E, 0.2)
+    grad = torch.randn(E, heads, generator=gen).cuda()
+    where = torch.randperm(E, generator=gen).cuda()            # edge k's row sits at where[k]
+    moved = torch.empty_like(grad)
+    moved[where] = grad
+    announce("edge_softmax_bwd with gradient positions kind=%s H=%d" % (kind, heads))
+    gd, te = _ops.edge_softmax_bwd(pc, out, mask, grad, n, 0.2)
+    gd2, te2 = _ops.edge_softmax_bwd(pc, out, mask, moved, n, 0.2, grad_pos=where)
+    torch.cuda.synchronize()
+    assert torch.equal(gd, gd2) and torch.equal(te, te2)
 
 
 @pytest.mark.parametrize("feat", [1, 2, 4, 8, 3, 16, 100])
