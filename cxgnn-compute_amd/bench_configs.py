@@ -270,7 +270,17 @@ def c3(iters):
     report("c3", "spmm_multihead_bwd + edge-value grad in one pass (spmm_dot) H=4 C=64",
            timeit(lambda: _ops.spmm_dot(gt.ptr_t, gt.idx_t, g, N, ev, gt.perm, x, gev), iters),
            spmm_bytes(N, E, H * C, H) + 8 * E + 4 * N * H * C + 4 * E * H, 4 * E * H * C)
-    del gev
+    report("c3", "the same with the edge-value grad left in the reversed graph's edge order (contiguous stores; the GAT layer's path)",
+           timeit(lambda: _ops.spmm_dot(gt.ptr_t, gt.idx_t, g, N, ev, gt.perm, x, gev, dot_at_edge=True), iters),
+           spmm_bytes(N, E, H * C, H) + 8 * E + 4 * N * H * C + 4 * E * H, 4 * E * H * C)
+    inv = _ops.inverse_perm_transposed(gt)
+    report("c3", "edge_softmax_bwd row pass H=4, gradient in edge order",
+           timeit(lambda: _ops.edge_softmax_bwd(ptr, ev, mask, gev, N, 0.2), iters),
+           E * (4 * H * 3 + H) + 8 * N + 4 * N * H, 6 * E * H)
+    report("c3", "edge_softmax_bwd row pass H=4, gradient read through the inverse permutation (the GAT layer's path)",
+           timeit(lambda: _ops.edge_softmax_bwd(ptr, ev, mask, gev, N, 0.2, grad_pos=inv), iters),
+           E * (4 * H * 3 + H + 8) + 8 * N + 4 * N * H, 6 * E * H)
+    del gev, inv
     dst = _ops.csr_row_ids(ptr, N, E)
     out = torch.empty(E, H, device="cuda")
     report("c3", "sddmm_coo H=4 C=64", timeit(lambda: _ops.sddmm_coo(idx, dst, x, g, out, E), iters),
@@ -355,11 +365,11 @@ def c4(iters):
     def fused(precision):
         out.zero_()
         _typed.typed_gemm(x, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, precision=precision)
-    report("c4", "rgcn fused gather-GEMM-scatter fp32 MFMA", timeit(lambda: fused("fp32"), iters), fused_bytes,
+    report("c4", "rgcn fused gather-GEMM-scatter (fp32 atomics; not the layer's path) fp32 MFMA", timeit(lambda: fused("fp32"), iters), fused_bytes,
            flops, MFMA_F32)
-    report("c4", "rgcn fused gather-GEMM-scatter fp32 as 6 bf16 products", timeit(lambda: fused("split6"), iters),
+    report("c4", "rgcn fused gather-GEMM-scatter (fp32 atomics; not the layer's path) fp32 as 6 bf16 products", timeit(lambda: fused("split6"), iters),
            fused_bytes, flops)
-    report("c4", "rgcn fused gather-GEMM-scatter fp32 as 3 scaled fp16 products (default)",
+    report("c4", "rgcn fused gather-GEMM-scatter (fp32 atomics; not the layer's path) fp32 as 3 scaled fp16 products (default precision)",
            timeit(lambda: fused("split_f16"), iters), fused_bytes, flops)
     # the same result without atomics: one GEMM row per edge written in CSR order, then
     # the sum over each destination's consecutive rows (the sparse strategy of the layer)
@@ -377,7 +387,7 @@ def c4(iters):
     def fused16():
         out.zero_()
         _typed.typed_gemm(x16, w, seg, E, src_idx=src, dst_idx=dst, out=out, atomic=True, bf16=True)
-    report("c4", "rgcn fused gather-GEMM-scatter bf16 MFMA", timeit(fused16, iters),
+    report("c4", "rgcn fused gather-GEMM-scatter (fp32 atomics; not the layer's path) bf16 MFMA", timeit(fused16, iters),
            E * (2 * K + 16 + 4 * K) + 2 * R * K * K, flops, MFMA_BF16)
     xe = torch.empty(E, K, device="cuda")
     xe.normal_()
@@ -385,7 +395,7 @@ def c4(iters):
     report("c4", "typed GEMM edge->edge fp32 (E x 128 x 128, sorted rows)",
            timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="fp32"), iters),
            E * 8 * K + 4 * R * K * K, flops, MFMA_F32)
-    report("c4", "typed GEMM edge->edge fp32 as 3 scaled fp16 products (default)",
+    report("c4", "typed GEMM edge->edge fp32 as 3 scaled fp16 products (default precision)",
            timeit(lambda: _typed.typed_gemm(xe, w, seg, E, out=oe, precision="split_f16"), iters),
            E * 8 * K + 4 * R * K * K, flops)
     for prec, nprod in (("split6", 6), ("split3", 3)):
@@ -404,7 +414,7 @@ def c4(iters):
     seg2 = (seg.double() * (E2 / E)).long()
     seg2[-1] = E2
     o2 = torch.empty(E2, K2, device="cuda")
-    for prec, what in (("fp32", "fp32 MFMA"), ("split_f16", "3 scaled fp16 products (default)")):
+    for prec, what in (("fp32", "fp32 MFMA"), ("split_f16", "3 scaled fp16 products (default precision; the tiled kernel for wide operands)")):
         report("c4", "typed GEMM 5M rows x 256 x 256, %s" % what,
                timeit(lambda: _typed.typed_gemm(x2, w2, seg2, E2, out=o2, precision=prec), iters),
                E2 * 8 * K2 + 4 * R * K2 * K2, 2.0 * E2 * K2 * K2, MFMA_F32 if prec == "fp32" else None)
