@@ -58,6 +58,14 @@ constexpr int kWBlockHalfs = 2 * kWN * kWK;   // fp16 elements of one (relation,
 constexpr int kWMaxTiles = 8;              // row tiles per block
 constexpr int kWBlockBytes = kWBlockHalfs * 2;                       // 32 KB
 constexpr int kWAsBytes = 2 * 2 * kWM * kWP * 2;                     // both stages, both parts of the A tile
+// Requests per producer wave and chunk: 16-byte A loads per lane, 1 KB memory -> LDS requests of the W
+// block.  The producers wait with hand-written counts -- vmcnt(12) before a set of A registers is
+// used, vmcnt(16) before the barrier that publishes a W block -- which hold for exactly these numbers.
+constexpr int kWReqA = 4;
+constexpr int kWReqW = 8;
+static_assert(kWReqA + kWReqW == 12 && 2 * kWReqA + kWReqW == 16, "the s_waitcnt vmcnt(12) / vmcnt(16) of the producers");
+static_assert(kWReqW * 1024 * 4 == kWBlockBytes, "four producer waves fetch one W block");
+static_assert(kWReqA * 16 * 64 * 4 == kWM * kWK * 4, "four producer waves fetch one A chunk");
 constexpr int kWCP = 136;                  // floats per row of a consumer wave's store staging area
 
 struct WideArgs {
@@ -412,7 +420,7 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
     // (inline assembly, like the W requests below and for the same reason: the waits are placed
     // by hand, see a_wait)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kWReqA; ++i) {
       const float* p = A + rowoff[i] + koff;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(ar[i]) : "v"(p) : "memory");
     }
@@ -436,7 +444,7 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
     const unsigned char* src = reinterpret_cast<const unsigned char*>(Wb) + (int64_t)dm_c * kWBlockBytes + pw * 8192;
     const unsigned dst = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)(Ws + dm_a * kWBlockBytes + pw * 8192);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kWReqW; ++j) {
       const unsigned char* sj = src + j * 1024;
       const unsigned dj = dst + j * 1024;
       asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane16), "s"(sj), "s"(dj) : "memory", "m0");
