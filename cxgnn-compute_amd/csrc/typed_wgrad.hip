@@ -144,12 +144,17 @@ void typed_wgrad_split_kernel(WgradArgs g) {
   };
   int (*s_exp)[2][4] = reinterpret_cast<int (*)[2][4]>(s_tiles + (size_t)4 * NS * 128 * kMP);   // [operand][buffer][column group]
   int64_t* const s_map = reinterpret_cast<int64_t*>(reinterpret_cast<unsigned char*>(s_exp) + kExpBytes);   // [operand][row of the chunk]
-  // The column tiles of one row chunk get consecutive slots of one XCD (blocks go to
-  // the 8 XCDs round-robin by index), so the chunk's A rows are fetched into one L2.
-  const int n_ct = (g.N + 127) / 128;
+  // A block owns one 128 x 128 tile of gw: columns n0 .. n0+127 of G against columns k0 .. k0+127 of
+  // A.  All tiles of one row chunk get consecutive slots of one XCD (blocks go to the 8 XCDs
+  // round-robin by index), so the chunk's A and G rows are fetched from memory into one L2 once and
+  // the other tiles of the chunk find them there (K = N = 512: sixteen tiles per chunk; one launch
+  // per 128 columns of A read G four times from memory and A once per column tile).
+  const int n_ct = (g.N + 127) / 128, n_kt = (g.K + 127) / 128;
+  const int n_tile = n_ct * n_kt;
   const int64_t slot = blockIdx.x / kXcds;
-  const int64_t chunk = (slot / n_ct) * kXcds + (blockIdx.x % kXcds);
-  const int n0 = (int)(slot % n_ct) * 128;
+  const int64_t chunk = (slot / n_tile) * kXcds + (blockIdx.x % kXcds);
+  const int n0 = (int)((slot % n_tile) % n_ct) * 128;
+  const int k0 = (int)((slot % n_tile) / n_ct) * 128;
   int rel = 0;
   int64_t row0 = 0, row_end = 0;
   const bool have = locate_chunk(g.seg, g.R, g.rows_per_chunk, chunk, rel, row0, row_end);
@@ -168,10 +173,10 @@ void typed_wgrad_split_kernel(WgradArgs g) {
     // the bits the other way round four lanes met in every bank), while a global load
     // still covers 8 rows with 128 contiguous bytes each.
     const int c4 = pwave * 8 + (lane >> 3), mg = lane & 7;
-    const bool col_ok = operand ? (n0 + 4 * c4 < N) : (4 * c4 < K);      // N % 4 == 0 is required
-    const float* const base = operand ? g.g + (col_ok ? n0 + 4 * c4 : 0) : g.a + (col_ok ? 4 * c4 : 0);
+    const bool col_ok = operand ? (n0 + 4 * c4 < N) : (k0 + 4 * c4 < K);      // K % 4 == 0 and N % 4 == 0 are required
+    const float* const base = operand ? g.g + (col_ok ? n0 + 4 * c4 : 0) : g.a + (col_ok ? k0 + 4 * c4 : 0);
     const int64_t ld = operand ? g.ldg : g.lda;
-    const uint16_t* const base16 = reinterpret_cast<const uint16_t*>(g.a) + (col_ok ? 4 * c4 : 0);
+    const uint16_t* const base16 = reinterpret_cast<const uint16_t*>(g.a) + (col_ok ? k0 + 4 * c4 : 0);
     // row of this operand behind row r of tile t (-1: no such row)
     auto row_index = [&](int t, int r) -> int64_t {
       if constexpr (MAPPED) {
@@ -313,7 +318,7 @@ void typed_wgrad_split_kernel(WgradArgs g) {
   }
 
   // ---- consumers --------------------------------------------------------------------
-  if (wave * 32 >= K) {
+  if (k0 + wave * 32 >= K) {
     // this wave's 32 rows of gw lie past K: nothing to multiply or store, only the barriers
     if (n_tiles > 0) {
       __syncthreads();                                 // #1
@@ -394,7 +399,7 @@ void typed_wgrad_split_kernel(WgradArgs g) {
     if (col >= N) continue;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int k = wave * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+      const int k = k0 + wave * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
       if (k < K) part[(size_t)k * N + col] = acc[nb][i];
     }
   }
@@ -451,9 +456,9 @@ __global__ __launch_bounds__(64 * kReduceSlices) void wgrad_reduce_kernel(
 // with a K x 128 partial that the reduction reads again, so few long chunks beat many short
 // ones: the number of rounds of one block per CU that the longest chunks would need, then
 // the chunk length that fills those rounds evenly.
-int64_t chunk_rows(int64_t M, int N, bool mapped) {
+int64_t chunk_rows(int64_t M, int K, int N, bool mapped) {
   const int64_t g_max = (mapped ? kMappedRows : 256 * kMT) / kMT;
-  const int64_t tiles = ceil_div(M, (int64_t)kMT) * ceil_div(N, 128);
+  const int64_t tiles = ceil_div(M, (int64_t)kMT) * ceil_div(N, 128) * ceil_div(K, 128);
   int64_t rounds = ceil_div(tiles, 256 * g_max);
   if (rounds < 1) rounds = 1;
   int64_t g = ceil_div(tiles, 256 * rounds);
@@ -470,7 +475,7 @@ extern "C" {
 size_t cxg_typed_gemm_wgrad_workspace_bytes(int64_t M, int K, int N, int R) {
   if (M < 0 || K < 1 || N < 1 || R < 1) return 0;
   // the chunks of a launch with row maps are the shorter ones: their count bounds both cases
-  const int64_t chunks = cxg::ceil_div(cxg::ceil_div(M, cxg::chunk_rows(M, N, true)) + R, cxg::kXcds) * cxg::kXcds;
+  const int64_t chunks = cxg::ceil_div(cxg::ceil_div(M, cxg::chunk_rows(M, K, N, true)) + R, cxg::kXcds) * cxg::kXcds;
   return (size_t)chunks * (size_t)K * (size_t)N * sizeof(float) + 256;
 }
 
@@ -483,9 +488,9 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
               CXG_ERR_ARG, "unknown flag");
   CXG_REQUIRE(gw && seg_ptr, CXG_ERR_ARG, "null gw/seg_ptr");
   CXG_REQUIRE(M == 0 || (a && g), CXG_ERR_ARG, "null a/g");
-  CXG_REQUIRE(K <= 128 && (K & 3) == 0 && (N & 3) == 0 && (lda & 3) == 0 && (ldg & 3) == 0 &&
+  CXG_REQUIRE(K <= 4096 && (K & 3) == 0 && (N & 3) == 0 && (lda & 3) == 0 && (ldg & 3) == 0 &&
                   ((uintptr_t)a & 15) == 0 && ((uintptr_t)g & 15) == 0,
-              CXG_ERR_UNSUPPORTED, "wgrad needs K <= 128, K, N, lda, ldg multiples of 4 and 16-byte aligned operands");
+              CXG_ERR_UNSUPPORTED, "wgrad needs K <= 4096, K, N, lda, ldg multiples of 4 and 16-byte aligned operands");
   CXG_REQUIRE(lda >= K && ldg >= N, CXG_ERR_ARG, "row stride smaller than row");
   const size_t need = cxg_typed_gemm_wgrad_workspace_bytes(M, K, N, R);
   CXG_REQUIRE(workspace && workspace_bytes >= need, CXG_ERR_WORKSPACE,
@@ -493,9 +498,9 @@ int cxg_typed_gemm_wgrad_f32(const float* a, int64_t lda, const float* g, int64_
   CXG_REQUIRE(((uintptr_t)workspace & 255) == 0, CXG_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool mapped = src_idx || dst_idx;
-  const int64_t rows = cxg::chunk_rows(M, N, mapped);
+  const int64_t rows = cxg::chunk_rows(M, K, N, mapped);
   const int64_t chunks = cxg::ceil_div(cxg::ceil_div(M, rows) + R, cxg::kXcds) * cxg::kXcds;
-  const int n_ct = (int)cxg::ceil_div(N, 128);
+  const int n_ct = (int)(cxg::ceil_div(N, 128) * cxg::ceil_div(K, 128));     // 128 x 128 tiles of gw
   CXG_REQUIRE(chunks * n_ct < ((int64_t)1 << 31), CXG_ERR_UNSUPPORTED, "too many chunks for one launch");
   cxg::WgradArgs wa{a, lda, g, ldg, src_idx, dst_idx, seg_ptr, reinterpret_cast<float*>(workspace),
                     M, K, N, R, rows, (int)((flags & CXG_WGRAD_A_BF16) != 0)};

@@ -351,9 +351,9 @@ def _edge_positions(n, device):
 
 def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=None, precision=None):
     """gw[r] = sum over the rows i of segment r of a[src(i)]^T (x) g[dst(i)] -> [num_rel, K, N]
-    (see cxg_typed_gemm_wgrad_f32).  One launch takes K <= 128; a wider K runs as one launch per
-    128 columns of ``a`` (a single relation writes its rows of gw in place, several relations go
-    through a [num_rel, 128, N] buffer per slice).  An N that is not a multiple of 4 (a class
+    (see cxg_typed_gemm_wgrad_f32).  One launch takes K <= 4096 (a block per 128 x 128 tile of gw and
+    row chunk; the tiles of a chunk share its rows through one L2); beyond that, one launch per
+    4096 columns of ``a``.  An N that is not a multiple of 4 (a class
     count, say) runs on a copy of g padded with zero columns.  Returns None when K is not a
     multiple of 4, which the kernel does not take."""
     lib = _lib.load()
@@ -373,9 +373,10 @@ def typed_gemm_wgrad(a, g, seg_ptr, m_rows, num_rel, *, src_idx=None, dst_idx=No
     flags |= WGRAD_A_BF16 if a_bf16 else 0
     esz = 2 if a_bf16 else 4
     gw = torch.empty((num_rel, K, N), dtype=torch.float32, device=a.device)
+    k_max = 4096                                            # what one launch takes
     with torch.cuda.device(a.device):
-        for k0 in range(0, K, 128):
-            kb = min(128, K - k0)
+        for k0 in range(0, K, k_max):
+            kb = min(k_max, K - k0)
             direct = num_rel == 1 or kb == K
             part = gw if direct else torch.empty((num_rel, kb, N), dtype=torch.float32, device=a.device)
             ws = _workspace(lib.cxg_typed_gemm_wgrad_workspace_bytes(m_rows, kb, N, num_rel), a.device)

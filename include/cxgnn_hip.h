@@ -414,7 +414,9 @@ int cxg_typed_gemm_wide_f32(const float* a, int64_t lda, const float* w, float* 
  * row chunk (the scale follows the largest magnitude met so far in the chunk; an
  * element keeps 22 significant bits down to 2^-17 of that magnitude); partial sums
  * over row chunks are added in
- * chunk order by a second kernel (deterministic).  Needs K <= 128, K, N, lda, ldg
+ * chunk order by a second kernel (deterministic).  A block computes one 128 x 128
+ * tile of gw over one row chunk, and the tiles of a chunk run side by side on one die
+ * so that its rows of A and G come from memory once.  Needs K <= 4096, K, N, lda, ldg
  * multiples of 4 and 16-byte aligned operands (otherwise CXG_ERR_UNSUPPORTED).
  * Replaces the per-relation torch.mm of TypedLinearE2EOP.backward and
  * TypedLinearS2DMMAggrOP.backward (cxgnncomp/typed_linear.py:114-137,205-221).
