@@ -40,6 +40,9 @@ namespace {
 #ifndef CXG_SPMM_U_V4
 #define CXG_SPMM_U_V4 8
 #endif
+#ifndef CXG_SPMM_U_DOT
+#define CXG_SPMM_U_DOT 4
+#endif
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWavesPerBlock * CXG_WAVE;
@@ -368,6 +371,12 @@ __global__ __launch_bounds__(kBlock) void spmm_span_kernel(SpmmArgs<IdxT> a) {
       if (PERM) my_vrow = stream_load(a.perm + pos);
       if (WMODE == 1 && !PERM) my_w = stream_load(a.val + pos);
     }
+    // (The loads of a group sit under a condition each, and the compiler, whose count of requests in
+    // flight is a guess at every join, waits for each gather before it issues the next.  Written without
+    // the conditions the gathers of a group do stay in flight together -- and every kernel built on this
+    // loop is slower for it, at any group size: multi-head forward 7.77 -> 8.03 ms, single head F = 256
+    // on the 2.3 M-entry graph 0.325 -> 0.350 ms.  With eight waves per SIMD one gather per wave already
+    // fills the fabric's queues; more only lengthens them.)
     for (int b = 0; b < cn; b += U) {
       vec_t v[U];
       float w[U];
@@ -912,7 +921,7 @@ int launch_spmm(const SpmmArgs<IdxT>& a_in, int64_t n_spans_cap, hipStream_t str
   // waves per SIMD resident (12.7 -> 11.5 ms on the GAT graph; 16 in flight: 14.5 ms).
   // (More gathers in flight for the narrow kernels on launches too small to fill the chip were
   // measured too: 15 k - 936 k edges of 47 floats, no gain or a loss.)
-  constexpr int U = DOTG > 0 ? 4 : ((V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U);
+  constexpr int U = DOTG > 0 ? CXG_SPMM_U_DOT : ((V == 4) ? CXG_SPMM_U_V4 : CXG_SPMM_U);
   const int tile = CXG_WAVE * V;
   const int64_t n_ct = ceil_div(a_in.F, tile);
   SpmmArgs<IdxT> a = a_in;
