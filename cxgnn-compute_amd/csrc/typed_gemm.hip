@@ -23,6 +23,7 @@
 #include <type_traits>
 
 #include "cxg_common.hpp"
+#include "split_f16.hpp"
 
 namespace cxg {
 namespace {
@@ -691,10 +692,7 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
     if constexpr (F16) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const unsigned b0 = __float_as_uint(areg[i].x) & 0x7fffffffu, b1 = __float_as_uint(areg[i].y) & 0x7fffffffu;
-        const unsigned b2 = __float_as_uint(areg[i].z) & 0x7fffffffu, b3 = __float_as_uint(areg[i].w) & 0x7fffffffu;
-        const unsigned m01 = b0 > b1 ? b0 : b1, m23 = b2 > b3 ? b2 : b3;
-        const unsigned m = m01 > m23 ? m01 : m23;
+        const unsigned m = abs_max4_bits(areg[i].x, areg[i].y, areg[i].z, areg[i].w);
         row_max[i] = k_ok ? m : 0u;
       }
 #pragma unroll
@@ -711,16 +709,13 @@ void typed_gemm_split_kernel(GemmArgs g, int G) {
         const float sc = (KS == 16 || k_ok) ? scale : 0.f;
         const float v[4] = {(KS < 16 || k_ok) ? areg[i].x : 0.f, (KS < 16 || k_ok) ? areg[i].y : 0.f,
                             (KS < 16 || k_ok) ? areg[i].z : 0.f, (KS < 16 || k_ok) ? areg[i].w : 0.f};
-        v4h part[2];
+        typedef unsigned v2u __attribute__((ext_vector_type(2)));
+        unsigned h01, l01, h23, l23;
+        split_f16_pair(v[0], v[1], sc, h01, l01);
+        split_f16_pair(v[2], v[3], sc, h23, l23);
+        const v2u part[2] = {{h01, h23}, {l01, l23}};      // [high / low parts][two packed pairs]
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float xs = v[j] * sc;
-          const _Float16 h0 = (_Float16)xs;
-          part[0][j] = h0;
-          part[1][j] = (_Float16)(xs - (float)h0);
-        }
-#pragma unroll
-        for (int q = 0; q < 2; ++q) *reinterpret_cast<v4h*>(&dst[q][row][4 * c4]) = part[q];
+        for (int q = 0; q < 2; ++q) *reinterpret_cast<v2u*>(&dst[q][row][4 * c4]) = part[q];
         if (c4 == 0) s_inv[t & 1][row] = inv;
       } else {
         const float v[4] = {k_ok ? areg[i].x : 0.f, k_ok ? areg[i].y : 0.f, k_ok ? areg[i].z : 0.f,

@@ -38,6 +38,7 @@
 // (cxgnncomp/codegen/triton_typed_matmul.py:752-860; test/ae/E3_ablation/test-batch.py:27-52
 // runs K = N = 512).
 #include "cxg_common.hpp"
+#include "split_f16.hpp"
 
 namespace cxg {
 namespace {
@@ -481,12 +482,7 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
     int lowered = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      // largest magnitude of the four values: float maxima with the absolute-value operand modifier (two
-      // instructions; four masks and three integer maxima before).  A NaN loses against a number and
-      // wins against nothing else, so a row of NaNs reads as exponent 255, like an infinity.
-      const float mf = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[i][0]), __builtin_fabsf(v[i][1])),
-                                       __builtin_fmaxf(__builtin_fabsf(v[i][2]), __builtin_fabsf(v[i][3])));
-      unsigned m = __float_as_uint(mf) & 0x7fffffffu;
+      unsigned m = abs_max4_bits(v[i][0], v[i][1], v[i][2], v[i][3]);
       m = wide_dpp_max<0xB1>(m);                         // lane ^ 1
       m = wide_dpp_max<0x4E>(m);                         // lane ^ 2
       m = wide_dpp_max<0x141>(m);                        // mirror of the 8 lanes that hold the row chunk
@@ -499,22 +495,9 @@ void typed_gemm_wide_kernel(WideArgs g, int G) {
       lowered |= lower;
       sb[i] = nsb;
       const float scale = __uint_as_float((unsigned)nsb << 23);
-      // Two values per register pair, four instructions: v_fma_mixlo / mixhi_f16 form x * scale (- high
-      // part) in fp32 and round once into one half of the destination, and they read a 16-bit operand
-      // out of either half of a packed register -- so the high parts need no separate multiply and
-      // conversion and the low parts no unpacking.  (From `(_Float16)(x * scale)` and
-      // `(_Float16)(x * scale - (float)h)` the compiler made seven instructions per pair: it formed
-      // every high part twice.)
       unsigned hi2[2], lo2[2];
 #pragma unroll
-      for (int jp = 0; jp < 2; ++jp) {
-        const float x0 = v[i][2 * jp], x1 = v[i][2 * jp + 1];
-        asm("v_fma_mixlo_f16 %0, %1, %2, 0\n\tv_fma_mixhi_f16 %0, %3, %2, 0"
-            : "=&v"(hi2[jp]) : "v"(x0), "v"(scale), "v"(x1));
-        asm("v_fma_mixlo_f16 %0, %1, %2, -%4 op_sel_hi:[0,0,1]\n\t"
-            "v_fma_mixhi_f16 %0, %3, %2, -%4 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
-            : "=&v"(lo2[jp]) : "v"(x0), "v"(scale), "v"(x1), "v"(hi2[jp]));
-      }
+      for (int jp = 0; jp < 2; ++jp) split_f16_pair(v[i][2 * jp], v[i][2 * jp + 1], scale, hi2[jp], lo2[jp]);
       typedef unsigned v2u __attribute__((ext_vector_type(2)));
       const v2u part0 = {hi2[0], hi2[1]}, part1 = {lo2[0], lo2[1]};
       const int row = rsub + 32 * i;

@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "cxg_common.hpp"
+#include "split_f16.hpp"
 
 namespace cxg {
 namespace {
@@ -248,28 +249,23 @@ void typed_wgrad_split_kernel(WgradArgs g) {
       if constexpr (F16) {
         unsigned m = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const unsigned b = __float_as_uint(v[i][c]) & 0x7fffffffu;
-            m = b > m ? b : m;
-          }
+        for (int i = 0; i < 4; ++i) {
+          const unsigned b = abs_max4_bits(v[i][0], v[i][1], v[i][2], v[i][3]);
+          m = b > m ? b : m;
+        }
         int eb = (int)(wave_max_u32(m) >> 23);
         eb = eb > 254 ? 254 : eb;                      // an infinity or NaN still comes out non-finite
         e_run = eb > e_run ? eb : e_run;
         const float scale = e_run >= 15 ? __uint_as_float((unsigned)(268 - e_run) << 23) : 0.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-          v4h out[2];
+          typedef unsigned v2u __attribute__((ext_vector_type(2)));
+          unsigned h01, l01, h23, l23;
+          split_f16_pair(v[0][c], v[1][c], scale, h01, l01);
+          split_f16_pair(v[2][c], v[3][c], scale, h23, l23);
+          const v2u out[2] = {{h01, h23}, {l01, l23}};     // [high / low parts][rows 0-1, rows 2-3 of the group]
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float xs = v[i][c] * scale;
-            const _Float16 h0 = (_Float16)xs;
-            out[0][i] = h0;
-            out[1][i] = (_Float16)(xs - (float)h0);
-          }
-#pragma unroll
-          for (int q = 0; q < 2; ++q) *reinterpret_cast<v4h*>(&dst[q][4 * c4 + c][mg * 4]) = out[q];
+          for (int q = 0; q < 2; ++q) *reinterpret_cast<v2u*>(&dst[q][4 * c4 + c][mg * 4]) = out[q];
         }
         if (lane == 0) s_exp[operand][t & 1][pwave] = e_run;
         return;
