@@ -170,6 +170,62 @@ def test_gat_configuration_full_size(big):
     assert abs(float(att_src.grad.double().sum()) - float(att_dst.grad.double().sum())) < 1e-2
 
 
+def test_gat_layer_full_size(big):
+    """MyGATConv 128 -> 4 x 64 on the 61.9M-edge graph: the layer's one autograd node (fused pass over
+    the reversed graph with the edge-value gradient left in that pass's edge order, softmax backward
+    reading it through the inverse permutation, bias in the aggregation's row stores) against the
+    composition of the separately verified operators -- linear, AttentionLogitsOP, edge_attention,
+    SpMMValOP, whose full-size results the test above holds against the oracle -- with the same
+    parameters and the same output gradient: output, input gradient and every parameter gradient.
+    Both sides compute the same sums in fp32, in different orders in places: 1e-4 of each tensor's
+    scale, 1e-5 absolute at that scale."""
+    import cxgnncomp
+    import cxgnncomp_backend as B
+    from cxgnncomp.graph_conv import AttentionLogitsOP, linear
+    from cxgnncomp.graph_kernel import SpMMValOP
+    cxgnncomp.set_timers()
+    ptr, idx = big
+    E = idx.shape[0]
+    H, C = 4, 64
+    torch.manual_seed(4)
+    layer = cxgnncomp.MyGATConv(128, C, heads=H, concat=True).cuda()
+    with torch.no_grad():
+        layer.bias.normal_()
+    x = (torch.randn(N_NODES, 128, device="cuda") / 4).requires_grad_(True)
+    gout = torch.randn(N_NODES, H * C, device="cuda") / 16
+    announce("MyGATConv layer fwd+bwd full size")
+    out = layer(x, ptr, idx, N_NODES, N_NODES, E)
+    out.backward(gout)
+    torch.cuda.synchronize()
+    got = {"out": out.detach(), "x": x.grad.clone()}
+    got.update({k: v.grad.clone() for k, v in layer.named_parameters()})
+    x.grad = None
+    for v in layer.parameters():
+        v.grad = None
+    del out
+    announce("the same layer as a composition of its operators, full size")
+    xs = linear(x, layer.lin_src).view(-1, H, C)
+    a_src, a_dst = AttentionLogitsOP.apply(xs, layer.att_src, layer.att_dst, N_NODES)
+    ev = B.edge_attention(ptr=ptr, idx=idx, att_dst=a_dst, att_src=a_src, num_edge=E, relu_l=layer.negative_slope)
+    ref = SpMMValOP.apply(xs, ptr, idx, ev, N_NODES).view(-1, H * C) + layer.bias
+    ref.backward(gout)
+    torch.cuda.synchronize()
+    want = {"out": ref.detach(), "x": x.grad}
+    want.update({k: v.grad for k, v in layer.named_parameters()})
+    for k in want:
+        assert got[k].shape == want[k].shape, k
+        sc = max(1e-30, float(want[k].abs().max()))
+        err = float((got[k].double() - want[k].double()).abs().max()) / sc
+        tol = 1e-4 + 1e-5
+        assert err <= tol, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
+    # and the node's own invariants: rows without edges hold the bias, nothing non-finite anywhere
+    deg = ptr[1:] - ptr[:-1]
+    empty = torch.nonzero(deg == 0).flatten()[:64]
+    if empty.numel():
+        assert torch.equal(got["out"][empty], layer.bias.detach().expand(empty.numel(), -1))
+    assert all(bool(torch.isfinite(t).all()) for t in got.values())
+
+
 def test_gspmm_full_size(big):
     """GSpMM_u MAX / GSpMM_u_e MIN x ADD on the full graph (thousands of rows above the
     512-edge piece size, hubs of ~17 k edges): exact against torch.segment_reduce over
