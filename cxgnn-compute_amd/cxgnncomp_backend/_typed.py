@@ -167,7 +167,8 @@ def dense_linear(x, w_kn, bias=None, addend=None):
     one segment, bias and addend added to the accumulator before the rows are stored.  Returns
     None for inputs the split kernels do not take (the caller then uses the library GEMM):
     other dtypes or layouts, few rows, K above 128 (256 when K >= 176, N >= 96 and at least
-    10^5 rows), K not a multiple of 4, a default precision other than the fp16 split form."""
+    10^5 rows; any K without bias and addend from 10^5 rows on: the tiled kernel), K not a multiple
+    of 4, a default precision other than the fp16 split form."""
     flags = _PRECISION_FLAGS.get(GEMM_PRECISION, 0)
     if flags != GEMM_SPLIT_F16X3 or not x.is_cuda or x.dim() != 2 or x.dtype != torch.float32 or w_kn.dtype != torch.float32:
         return None
@@ -176,7 +177,10 @@ def dense_linear(x, w_kn, bias=None, addend=None):
     # the 256-wide form stores from the accumulators (no staged 16-byte stores): it beats the
     # library from about 10^5 rows on (measured on 4 k - 2.4 M rows, with and without addend)
     wide = 176 <= K <= 256 and N >= 96 and M >= DENSE_WIDE_MIN_ROWS
-    if M < DENSE_MIN_ROWS or K % 4 or not (K <= 128 or wide) or w_kn.shape[0] != K:
+    # the tiled kernel has no epilogue; without one it also takes K above 256 (2.33 M x 512 x 512: 4.0 ms
+    # against 8.6 ms in the library)
+    tiled = (bias is None and addend is None and K > 256 and K % 4 == 0 and M >= DENSE_WIDE_MIN_ROWS)
+    if M < DENSE_MIN_ROWS or K % 4 or not (K <= 128 or wide or tiled) or w_kn.shape[0] != K:
         return None
     if not x.is_contiguous() or x.data_ptr() % 16:
         return None
@@ -185,8 +189,12 @@ def dense_linear(x, w_kn, bias=None, addend=None):
     if addend is not None and (addend.dtype != torch.float32 or tuple(addend.shape) != (M, N)
                                or not addend.is_contiguous()):
         return None
-    lib = _lib.load()
     w_kn = w_kn.contiguous()
+    if bias is None and addend is None and _takes_wide_form(K, N, flags, False):
+        # no epilogue: the tiled kernel for wide operands where it is the faster one (K >= 160 and more
+        # than 128 columns; 169,865 x 256 x 256: 0.135 against 0.158 ms)
+        return typed_gemm(x, w_kn.unsqueeze(0), _one_segment(M, x.device), M, precision="split_f16")
+    lib = _lib.load()
     out = torch.empty((M, N), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         st = lib.cxg_typed_gemm_epilogue_f32(x.data_ptr(), K, w_kn.data_ptr(), _lib.ptr(bias), _lib.ptr(addend), N,

@@ -180,3 +180,28 @@ def test_wide_entry_point_rejects_what_it_does_not_take():
     assert lib.cxg_typed_gemm_wide_f32(*args, 512, 64, 1, 4, ws.data_ptr(), need, st) == -1   # bf16 split flag
     assert lib.cxg_typed_gemm_wide_f32(*args, 512, 64, 1, 16, ws.data_ptr(), need, st) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("K,N", [(256, 256), (512, 384), (300, 72)])
+def test_dense_products_without_an_epilogue_take_the_tiled_kernel(K, N):
+    """dense_linear(x, W) without bias and addend from 10^5 rows on: 176 <= K <= 256 with more than 128
+    columns and any K above 256 run on the tiled kernel (one relation); against float64 on sampled
+    rows, and linear in x on every row."""
+    from cxgnncomp_backend import _typed
+    M = 120000
+    gen = torch.Generator().manual_seed(K + N)
+    x = (torch.randn(M, K, generator=gen) / K ** 0.5).cuda()
+    x2 = (torch.randn(M, K, generator=gen) / K ** 0.5).cuda()
+    w = torch.randn(K, N, generator=gen).cuda()
+    announce("dense_linear on the tiled kernel M=%d K=%d N=%d" % (M, K, N))
+    got = _typed.dense_linear(x, w)
+    if K <= 256 and N <= 128:
+        assert got is None or got.shape == (M, N)          # shapes the rule leaves to other kernels or the library
+        return
+    assert got is not None and got.shape == (M, N)
+    rows = torch.randint(0, M, (3000,), generator=gen).cuda()
+    want = x[rows].double() @ w.double()
+    assert_close(_np(got[rows]), _np(want), RTOL, ATOL, "dense product rows")
+    both = _typed.dense_linear(x + x2, w)
+    sep = got + _typed.dense_linear(x2, w)
+    assert float((both - sep).abs().max()) <= 1e-4 * max(1.0, float(sep.abs().max()))
