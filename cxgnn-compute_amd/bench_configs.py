@@ -298,7 +298,16 @@ def c3(iters):
     report("c3", "attention_logits bwd H=4 C=64 (grad x, grad att_src, grad att_dst)",
            timeit(lambda: _ops.attention_logits_bwd(x, a_s, a_d, gs, gs), iters), 8 * N * H * C + 8 * N * H,
            8 * N * H * C)
-    del x, g, gs
+    # the same logits read off the layer's 128-column input (the layer's path when the input is
+    # narrower than the transformed features): x @ m.T with m = att @ W per head
+    xin, m = x.view(N, H * C)[:, :128].contiguous(), torch.randn(2 * H, 128, device="cuda")
+    gxin = torch.zeros(N, 128, device="cuda")
+    report("c3", "attention_logits from the 128-column input, fwd H=4",
+           timeit(lambda: _ops.attention_logits_proj(xin, m, N, H), iters), 4 * N * 128 + 8 * N * H, 4 * N * 128 * H)
+    report("c3", "attention_logits from the 128-column input, bwd H=4 (adds into grad x_in; grad m)",
+           timeit(lambda: _ops.attention_logits_proj_bwd(xin, m, gs, gs, H, add_to=gxin), iters),
+           12 * N * 128 + 8 * N * H, 8 * N * 128 * H)
+    del x, g, gs, xin, gxin
     # the configuration's layer: GAT 128 -> 4 heads x 64, forward + backward through the
     # softmax and the edge-weighted aggregation including the edge-value gradient
     import cxgnncomp

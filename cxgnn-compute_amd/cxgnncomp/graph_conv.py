@@ -481,13 +481,29 @@ class GatLayerOP(torch.autograd.Function):
     nodes do, but the two gradients of the transformed features -- from the aggregation
     and from the logits -- meet in one buffer (the logits kernel adds into what the
     transposed aggregation wrote) instead of two tensors and a full-size add, and the
-    intermediate views cost no copies."""
+    intermediate views cost no copies.  Where the input is narrower than the transformed
+    features (and the kernels take the shape) the logits are read off the input instead,
+    ``x @ m.T`` with ``m = att @ W`` per head -- the contraction order of the single-head
+    path's einsum (upstream cxgnncomp/graph_conv.py:500-511); their backward pass then adds a
+    rank-2H term to the input gradient and returns grad m, from which the shares of the weight
+    and attention-vector gradients follow by the chain rule on [2H, in] tensors."""
+
+    @staticmethod
+    def _logit_rows(w, att_src, att_dst, H, C):
+        w3 = w.view(H, C, -1)
+        return torch.cat([torch.bmm(att_src.reshape(H, 1, C), w3), torch.bmm(att_dst.reshape(H, 1, C), w3)]).squeeze(1)
 
     @staticmethod
     def forward(ctx, x, w, att_src, att_dst, bias, ptr, idx, num_dst, num_src, num_edge, slope, heads, concat):
         H, C = heads, w.shape[0] // heads
         xs = _mm(x[:num_src], w.t()).view(-1, H, C)
-        a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
+        from_input = (x.shape[1] < H * C and _ops.logits_proj_supported(x.shape[1], H) and x.stride(1) == 1
+                      and x.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0)
+        if from_input:
+            a_src, a_dst = _ops.attention_logits_proj(x[:num_src], GatLayerOP._logit_rows(w, att_src, att_dst, H, C),
+                                                      num_dst, H)
+        else:
+            a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
         ev, mask = _ops.edge_softmax_fwd(ptr, idx, a_dst, a_src, num_edge, slope)
         if concat:
             # the bias goes into the aggregation's row stores
@@ -497,13 +513,13 @@ class GatLayerOP(torch.autograd.Function):
             if bias is not None:
                 out.add_(bias)
         ctx.save_for_backward(x, w, att_src, att_dst, xs, ev, mask, ptr, idx)
-        ctx.dims = (num_dst, num_src, H, C, concat, float(slope), bias is not None)
+        ctx.dims = (num_dst, num_src, H, C, concat, float(slope), bias is not None, from_input)
         return out
 
     @staticmethod
     def backward(ctx, g):
         x, w, att_src, att_dst, xs, ev, mask, ptr, idx = ctx.saved_tensors
-        num_dst, num_src, H, C, concat, slope, has_bias = ctx.dims
+        num_dst, num_src, H, C, concat, slope, has_bias, from_input = ctx.dims
         g = g.contiguous()
         g_bias = _ops.column_sum(g) if has_bias and ctx.needs_input_grad[4] else None
         if concat:
@@ -526,15 +542,27 @@ class GatLayerOP(torch.autograd.Function):
             g_ev = _ops.sddmm_csr(ptr, idx, xs, g3, num_dst, out=g_ev)
             g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope)
         g_asrc = _ops.narrow_gather_sum(tg.ptr_t, tg.perm, t_edge, xs.shape[0], rows32=_ops.rows32_transposed(tg))
-        _, g_att_src, g_att_dst = _ops.attention_logits_bwd(xs, att_src, att_dst, g_asrc, g_adst, add_to=g_xs)
+        if not from_input:
+            _, g_att_src, g_att_dst = _ops.attention_logits_bwd(xs, att_src, att_dst, g_asrc, g_adst, add_to=g_xs)
         g_xs2 = g_xs.view(-1, H * C)
         g_x = g_w = None
         if ctx.needs_input_grad[0]:
             g_x = _mm(g_xs2, w)
-            if g_x.shape[0] < x.shape[0]:
-                g_x = torch.cat([g_x, g_x.new_zeros(x.shape[0] - g_x.shape[0], g_x.shape[1])])
         if ctx.needs_input_grad[1]:
             g_w = _weight_grad(x[:num_src], g_xs2)
+        if from_input:
+            # the logits' share: rank 2H into g_x, and through m = att @ W into g_w and g_att
+            m = GatLayerOP._logit_rows(w, att_src, att_dst, H, C)
+            _, g_m = _ops.attention_logits_proj_bwd(x[:num_src], m, g_asrc, g_adst, H, add_to=g_x, need_x=False)
+            g_m = g_m.view(2, H, 1, -1)
+            w3t = w.view(H, C, -1).transpose(1, 2)
+            g_att_src, g_att_dst = torch.bmm(g_m[0], w3t), torch.bmm(g_m[1], w3t)
+            if g_w is not None:
+                g_w3 = g_w.view(H, C, -1)
+                g_w3.baddbmm_(att_src.reshape(H, C, 1), g_m[0])
+                g_w3.baddbmm_(att_dst.reshape(H, C, 1), g_m[1])
+        if g_x is not None and g_x.shape[0] < x.shape[0]:
+            g_x = torch.cat([g_x, g_x.new_zeros(x.shape[0] - g_x.shape[0], g_x.shape[1])])
         return (g_x, g_w, g_att_src.view_as(att_src), g_att_dst.view_as(att_dst), g_bias,
                 None, None, None, None, None, None, None, None)
 

@@ -87,6 +87,11 @@ SIGNATURES = {
     "cxg_attention_logits_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "cxg_attention_logits_bwd_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _I32, _P, _P, _P, _SZ,
                                             _P]),
+    "cxg_attention_logits_proj_supported": (_I32, [_I32, _I32]),
+    "cxg_attention_logits_proj_fwd_f32": (_I32, [_P, _I64, _P, _I64, _I64, _I32, _I32, _P, _P, _P]),
+    "cxg_attention_logits_proj_workspace_bytes": (_SZ, [_I32, _I32]),
+    "cxg_attention_logits_proj_bwd_f32": (_I32, [_P, _I64, _P, _P, _P, _I64, _I64, _I32, _I32, _P, _I64, _I32, _P,
+                                                _P, _SZ, _P]),
     "cxg_batchnorm_workspace_bytes": (_SZ, [_I64, _I32]),
     "cxg_column_sum_f32": (_I32, [_P, _I64, _I32, _I64, _P, _P, _SZ, _P]),
     "cxg_batchnorm_stats_f32": (_I32, [_P, _I64, _I32, _I64, _F32, _P, _P, _P, _P, _SZ, _P]),

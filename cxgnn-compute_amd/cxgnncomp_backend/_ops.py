@@ -313,6 +313,71 @@ def attention_logits_bwd(x, att_src, att_dst, g_src, g_dst, add_to=None):
     return grad_x, ga_src, ga_dst
 
 
+def logits_proj_supported(n_in, heads):
+    """Whether the kernels that take a GAT layer's logits from its input handle this shape."""
+    return bool(_lib.load().cxg_attention_logits_proj_supported(int(n_in), int(heads)))
+
+
+def _proj_rows(x, m, heads):
+    _req(m, "m", torch.float32, 2)
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32 or x.dim() != 2:
+        raise ValueError("x must be a 2-d float32 CUDA tensor")
+    if x.stride(1) != 1 and x.shape[1] != 1:
+        raise ValueError("the rows of x must be contiguous")
+    if m.shape != (2 * heads, x.shape[1]) or m.device != x.device:
+        raise ValueError("m %s does not fit x %s with %d heads" % (tuple(m.shape), tuple(x.shape), heads))
+    return x.shape[0], x.shape[1], (x.stride(0) if x.shape[0] > 1 else x.shape[1])
+
+
+def attention_logits_proj(x, m, n_dst, heads):
+    """(x @ m[:H].T, x[:n_dst] @ m[H:].T) for x [n_src, in] (rows may be strided) and
+    m [2H, in]: both per-node logits of a GAT layer taken from the layer's input, where m
+    holds att_src / att_dst carried through the layer's weight."""
+    lib = _lib.load()
+    n_src, n_in, ldx = _proj_rows(x, m, heads)
+    if not 0 <= n_dst <= n_src:
+        raise ValueError("n_dst=%d outside [0, %d]" % (n_dst, n_src))
+    out_src = torch.empty(n_src, heads, dtype=torch.float32, device=x.device)
+    out_dst = torch.empty(n_dst, heads, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_attention_logits_proj_fwd_f32(_lib.ptr(x), ldx, m.data_ptr(), n_src, n_dst, n_in, heads,
+                                                   _lib.ptr(out_src), _lib.ptr(out_dst),
+                                                   _lib.current_stream(x.device))
+    _lib.check(st)
+    return out_src, out_dst
+
+
+def attention_logits_proj_bwd(x, m, g_src, g_dst, heads, add_to=None, need_x=True):
+    """Gradients of ``attention_logits_proj``: (grad_x, grad_m), reproducible.  ``add_to``
+    ([n_src, in], contiguous) receives grad_x added in place and is returned as grad_x;
+    with ``need_x=False`` grad_x is None and only grad_m [2H, in] is computed."""
+    lib = _lib.load()
+    n_src, n_in, ldx = _proj_rows(x, m, heads)
+    n_dst = g_dst.shape[0]
+    _req(g_src, "g_src", torch.float32, 2)
+    _req(g_dst, "g_dst", torch.float32, 2)
+    if tuple(g_src.shape) != (n_src, heads) or g_dst.shape[1] != heads or n_dst > n_src:
+        raise ValueError("gradient shapes %s / %s do not fit x %s"
+                         % (tuple(g_src.shape), tuple(g_dst.shape), tuple(x.shape)))
+    grad_x = None
+    if add_to is not None:
+        _req(add_to, "add_to", torch.float32, 2)
+        if tuple(add_to.shape) != (n_src, n_in) or add_to.device != x.device:
+            raise ValueError("add_to %s does not fit x %s" % (tuple(add_to.shape), tuple(x.shape)))
+        grad_x = add_to
+    elif need_x:
+        grad_x = torch.empty(n_src, n_in, dtype=torch.float32, device=x.device)
+    grad_m = torch.empty_like(m)
+    ws = _workspace(lib.cxg_attention_logits_proj_workspace_bytes(n_in, heads), x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_attention_logits_proj_bwd_f32(_lib.ptr(x), ldx, m.data_ptr(), _lib.ptr(g_src), _lib.ptr(g_dst),
+                                                   n_src, n_dst, n_in, heads, _lib.ptr(grad_x), n_in,
+                                                   int(add_to is not None), grad_m.data_ptr(), ws.data_ptr(),
+                                                   ws.numel(), _lib.current_stream(x.device))
+    _lib.check(st)
+    return grad_x, grad_m
+
+
 def _bn_vec(t, name, c, device):
     if t is None:
         return None

@@ -490,6 +490,36 @@ int cxg_attention_logits_bwd_f32(const float* x, const float* att_src, const flo
                                  int accumulate, float* grad_att_src, float* grad_att_dst,
                                  void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same logits and gradients taken from the layer's input.  With xs = x_in W^T
+ * (W [heads*channels, in]) both logits are linear in x_in:
+ *   out_src[n, h] = x_in[n, :] . m[h, :],          m[h, :]         = sum_c att_src[h, c] W[h*channels + c, :]
+ *   out_dst[n, h] = x_in[n, :] . m[heads + h, :],  m[heads + h, :] = sum_c att_dst[h, c] W[h*channels + c, :]
+ * the contraction order upstream's single-head path uses (einsum "mn,nho,ho->mh",
+ * cxgnncomp/graph_conv.py:500-511); the several-head path computes the same numbers from
+ * xs (cxgnncomp/graph_conv.py:466-467), results agree to fp32 rounding.  The caller forms
+ * m [2*heads, in] (a tiny product).  x_in is [n_src, in] with row stride ldx (floats).
+ * Shapes: 4 | in <= 256, heads 1, 2, 4 or 8 (cxg_attention_logits_proj_supported);
+ * x_in, m, grad_x 16-byte aligned, strides multiples of 4; g_src / g_dst 16-byte aligned
+ * when heads is a multiple of 4.
+ * Backward, for g_src [n_src, heads], g_dst [n_dst, heads]:
+ *   grad_x[n, :]  (+)= sum_h g_src[n, h] m[h, :] + (n < n_dst) g_dst[n, h] m[heads + h, :]
+ *                     (grad_x NULL: skipped; accumulate != 0: added to what is there, the
+ *                     other gradient of x_in, from the linear map)
+ *   grad_m[h, :]         = sum_n g_src[n, h] x_in[n, :]
+ *   grad_m[heads + h, :] = sum_{n < n_dst} g_dst[n, h] x_in[n, :]
+ * from which the caller takes the logits' share of grad_att_* and grad_W by the chain rule
+ * through m.  Sums in a fixed order (reproducible). */
+int cxg_attention_logits_proj_supported(int in, int heads);
+int cxg_attention_logits_proj_fwd_f32(const float* x, int64_t ldx, const float* m, int64_t n_src,
+                                      int64_t n_dst, int in, int heads, float* out_src,
+                                      float* out_dst, void* stream);
+size_t cxg_attention_logits_proj_workspace_bytes(int in, int heads);
+int cxg_attention_logits_proj_bwd_f32(const float* x, int64_t ldx, const float* m,
+                                      const float* g_src, const float* g_dst, int64_t n_src,
+                                      int64_t n_dst, int in, int heads, float* grad_x, int64_t ldg,
+                                      int accumulate, float* grad_m, void* workspace,
+                                      size_t workspace_bytes, void* stream);
+
 /* Batch normalisation over the rows of x[n, c] (row stride ldx), the layer the upstream
  * models put between two convolutions (torch.nn.BatchNorm1d, cxgnncomp/model.py:28 and
  * its use followed by F.relu in GNN.forward_cxg, cxgnncomp/model.py:66-67).  Three calls:

@@ -170,7 +170,8 @@ def test_gat_configuration_full_size(big):
     assert abs(float(att_src.grad.double().sum()) - float(att_dst.grad.double().sum())) < 1e-2
 
 
-def test_gat_layer_full_size(big):
+@pytest.mark.parametrize("route", ["logits from xs", "logits from the input, slope 1", "logits from the input"])
+def test_gat_layer_full_size(big, route, monkeypatch):
     """MyGATConv 128 -> 4 x 64 on the 61.9M-edge graph: the layer's one autograd node (fused pass over
     the reversed graph with the edge-value gradient left in that pass's edge order, softmax backward
     reading it through the inverse permutation, bias in the aggregation's row stores) against the
@@ -178,22 +179,39 @@ def test_gat_layer_full_size(big):
     SpMMValOP, whose full-size results the test above holds against the oracle -- with the same
     parameters and the same output gradient: output, input gradient and every parameter gradient.
     Both sides compute the same sums in fp32, in different orders in places: 1e-4 of each tensor's
-    scale, 1e-5 absolute at that scale."""
+    scale, 1e-5 absolute at that scale.
+
+    The node takes the logits from the layer's input here (128 columns against 256 of xs), the
+    composition from xs: the two agree to rounding, ~1e-7.  LeakyReLU's derivative jumps at 0, so an
+    edge whose pre-activation lies within that rounding of 0 (a few dozen of 247 M) gets a gradient
+    that differs by the factor 1 - slope between the two sides, in any two fp32 implementations whose
+    logits are not bit-identical.  Hence three routes: the node with the logits from xs (bit-identical
+    logits on both sides, every tensor element by element, default slope); the node as shipped with
+    slope 1, where nothing jumps (every tensor element by element; grad att_dst is 0 in exact
+    arithmetic there and is held to 1e-5 of grad att_src's scale); and the node as shipped with the
+    default slope, where the output is held element by element, the input gradient may leave the
+    bound in at most 1e-4 of its rows and the parameter gradients (sums over every node) stay within
+    2e-3 of their scale."""
     import cxgnncomp
     import cxgnncomp_backend as B
+    from cxgnncomp_backend import _ops
     from cxgnncomp.graph_conv import AttentionLogitsOP, linear
     from cxgnncomp.graph_kernel import SpMMValOP
     cxgnncomp.set_timers()
     ptr, idx = big
     E = idx.shape[0]
     H, C = 4, 64
+    assert _ops.logits_proj_supported(128, H)
+    if route == "logits from xs":
+        monkeypatch.setattr(_ops, "logits_proj_supported", lambda n_in, heads: False)
+    slope = 1.0 if route.endswith("slope 1") else 0.2
     torch.manual_seed(4)
-    layer = cxgnncomp.MyGATConv(128, C, heads=H, concat=True).cuda()
+    layer = cxgnncomp.MyGATConv(128, C, heads=H, concat=True, negative_slope=slope).cuda()
     with torch.no_grad():
         layer.bias.normal_()
     x = (torch.randn(N_NODES, 128, device="cuda") / 4).requires_grad_(True)
     gout = torch.randn(N_NODES, H * C, device="cuda") / 16
-    announce("MyGATConv layer fwd+bwd full size")
+    announce("MyGATConv layer fwd+bwd full size, %s" % route)
     out = layer(x, ptr, idx, N_NODES, N_NODES, E)
     out.backward(gout)
     torch.cuda.synchronize()
@@ -212,12 +230,23 @@ def test_gat_layer_full_size(big):
     torch.cuda.synchronize()
     want = {"out": ref.detach(), "x": x.grad}
     want.update({k: v.grad for k, v in layer.named_parameters()})
+    tol = 1e-4 + 1e-5
+    jumps = route == "logits from the input"
     for k in want:
         assert got[k].shape == want[k].shape, k
         sc = max(1e-30, float(want[k].abs().max()))
-        err = float((got[k].double() - want[k].double()).abs().max()) / sc
-        tol = 1e-4 + 1e-5
-        assert err <= tol, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
+        if k == "att_dst" and slope == 1.0:
+            sc = float(want["att_src"].abs().max())
+        diff = (got[k].double() - want[k].double()).abs()
+        err = float(diff.max()) / sc
+        if not jumps or k in ("out", "bias"):
+            assert err <= tol, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
+        elif k == "x":
+            rows = int((diff.max(dim=1).values > tol * sc).sum())
+            assert rows <= 1e-4 * N_NODES, "%d rows of the input gradient leave the bound (largest %.3e)" % (rows, err)
+            assert err <= 0.1, "input gradient: largest difference %.3e of its scale" % err
+        else:
+            assert err <= 2e-3, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
     # and the node's own invariants: rows without edges hold the bias, nothing non-finite anywhere
     deg = ptr[1:] - ptr[:-1]
     empty = torch.nonzero(deg == 0).flatten()[:64]

@@ -262,6 +262,62 @@ def test_attention_logits_forward_backward(shape, n_src, n_dst):
     assert_close(_np(acc), base.numpy() + xd.grad.numpy(), RTOL, ATOL, "grad x added in place")
 
 
+PROJ_SHAPES = [(128, 4), (100, 4), (64, 8), (256, 2), (4, 1), (8, 4), (16, 8), (36, 1), (128, 8), (252, 4)]
+
+
+@pytest.mark.parametrize("shape", PROJ_SHAPES)
+@pytest.mark.parametrize("n_src,n_dst", [(1, 1), (1000, 0), (1000, 333), (70001, 70001), (70001, 12345)])
+def test_attention_logits_from_the_layer_input(shape, n_src, n_dst):
+    """The logits taken from the layer's input, ``x @ m[:H].T`` and ``x[:n_dst] @ m[H:].T``, and
+    their gradients against the same expressions differentiated in double precision (same
+    tolerances as the test above); rows of x with a stride, adding into an existing
+    gradient, and the call that skips grad_x."""
+    from cxgnncomp_backend import _ops
+    n_in, H = shape
+    assert _ops.logits_proj_supported(n_in, H)
+    torch.manual_seed(n_in * 100 + H + n_src)
+    wide = torch.randn(n_src, n_in + 4) / n_in ** 0.5
+    x = wide[:, :n_in]
+    m = torch.randn(2 * H, n_in)
+    gs, gd = torch.randn(n_src, H), torch.randn(n_dst, H)
+    xd, md = x.double().requires_grad_(True), m.double().requires_grad_(True)
+    ref_s, ref_d = xd @ md[:H].t(), xd[:n_dst] @ md[H:].t()
+    ((ref_s * gs.double()).sum() + (ref_d * gd.double()).sum()).backward()
+    announce("attention_logits_proj in=%d H=%d n_src=%d n_dst=%d" % (n_in, H, n_src, n_dst))
+    xg = wide.cuda()[:, :n_in]                       # row stride n_in + 4
+    out_s, out_d = _ops.attention_logits_proj(xg, m.cuda(), n_dst, H)
+    torch.cuda.synchronize()
+    assert out_s.shape == (n_src, H) and out_d.shape == (n_dst, H)
+    assert_close(_np(out_s), ref_s.detach().numpy(), RTOL, ATOL, "logits src")
+    assert_close(_np(out_d), ref_d.detach().numpy(), RTOL, ATOL, "logits dst")
+    out_s2, _ = _ops.attention_logits_proj(x.contiguous().cuda(), m.cuda(), n_dst, H)
+    assert torch.equal(out_s, out_s2)
+    announce("attention_logits_proj_bwd in=%d H=%d n_src=%d n_dst=%d" % (n_in, H, n_src, n_dst))
+    gx, gm = _ops.attention_logits_proj_bwd(xg, m.cuda(), gs.cuda(), gd.cuda(), H)
+    gx2, gm2 = _ops.attention_logits_proj_bwd(xg, m.cuda(), gs.cuda(), gd.cuda(), H)
+    none, gm3 = _ops.attention_logits_proj_bwd(xg, m.cuda(), gs.cuda(), gd.cuda(), H, need_x=False)
+    torch.cuda.synchronize()
+    assert none is None and torch.equal(gm, gm2) and torch.equal(gm, gm3) and torch.equal(gx, gx2)
+    assert_close(_np(gx), xd.grad.numpy(), RTOL, ATOL, "grad x")
+    ref_m = md.grad.numpy()
+    scale = max(1.0, float(np.abs(ref_m).max()))
+    assert_close(_np(gm) / scale, ref_m / scale, RTOL, ATOL, "grad m")
+    base = torch.randn(n_src, n_in, generator=torch.Generator().manual_seed(8))
+    acc = base.cuda()
+    gx3, gm4 = _ops.attention_logits_proj_bwd(xg, m.cuda(), gs.cuda(), gd.cuda(), H, add_to=acc)
+    assert gx3.data_ptr() == acc.data_ptr() and torch.equal(gm4, gm)
+    assert_close(_np(acc), base.numpy() + xd.grad.numpy(), RTOL, ATOL, "grad x added in place")
+
+
+def test_attention_logits_from_the_layer_input_rejects_other_shapes():
+    from cxgnncomp_backend import _ops
+    for n_in, H in [(130, 4), (260, 4), (128, 3), (128, 16), (2, 1)]:
+        assert not _ops.logits_proj_supported(n_in, H)
+    x, m = torch.zeros(8, 130, device="cuda"), torch.zeros(8, 130, device="cuda")
+    with pytest.raises(RuntimeError):
+        _ops.attention_logits_proj(x, m, 8, 4)
+
+
 def test_attention_logits_op_autograd():
     """The autograd wrapper used by MyGATConv: gradients flow to x and both parameters."""
     import cxgnncomp
