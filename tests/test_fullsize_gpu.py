@@ -190,8 +190,9 @@ def test_gat_layer_full_size(big, route, monkeypatch):
     slope 1, where nothing jumps (every tensor element by element; grad att_dst is 0 in exact
     arithmetic there and is held to 1e-5 of grad att_src's scale); and the node as shipped with the
     default slope, where the output is held element by element, the input gradient may leave the
-    bound in at most 1e-4 of its rows and the parameter gradients (sums over every node) stay within
-    2e-3 of their scale."""
+    bound in at most 64 of its 2.4 M rows (2 to 6 over three seeds) and by at most 1e-2 of its scale
+    (up to 9e-4 seen), and the parameter gradients (sums over every node) stay within 2e-3 of their
+    scale (up to 5e-4 seen)."""
     import cxgnncomp
     import cxgnncomp_backend as B
     from cxgnncomp_backend import _ops
@@ -243,8 +244,8 @@ def test_gat_layer_full_size(big, route, monkeypatch):
             assert err <= tol, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
         elif k == "x":
             rows = int((diff.max(dim=1).values > tol * sc).sum())
-            assert rows <= 1e-4 * N_NODES, "%d rows of the input gradient leave the bound (largest %.3e)" % (rows, err)
-            assert err <= 0.1, "input gradient: largest difference %.3e of its scale" % err
+            assert rows <= 64, "%d rows of the input gradient leave the bound (largest %.3e)" % (rows, err)
+            assert err <= 1e-2, "input gradient: largest difference %.3e of its scale" % err
         else:
             assert err <= 2e-3, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
     # and the node's own invariants: rows without edges hold the bias, nothing non-finite anywhere
