@@ -254,6 +254,18 @@ def c3(iters):
     g = torch.randn(N, H, C, device="cuda") / 8
     report("c3", "spmm_multihead_fwd H=4 C=64", timeit(lambda: _ops.spmm(ptr, idx, x, N, val=ev), iters),
            spmm_bytes(N, E, H * C, H), 2 * E * H * C)
+    # the GAT layer's forward aggregation when its input has 128 columns: the input rows gathered once
+    # under the four edge weights (out [N, 4, 128]), then one 128 -> 64 product per head
+    x_in = x.view(N, H * C)[:, :128].contiguous()
+    report("c3", "spmm, one gathered 128-float row under H=4 weights (out [N, 4, 128])",
+           timeit(lambda: _ops.spmm_weighted_heads(ptr, idx, ev, x_in, N), iters),
+           E * (4 * 128 + 8 + 4 * H) + 4 * N * H * 128 + 8 * (N + 1), 2 * E * H * 128)
+    from cxgnncomp_backend import _typed
+    aggr, w_heads = torch.randn(N, H, 128, device="cuda") / 8, torch.randn(H * C, 128, device="cuda") / 8
+    b_heads = torch.randn(H * C, device="cuda")
+    report("c3", "per-head products [N, 4, 128] x 4 [128, 64] + bias after that aggregation",
+           timeit(lambda: _typed.dense_linear_heads(aggr, w_heads, b_heads), iters), 4 * N * H * (128 + C), 2 * N * H * 128 * C)
+    del x_in, aggr, w_heads, b_heads
     import cxgnncomp_backend as B
     report("c3", "spmm_multihead PreReduce H=4 C=64 (heads summed inside the kernel, out [N, 64])",
            timeit(lambda: B.spmm_multihead(ptr, idx, ev, x, N, B.SPMM_MULTIHEAD_SCHEDULE.PreReduce), iters),

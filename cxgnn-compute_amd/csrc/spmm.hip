@@ -541,16 +541,21 @@ __device__ __forceinline__ void store_bf16x8(uint16_t* p, float8 v) {
 // a lane then gathers 16 bytes of a bf16 row like it does of an fp32 row, a 256-byte row takes 16
 // lanes and a step gathers four edges instead of two (a pair row of the relational layer has
 // three edges on average).
-template <typename IdxT, int V, int L, int WMODE, bool PERM, int IO = 0>
+// HM > 1 (WMODE == 3): every edge carries HM weights and the gathered row is added HM times, once per
+// weight, into HM output blocks of F floats: out[r, h, :] = sum_e val[e, h] * x[idx[e], :] (out rows
+// and carried partial rows of HM * F floats).  One gather of F floats serves HM heads.
+template <typename IdxT, int V, int L, int WMODE, bool PERM, int IO = 0, int HM = 1>
 __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   static_assert(IO == 0 || V == 4 || (V == 8 && (IO & 1)), "bf16 rows are handled four or eight values at a time");
   static_assert(V != 8 || (IO & 1), "eight values per lane: bf16 rows of x only");
+  static_assert((HM == 1) == (WMODE != 3), "several weights per edge are WMODE 3");
+  static_assert(HM == 1 || (IO == 0 && !PERM), "several weights per edge: fp32 rows, weights in edge order");
   using vec_t = typename Vec<V>::type;
   using raw_t = typename RawPiece<V, IO>::type;
   constexpr int G = CXG_WAVE / L;
   // steps requested together inside long rows (eight values per lane: half as many -- the same edges in
   // flight, and registers for eight waves per SIMD)
-  constexpr int UF = V == 8 ? (CXG_SPMM_GROUP_UF + 1) / 2 : CXG_SPMM_GROUP_UF;
+  constexpr int UF = (V == 8 || HM > 1) ? (CXG_SPMM_GROUP_UF + 1) / 2 : CXG_SPMM_GROUP_UF;
   const int lane = lane_id();
   const int wave = uniform_i32(threadIdx.x >> 6);
   const int64_t s = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -586,14 +591,21 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
 
   int head_of_lane = 0;
   if (WMODE == 2) head_of_lane = col_ok ? col / a.channels : 0;
-  vec_t acc = vzero<V>();
+  vec_t acc[HM];
+#pragma unroll
+  for (int h = 0; h < HM; ++h) acc[h] = vzero<V>();
   int row_take = 0;                          // most groups used by a step of the current row
-  float* const carry_head = a.carry + (size_t)(2 * s) * F;
-  float* const carry_tail = carry_head + F;
+  float* const carry_head = a.carry + (size_t)(2 * s) * F * HM;
+  float* const carry_tail = carry_head + F * HM;
 
   // What finish_row leaves in a row without edges.
   auto store_empty_row = [&](int64_t row) {
     if ((a.accumulate && !a.bias) || !col_ok) return;
+    if constexpr (HM > 1) {
+#pragma unroll
+      for (int h = 0; h < HM; ++h) *reinterpret_cast<vec_t*>(a.out + row * a.ldo + h * F + col) = vzero<V>();
+      return;
+    }
     if constexpr ((IO & 2) != 0) {
       uint16_t* d16 = reinterpret_cast<uint16_t*>(a.out) + row * a.ldo + col;
       *reinterpret_cast<uint2*>(d16) = make_uint2(0u, 0u);
@@ -659,45 +671,54 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
   }
   // sum of the groups' partials, valid in group 0 afterwards
   auto reduce_groups = [&]() {
-    if constexpr (L <= 1) { if (row_take > 1 / L) vshift_add<1>(acc); }
-    if constexpr (L <= 2) { if (row_take > 2 / L) vshift_add<2>(acc); }
-    if constexpr (L <= 4) { if (row_take > 4 / L) vshift_add<4>(acc); }
-    if constexpr (L <= 8) { if (row_take > 8 / L) vshift_add<8>(acc); }
-    if constexpr (L <= 16) { if (row_take > 16 / L) vshift_add<16>(acc); }
-    if constexpr (L <= 32) { if (row_take > 32 / L) vshift_add<32>(acc); }
+#pragma unroll
+    for (int h = 0; h < HM; ++h) {
+      if constexpr (L <= 1) { if (row_take > 1 / L) vshift_add<1>(acc[h]); }
+      if constexpr (L <= 2) { if (row_take > 2 / L) vshift_add<2>(acc[h]); }
+      if constexpr (L <= 4) { if (row_take > 4 / L) vshift_add<4>(acc[h]); }
+      if constexpr (L <= 8) { if (row_take > 8 / L) vshift_add<8>(acc[h]); }
+      if constexpr (L <= 16) { if (row_take > 16 / L) vshift_add<16>(acc[h]); }
+      if constexpr (L <= 32) { if (row_take > 32 / L) vshift_add<32>(acc[h]); }
+    }
   };
-  auto store_vec = [&](float* dst, vec_t v) {
-    if (writer) stream_store(dst + col, v);
+  auto store_vec = [&](float* dst, const vec_t (&v)[HM]) {
+#pragma unroll
+    for (int h = 0; h < HM; ++h) {
+      if (writer) stream_store(dst + h * F + col, v[h]);
+    }
   };
   auto finish_row = [&]() {
     reduce_groups();
     if (is_head) {
       store_vec(carry_head, acc);
+    } else if constexpr (HM > 1) {
+      store_vec(a.out + r * a.ldo, acc);
     } else if constexpr ((IO & 2) != 0) {
       if (a.mean) {
         const int deg = cur_end - cur_start;
-        if (deg > 0) vscale(acc, 1.0f / (float)deg);
+        if (deg > 0) vscale(acc[0], 1.0f / (float)deg);
       }
       if constexpr (V == 4) {
-        if (writer) store_bf16x4(reinterpret_cast<uint16_t*>(a.out) + r * a.ldo + col, acc);
+        if (writer) store_bf16x4(reinterpret_cast<uint16_t*>(a.out) + r * a.ldo + col, acc[0]);
       } else if constexpr (V == 8) {
-        if (writer) store_bf16x8(reinterpret_cast<uint16_t*>(a.out) + r * a.ldo + col, acc);
+        if (writer) store_bf16x8(reinterpret_cast<uint16_t*>(a.out) + r * a.ldo + col, acc[0]);
       }
     } else {
       float* dst = a.out + r * a.ldo;
       if (a.mean) {
         const int deg = cur_end - cur_start;
-        if (deg > 0) vscale(acc, 1.0f / (float)deg);
+        if (deg > 0) vscale(acc[0], 1.0f / (float)deg);
       }
       if (a.bias) {
-        if (writer) vadd(acc, *reinterpret_cast<const vec_t*>(a.bias + col));
+        if (writer) vadd(acc[0], *reinterpret_cast<const vec_t*>(a.bias + col));
       }
       if (a.accumulate) {
-        if (writer) vadd(acc, *reinterpret_cast<const vec_t*>(dst + col));
+        if (writer) vadd(acc[0], *reinterpret_cast<const vec_t*>(dst + col));
       }
       store_vec(dst, acc);
     }
-    acc = vzero<V>();
+#pragma unroll
+    for (int h = 0; h < HM; ++h) acc[h] = vzero<V>();
     row_take = 0;
   };
 
@@ -719,8 +740,8 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     // (the weight first: it comes out of a register that a load filled at the start of the chunk, and a
     // look at such a register behind a row request that may or may not have been issued -- the request
     // sits under a condition -- makes the compiler wait for everything in flight)
-    auto gather = [&](int e_idx, bool act, raw_t& v, float& w) {
-      if (WMODE == 1 && !PERM) w = __shfl(my_w, e_idx & 63, CXG_WAVE);
+    auto gather = [&](int e_idx, bool act, raw_t& v, float (&w)[HM]) {
+      if (WMODE == 1 && !PERM) w[0] = __shfl(my_w, e_idx & 63, CXG_WAVE);
       const int64_t src = shfl_i64(my_src, e_idx & 63);
       int64_t vrow = 0;
       if (WMODE != 0 && PERM) vrow = shfl_i64(my_vrow, e_idx & 63);
@@ -731,10 +752,31 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
         v = (act && col_ok) ? *reinterpret_cast<const raw_t*>(a.x + src * a.ldx + col) : zero_piece<raw_t>();
       }
       if (WMODE == 1) {
-        if (PERM) w = act ? a.val[vrow] : 0.f;
+        if (PERM) w[0] = act ? a.val[vrow] : 0.f;
       } else if (WMODE == 2) {
         if (!PERM) vrow = e0 + c0 + e_idx;
-        w = (act && col_ok) ? a.val[vrow * a.heads + head_of_lane] : 0.f;
+        w[0] = (act && col_ok) ? a.val[vrow * a.heads + head_of_lane] : 0.f;
+      } else if (WMODE == 3) {
+        // the HM weights of the edge: one address for all lanes of the group
+        const float* wp = a.val + (e0 + c0 + e_idx) * HM;
+        if constexpr (HM % 4 == 0) {
+#pragma unroll
+          for (int h = 0; h < HM; h += 4) {
+            const float4 q = act ? *reinterpret_cast<const float4*>(wp + h) : make_float4(0.f, 0.f, 0.f, 0.f);
+            w[h] = q.x; w[h + 1] = q.y; w[h + 2] = q.z; w[h + 3] = q.w;
+          }
+        } else {
+#pragma unroll
+          for (int h = 0; h < HM; ++h) w[h] = act ? wp[h] : 0.f;
+        }
+      }
+    };
+    auto add_edge = [&](const raw_t& v, const float (&w)[HM]) {
+      if (WMODE == 0) {
+        vadd(acc[0], widen_piece(v));
+      } else {
+#pragma unroll
+        for (int h = 0; h < HM; ++h) vfma(acc[h], widen_piece(v), w[h]);
       }
     };
     int j = 0;
@@ -746,23 +788,19 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
       const int left = (cur_end - (c0 + j)) < (cn - j) ? (cur_end - (c0 + j)) : (cn - j);
       if (left >= UF * G) {                   // long row: UF steps of G edges, loads first
         raw_t v[UF];
-        float w[UF];
+        float w[UF][HM];
 #pragma unroll
         for (int u = 0; u < UF; ++u) gather(j + u * G + g, true, v[u], w[u]);
 #pragma unroll
-        for (int u = 0; u < UF; ++u) {
-          if (WMODE == 0) vadd(acc, widen_piece(v[u]));
-          else vfma(acc, widen_piece(v[u]), w[u]);
-        }
+        for (int u = 0; u < UF; ++u) add_edge(v[u], w[u]);
         row_take = G;
         j += UF * G;
       } else {
         const int take = left < G ? left : G;
         raw_t v;
-        float w = 0.f;
+        float w[HM] = {};
         gather(j + g, g < take, v, w);
-        if (WMODE == 0) vadd(acc, widen_piece(v));
-        else vfma(acc, widen_piece(v), w);
+        add_edge(v, w);
         if (take > row_take) row_take = take;
         j += take;
       }
@@ -1306,6 +1344,56 @@ int cxg_spmm_bf16_rows(const int64_t* ptr, const int64_t* idx, const float* val,
     hipLaunchKernelGGL((spmm_fixup_kernel<int64_t, 2, false>), dim3(grid.x, (unsigned)(feat / 128), 1), block, 0, st, a);
   } else {
     hipLaunchKernelGGL((spmm_fixup_kernel<int64_t, 1, true>), dim3(grid.x, (unsigned)ceil_div(feat, CXG_WAVE), 1), block, 0, st, a);
+  }
+  CXG_LAUNCH_CHECK("spmm_fixup_kernel");
+  return CXG_OK;
+}
+
+// out[r, h, :] = sum_e val[e, h] * x[idx[e], :]: one gathered row of `feat` floats per edge, `heads` weights
+int cxg_spmm_weighted_heads_f32(const int64_t* ptr, const int64_t* idx, const float* val, const float* x, int64_t ldx,
+                                float* out, int64_t ldo, int64_t n_rows, int64_t n_edges_cap, int heads, int feat,
+                                unsigned flags, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace cxg;
+  CXG_REQUIRE(n_rows >= 0 && n_edges_cap >= 0, CXG_ERR_ARG, "negative size");
+  CXG_REQUIRE((flags & ~CXG_SPMM_HINT_EXACT_EDGES) == 0, CXG_ERR_ARG, "unknown flag");
+  CXG_REQUIRE((heads == 2 || heads == 4 || heads == 8) && feat >= 20 && feat <= 128 && feat % 4 == 0, CXG_ERR_UNSUPPORTED,
+              "heads = %d, feat = %d: takes 2, 4 or 8 heads and 20 <= feat <= 128, a multiple of 4", heads, feat);
+  if (n_rows == 0) return CXG_OK;
+  CXG_REQUIRE(ptr && out && (n_edges_cap == 0 || (idx && x && val)), CXG_ERR_ARG, "null pointer");
+  CXG_REQUIRE(ldx >= feat && ldo >= (int64_t)heads * feat && ldx % 4 == 0 && ldo % 4 == 0, CXG_ERR_ARG,
+              "row strides: at least feat / heads * feat, multiples of 4");
+  CXG_REQUIRE((((uintptr_t)x | (uintptr_t)out | (uintptr_t)val) & 15) == 0, CXG_ERR_ARG, "x, out and val must be 16-byte aligned");
+  const Plan plan = make_plan(n_edges_cap, (int64_t)heads * feat);
+  CXG_REQUIRE(workspace && workspace_bytes >= plan.tail_bytes + plan.carry_bytes && ((uintptr_t)workspace & 255) == 0,
+              CXG_ERR_WORKSPACE, "workspace of %zu bytes (256-byte aligned) needed", plan.tail_bytes + plan.carry_bytes);
+  SpmmArgs<int64_t> a;
+  a.ptr = ptr; a.idx = idx; a.x = x; a.out = out; a.val = val; a.perm = nullptr; a.ldx = ldx; a.ldo = ldo;
+  a.n_rows = n_rows; a.F = feat; a.heads = heads; a.channels = feat;
+  a.T = plan.T; a.exact_edges = 0; a.mean = 0; a.accumulate = 0;
+  a.tail_row = reinterpret_cast<int64_t*>(workspace);
+  a.carry = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + plan.tail_bytes);
+  a.mask = nullptr; a.mask_perm = nullptr; a.rel = nullptr; a.rel_stride = 0; a.src_map = nullptr; a.targets = nullptr;
+  a.dot_b = nullptr; a.ld_dot_b = 0; a.dot_out = nullptr; a.dot_at_edge = 0; a.bias = nullptr; a.out_bf16 = 0;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int L = feat > 64 ? 32 : (feat > 32 ? 16 : 8);
+  const dim3 grid((unsigned)ceil_div(plan.n_spans_cap, kWavesPerBlock), 1, 1), block(kBlock, 1, 1);
+  bool done = false;
+#define CXG_HM(LL, HH)                                                                                 \
+  if (!done && L == LL && heads == HH) {                                                               \
+    hipLaunchKernelGGL((spmm_group_kernel<int64_t, 4, LL, 3, false, 0, HH>), grid, block, 0, st, a);     \
+    done = true;                                                                                       \
+  }
+  CXG_HM(8, 2) CXG_HM(8, 4) CXG_HM(8, 8) CXG_HM(16, 2) CXG_HM(16, 4) CXG_HM(16, 8) CXG_HM(32, 2) CXG_HM(32, 4) CXG_HM(32, 8)
+#undef CXG_HM
+  CXG_REQUIRE(done, CXG_ERR_UNSUPPORTED, "no kernel for this combination");
+  CXG_LAUNCH_CHECK("spmm_group_kernel");
+  // the carried partial rows and the output rows are heads * feat floats to the fix-up kernel
+  SpmmArgs<int64_t> f = a;
+  f.F = heads * feat;
+  if (f.F % 128 == 0) {
+    hipLaunchKernelGGL((spmm_fixup_kernel<int64_t, 2, false>), dim3(grid.x, (unsigned)(f.F / 128), 1), block, 0, st, f);
+  } else {
+    hipLaunchKernelGGL((spmm_fixup_kernel<int64_t, 1, true>), dim3(grid.x, (unsigned)ceil_div(f.F, CXG_WAVE), 1), block, 0, st, f);
   }
   CXG_LAUNCH_CHECK("spmm_fixup_kernel");
   return CXG_OK;

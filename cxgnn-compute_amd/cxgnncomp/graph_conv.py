@@ -486,7 +486,13 @@ class GatLayerOP(torch.autograd.Function):
     ``x @ m.T`` with ``m = att @ W`` per head -- the contraction order of the single-head
     path's einsum (upstream cxgnncomp/graph_conv.py:500-511); their backward pass then adds a
     rank-2H term to the input gradient and returns grad m, from which the shares of the weight
-    and attention-vector gradients follow by the chain rule on [2H, in] tensors."""
+    and attention-vector gradients follow by the chain rule on [2H, in] tensors.  Where the input
+    has at most half the columns of the transformed features and the rows have eight edges or
+    more on average, the forward aggregation gathers input rows under the H edge weights
+    (``sum_e ev[e, h] x[idx[e]]``, [num_dst, H, in]) and transforms per head afterwards -- the
+    order "aggregate, then transform" that upstream's single-head path takes when
+    in < out (cxgnncomp/graph_conv.py:513-527); the transformed features are then formed in the
+    backward pass only, which needs them for the edge-value gradient."""
 
     @staticmethod
     def _logit_rows(w, att_src, att_dst, H, C):
@@ -496,16 +502,31 @@ class GatLayerOP(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w, att_src, att_dst, bias, ptr, idx, num_dst, num_src, num_edge, slope, heads, concat):
         H, C = heads, w.shape[0] // heads
-        xs = _mm(x[:num_src], w.t()).view(-1, H, C)
-        from_input = (x.shape[1] < H * C and _ops.logits_proj_supported(x.shape[1], H) and x.stride(1) == 1
+        n_in = x.shape[1]
+        from_input = (n_in < H * C and _ops.logits_proj_supported(n_in, H) and x.stride(1) == 1
                       and x.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0)
+        # aggregate the input rows under the H edge weights, then transform per head: half the gathered
+        # bytes or less; pays from about eight edges per destination row on
+        aggr_first = (from_input and 2 * n_in <= H * C and _ops.spmm_heads_supported(H, n_in)
+                      and num_edge >= 8 * num_dst)
+        xs = None if aggr_first else _mm(x[:num_src], w.t()).view(-1, H, C)
         if from_input:
             a_src, a_dst = _ops.attention_logits_proj(x[:num_src], GatLayerOP._logit_rows(w, att_src, att_dst, H, C),
                                                       num_dst, H)
         else:
             a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
         ev, mask = _ops.edge_softmax_fwd(ptr, idx, a_dst, a_src, num_edge, slope)
-        if concat:
+        if aggr_first:
+            aggr = _ops.spmm_weighted_heads(ptr, idx, ev, x[:num_src], num_dst)
+            if concat:
+                out = _typed.dense_linear_heads(aggr, w, bias)
+            else:
+                # mean over heads of aggr[:, h] @ W_h^T = one product over K = H * in
+                out = _mm(aggr.view(-1, H * n_in), w.view(H, C, n_in).transpose(1, 2).reshape(H * n_in, C)).div_(H)
+                if bias is not None:
+                    out.add_(bias)
+            del aggr
+        elif concat:
             # the bias goes into the aggregation's row stores
             out = _ops.spmm(ptr, idx, xs, num_dst, val=ev, bias=bias).view(-1, H * C)
         else:
@@ -521,6 +542,8 @@ class GatLayerOP(torch.autograd.Function):
         x, w, att_src, att_dst, xs, ev, mask, ptr, idx = ctx.saved_tensors
         num_dst, num_src, H, C, concat, slope, has_bias, from_input = ctx.dims
         g = g.contiguous()
+        if xs is None:                       # the forward pass aggregated the input rows and never formed them
+            xs = _mm(x[:num_src], w.t()).view(-1, H, C)
         g_bias = _ops.column_sum(g) if has_bias and ctx.needs_input_grad[4] else None
         if concat:
             g3 = g.view(-1, H, C)

@@ -30,6 +30,7 @@ SIGNATURES = {
     "cxg_spmm_sum_f32_i32": (_I32, [_P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
     "cxg_spmm_weighted_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32,
                                      _U32, _P, _SZ, _P]),
+    "cxg_spmm_weighted_heads_f32": (_I32, [_P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32, _U32, _P, _SZ, _P]),
     "cxg_spmm_bf16_rows": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _P, _I64, _I32, _I64, _I64, _I32, _U32, _P, _SZ, _P]),
     "cxg_spmm_prereduce_f32": (_I32, [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32,
                                       _U32, _P, _SZ, _P]),

@@ -149,6 +149,35 @@ def spmm_bf16_rows(ptr, idx, x, n_rows, val=None, val_perm=None, out_bf16=False,
     return out
 
 
+def spmm_heads_supported(heads, feat):
+    """Shapes cxg_spmm_weighted_heads_f32 takes."""
+    return heads in (2, 4, 8) and 20 <= feat <= 128 and feat % 4 == 0
+
+
+def spmm_weighted_heads(ptr, idx, val, x, n_rows):
+    """out[r, h, :] = sum_e val[e, h] * x[idx[e], :] for val [E, H] and x [n_src, F] (rows may be
+    strided): one gathered row per edge under H weights; returns [n_rows, H, F]."""
+    lib = _lib.load()
+    _check_graph(ptr, idx, n_rows)
+    _req(val, "val", torch.float32, 2)
+    if x.dim() != 2 or x.dtype != torch.float32 or not x.is_cuda or (x.shape[1] != 1 and x.stride(1) != 1):
+        raise ValueError("x must be a [N, F] float32 CUDA tensor with contiguous rows")
+    heads, feat = val.shape[1], x.shape[1]
+    if val.shape[0] < idx.shape[0]:
+        raise ValueError("val has %d rows for %d edges" % (val.shape[0], idx.shape[0]))
+    out = torch.empty((n_rows, heads, feat), dtype=torch.float32, device=x.device)
+    if n_rows == 0:
+        return out
+    ldx = x.stride(0) if x.shape[0] > 1 else feat
+    ws = _workspace(lib.cxg_spmm_workspace_bytes(idx.shape[0], heads * feat), x.device)
+    with torch.cuda.device(x.device):
+        st = lib.cxg_spmm_weighted_heads_f32(ptr.data_ptr(), _lib.ptr(idx), _lib.ptr(val), _lib.ptr(x), ldx,
+                                             out.data_ptr(), heads * feat, n_rows, idx.shape[0], heads, feat, 0,
+                                             ws.data_ptr(), ws.numel(), _lib.current_stream(x.device))
+    _lib.check(st)
+    return out
+
+
 def clear_graph_cache():
     _C.clear_graph_cache()
 

@@ -204,6 +204,35 @@ def dense_linear(x, w_kn, bias=None, addend=None):
     return out
 
 
+def dense_linear_heads(x, weight, bias=None):
+    """out[:, h*C:(h+1)*C] = x[:, h, :] @ weight[h*C:(h+1)*C, :].T (+ bias) for x [M, H, K] and a
+    layer weight [H*C, K]: the per-head products that follow an aggregation of the layer's input
+    under H weights.  One launch of the split GEMM per head over strided rows (row stride H*K in,
+    H*C out; bias in the epilogue); shapes the kernel does not take go through torch.bmm."""
+    M, H, K = x.shape
+    C = weight.shape[0] // H
+    flags = _PRECISION_FLAGS.get(GEMM_PRECISION, 0)
+    ok = (flags == GEMM_SPLIT_F16X3 and x.is_cuda and x.dtype == torch.float32 and weight.dtype == torch.float32
+          and x.is_contiguous() and M >= DENSE_MIN_ROWS and K <= 128 and K % 4 == 0 and C % 4 == 0
+          and x.data_ptr() % 16 == 0 and (bias is None or (bias.dtype == torch.float32 and bias.is_contiguous()
+                                                           and bias.numel() == H * C)))
+    if not ok:
+        out = torch.bmm(x.transpose(0, 1), weight.view(H, C, K).transpose(1, 2)).transpose(0, 1).reshape(M, H * C)
+        return out if bias is None else out.add_(bias)
+    lib = _lib.load()
+    w_kn = weight.view(H, C, K).transpose(1, 2).contiguous()          # [H, K, C]
+    out = torch.empty((M, H * C), dtype=torch.float32, device=x.device)
+    seg = _one_segment(M, x.device)
+    with torch.cuda.device(x.device):
+        for h in range(H):
+            st = lib.cxg_typed_gemm_epilogue_f32(x.data_ptr() + 4 * h * K, H * K, w_kn.data_ptr() + 4 * h * K * C,
+                                                 None if bias is None else bias.data_ptr() + 4 * h * C, None, 0,
+                                                 out.data_ptr() + 4 * h * C, H * C, None, None, seg.data_ptr(),
+                                                 M, K, C, 1, flags, _lib.current_stream(x.device))
+            _lib.check(st)
+    return out
+
+
 def dense_linear_add_(out, x, w_kn):
     """out [M, N] += x [M, K] @ w_kn [K, N] in place through the typed GEMM (one segment);
     False when the shapes are not taken (nothing is written then)."""

@@ -136,6 +136,24 @@ int cxg_spmm_prereduce_f32(const int64_t* ptr, const int64_t* idx, const float* 
                            void* stream);
 
 /*
+ * Edge-weighted aggregation of ONE gathered row under several weights:
+ *   out[r, h, :] = sum_e val[e, h] * x[idx[e], :]      (x [n_src, feat], out [n_rows, heads, feat]).
+ * Where a multi-head layer's features are a linear map of a narrower input, xs[:, h, :] = x W_h^T,
+ * its aggregation sum_e val[e, h] xs[idx[e], h, :] equals out[r, h, :] W_h^T: the edges gather
+ * feat floats instead of heads * channels, the product follows per destination row (the order
+ * "aggregate, then transform" of MyGATConv.forward_1, cxgnncomp/graph_conv.py:513-527, applied to
+ * forward_many's aggregation, :488-490).  Takes 2, 4 or 8 heads and 20 <= feat <= 128, a
+ * multiple of 4; x, out and val 16-byte aligned, strides multiples of 4; otherwise
+ * CXG_ERR_UNSUPPORTED.  Workspace: cxg_spmm_workspace_bytes(n_edges_cap, heads * feat).
+ * Deterministic (no atomics), like the other aggregations.
+ */
+int cxg_spmm_weighted_heads_f32(const int64_t* ptr, const int64_t* idx, const float* val,
+                                const float* x, int64_t ldx, float* out, int64_t ldo,
+                                int64_t n_rows, int64_t n_edges_cap, int heads, int feat,
+                                unsigned flags, void* workspace, size_t workspace_bytes,
+                                void* stream);
+
+/*
  * Single-head aggregation (sum, CXG_SPMM_MEAN, or one weight per edge, optionally read through
  * val_perm) of rows of 4 .. 128 values (a multiple of 4) whose rows are bf16 on the gathered
  * side (x_bf16), on the stored side (out_bf16), or both; sums are formed in fp32 and rounded to

@@ -528,18 +528,22 @@ def test_sage_layer_on_a_row_prefix(widths):
         assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "frozen input, grad " + k)
 
 
-@pytest.mark.parametrize("heads_channels", [(4, 8), (4, 64)])
+@pytest.mark.parametrize("heads_channels", [(4, 8), (4, 64), (2, 32), (8, 16)])
 @pytest.mark.parametrize("concat", [True, False])
-def test_gat_layer_on_a_row_prefix(concat, heads_channels):
+@pytest.mark.parametrize("max_deg", [12, 40])
+def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
     """MyGATConv (several heads, one autograd node on CUDA) on a sampled-batch layer: num_dst
     destination rows over num_src source rows of a longer x; output and every gradient against
-    the float64 composition of the upstream expressions."""
+    the float64 composition of the upstream expressions.  With about 20 edges per row and an
+    input of 24 columns against 64 or more of transformed features the layer aggregates the
+    input rows under the H edge weights and transforms afterwards; with about 6 it aggregates
+    the transformed rows."""
     import cxgnncomp
     cxgnncomp.set_timers()               # MyGATConv brackets its phases with TimerOP, as upstream
     torch.manual_seed(6)
     n_all, n_src, n_dst, fin = 700, 600, 200, 24
     H, C = heads_channels       # 4 x 64 = 256 floats per row: the backward pass with the fused edge products
-    deg = torch.randint(0, 12, (n_dst,))
+    deg = torch.randint(0, max_deg, (n_dst,))
     deg[3] = 0
     ptr = torch.zeros(n_dst + 1, dtype=torch.int64)
     ptr[1:] = torch.cumsum(deg, 0)
@@ -551,7 +555,7 @@ def test_gat_layer_on_a_row_prefix(concat, heads_channels):
     with torch.no_grad():
         layer.bias.normal_()
     xg = x.cuda().requires_grad_(True)
-    announce("GatLayerOP prefix rows concat=%s" % concat)
+    announce("GatLayerOP prefix rows concat=%s H=%d C=%d E=%d" % (concat, H, C, E))
     out = layer(xg, ptr.cuda(), idx.cuda(), n_dst, n_src, E)
     w = torch.randn(*out.shape)
     (out * w.cuda()).sum().backward()

@@ -121,6 +121,60 @@ def test_spmm_width_sweep(feat):
     assert torch.equal(got, got2)
 
 
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "no_edges", "one_hub", "c2", "empty_runs"])
+@pytest.mark.parametrize("heads,feat", [(4, 128), (2, 128), (8, 128), (4, 100), (4, 64), (2, 40), (8, 24), (4, 20)])
+def test_spmm_one_gathered_row_under_several_weights(kind, heads, feat):
+    """cxg_spmm_weighted_heads_f32: out[r, h, :] = sum_e val[e, h] x[idx[e], :].  Every head against
+    the oracle's weighted SpMM with that head's column of weights (1e-4 / 1e-5), bit for bit
+    against the single-weight kernel (the same additions in the same order), rows of x with a
+    stride, a row prefix, and run-to-run equality."""
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    if kind == "c2":
+        if (heads, feat) not in ((4, 128), (2, 40)):
+            pytest.skip("the large graph runs two shapes")
+        ptr, idx = S.powerlaw_directed_symmetrised(169343, 1166243, seed=3)
+    elif kind == "empty_runs":
+        ptr, idx, _ = _graph_with_empty_runs(5)
+    else:
+        ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    assert _ops.spmm_heads_supported(heads, feat)
+    torch.manual_seed(heads * 1000 + feat)
+    wide = torch.randn(n, feat + 4) * _scale(ptr)
+    x = wide[:, :feat]
+    val = torch.rand(E, heads) + 0.25
+    pc, ic = ptr.cuda(), idx.cuda()
+    announce("spmm several weights kind=%s H=%d F=%d n=%d E=%d" % (kind, heads, feat, n, E))
+    got = _ops.spmm_weighted_heads(pc, ic, val.cuda(), wide.cuda()[:, :feat], n)
+    torch.cuda.synchronize()
+    assert got.shape == (n, heads, feat)
+    xc = x.contiguous().cuda()
+    assert torch.equal(got, _ops.spmm_weighted_heads(pc, ic, val.cuda(), xc, n))
+    for h in range(heads):
+        vh = val[:, h].contiguous()
+        want = oracle.spmm(ptr.numpy(), idx.numpy(), x.contiguous().numpy(), n, val=vh.numpy())
+        sc = max(1.0, float(np.abs(want).max()))
+        assert_close(got[:, h].cpu().numpy() / sc, want / sc, RTOL, ATOL, "head %d" % h)
+        if E > 0:
+            assert torch.equal(got[:, h], _ops.spmm(pc, ic, xc, n, val=vh.cuda())), "head %d against the single-weight kernel" % h
+    rows = n // 3
+    if rows > 0:
+        part = _ops.spmm_weighted_heads(pc, ic, val.cuda(), xc, rows)
+        assert torch.equal(part, got[:rows])
+
+
+def test_spmm_several_weights_rejects_other_shapes():
+    from cxgnncomp_backend import _ops
+    ptr, idx = _graph("uniform")
+    n, E = ptr.shape[0] - 1, idx.shape[0]
+    for heads, feat in [(3, 128), (4, 132), (4, 16), (16, 64), (4, 30)]:
+        assert not _ops.spmm_heads_supported(heads, feat)
+        with pytest.raises(RuntimeError):
+            _ops.spmm_weighted_heads(ptr.cuda(), idx.cuda(), torch.zeros(E, heads).cuda(), torch.zeros(n, feat).cuda(), n)
+
+
 def _graph_with_empty_runs(seed):
     """Long runs of rows without edges at the start, in the middle (two of them inside one
     64-edge span, one across a span boundary) and at the end, between rows of 1-3 edges and

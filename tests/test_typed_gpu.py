@@ -507,6 +507,26 @@ def test_dense_linear_helpers_match_library(M, K, N):
     assert _typed.dense_linear(x.double(), w.t().double(), b.double()) is None
 
 
+@pytest.mark.parametrize("M,H,K,C", [(70001, 4, 128, 64), (5003, 2, 100, 32), (8192, 8, 24, 16), (9000, 4, 36, 20),
+                                     (300, 4, 128, 64), (6000, 4, 132, 64)])
+def test_dense_linear_heads(M, H, K, C):
+    """dense_linear_heads (the per-head products after GatLayerOP's aggregation of the input rows):
+    out[:, h*C:(h+1)*C] = x[:, h, :] @ W_h^T (+ bias) against float64, on shapes the split GEMM
+    takes (one launch per head over strided rows) and on shapes that go through torch.bmm."""
+    from cxgnncomp_backend import _typed
+    gen = torch.Generator().manual_seed(M + K)
+    x = (torch.randn(M, H, K, generator=gen) / K ** 0.5).cuda()
+    w = torch.randn(H * C, K, generator=gen).cuda()
+    b = torch.randn(H * C, generator=gen).cuda()
+    want = torch.einsum("mhk,hck->mhc", x.double(), w.double().view(H, C, K)).reshape(M, H * C)
+    announce("dense_linear_heads M=%d H=%d K=%d C=%d" % (M, H, K, C))
+    got = _typed.dense_linear_heads(x, w, b)
+    assert got.shape == (M, H * C)
+    assert_close(_np(got), _np(want + b.double()), RTOL, 2 * ATOL, "per-head products with bias")
+    got = _typed.dense_linear_heads(x, w)
+    assert_close(_np(got), _np(want), RTOL, 2 * ATOL, "per-head products")
+
+
 def test_linear_op_gradients_through_typed_gemm():
     """LinearOP on a shape dense_linear takes: output and the three gradients against float64
     autograd of F.linear."""
