@@ -333,6 +333,17 @@ def c3(iters):
         layer(xin, ptr, idx, N, N, E).backward(gout)
     report("c3", "MyGATConv 128 -> 4x64 fwd+bwd (linear, softmax, SpMM, SDDMM)", timeit(gat_step, max(2, iters // 3)))
     del layer, xin
+    # one head, the reference's default (MyGATConv.forward_1): both orders of aggregation and transform
+    for fin, fout in ((128, 256), (256, 256), (256, 64)):
+        layer = cxgnncomp.MyGATConv(fin, fout, heads=1).cuda()
+        xin = torch.randn(N, fin, device="cuda").requires_grad_(True)
+        gout1 = torch.randn(N, fout, device="cuda") / 16
+
+        def gat1_step():
+            xin.grad = None
+            layer(xin, ptr, idx, N, N, E).backward(gout1)
+        report("c3", "MyGATConv one head %d -> %d fwd+bwd" % (fin, fout), timeit(gat1_step, max(2, iters // 3)))
+        del layer, xin, gout1
     torch.cuda.empty_cache()
     # scheduling helpers (index work): bytes = arrays read + written once
     new_ptr, _ = cxgnncomp.neighbor_grouping(ptr, 32)

@@ -509,14 +509,21 @@ class GatLayerOP(torch.autograd.Function):
         # bytes or less; pays from about eight edges per destination row on
         aggr_first = (from_input and 2 * n_in <= H * C and _ops.spmm_heads_supported(H, n_in)
                       and num_edge >= 8 * num_dst)
-        xs = None if aggr_first else _mm(x[:num_src], w.t()).view(-1, H, C)
+        # one head and a narrower input: the whole layer is "aggregate the input rows, then transform"
+        # (the branch upstream's forward_1 takes), forward and backward on rows of `in` floats
+        single_first = from_input and H == 1 and x.is_contiguous()
+        xs = None if (aggr_first or single_first) else _mm(x[:num_src], w.t()).view(-1, H, C)
         if from_input:
             a_src, a_dst = _ops.attention_logits_proj(x[:num_src], GatLayerOP._logit_rows(w, att_src, att_dst, H, C),
                                                       num_dst, H)
         else:
             a_src, a_dst = _ops.attention_logits(xs, att_src, att_dst, num_dst)
         ev, mask = _ops.edge_softmax_fwd(ptr, idx, a_dst, a_src, num_edge, slope)
-        if aggr_first:
+        aggr = None
+        if single_first:
+            aggr = _ops.spmm(ptr, idx, x[:num_src], num_dst, val=ev.view(-1))
+            out = _mm(aggr, w.t(), bias)
+        elif aggr_first:
             aggr = _ops.spmm_weighted_heads(ptr, idx, ev, x[:num_src], num_dst)
             if concat:
                 out = _typed.dense_linear_heads(aggr, w, bias)
@@ -525,7 +532,7 @@ class GatLayerOP(torch.autograd.Function):
                 out = _mm(aggr.view(-1, H * n_in), w.view(H, C, n_in).transpose(1, 2).reshape(H * n_in, C)).div_(H)
                 if bias is not None:
                     out.add_(bias)
-            del aggr
+            aggr = None
         elif concat:
             # the bias goes into the aggregation's row stores
             out = _ops.spmm(ptr, idx, xs, num_dst, val=ev, bias=bias).view(-1, H * C)
@@ -533,15 +540,57 @@ class GatLayerOP(torch.autograd.Function):
             out = _ops.spmm(ptr, idx, xs, num_dst, val=ev).mean(dim=1)
             if bias is not None:
                 out.add_(bias)
-        ctx.save_for_backward(x, w, att_src, att_dst, xs, ev, mask, ptr, idx)
+        ctx.save_for_backward(x, w, att_src, att_dst, xs, ev, mask, ptr, idx, aggr)
         ctx.dims = (num_dst, num_src, H, C, concat, float(slope), bias is not None, from_input)
         return out
 
     @staticmethod
+    def _backward_single_first(ctx, g, x, w, att_src, att_dst, ev, mask, ptr, idx, aggr):
+        """One head, input narrower than the output: out = (sum_e ev x[src]) W^T + bias.  The
+        gradient rows g W have `in` columns; they are what the pass over the reversed graph
+        aggregates, and their products with the source rows of x are the edge-value gradient."""
+        num_dst, num_src, H, C, concat, slope, has_bias, from_input = ctx.dims
+        g_bias = _ops.column_sum(g) if has_bias and ctx.needs_input_grad[4] else None
+        g_w = _weight_grad(aggr, g) if ctx.needs_input_grad[1] else None
+        gw_rows = _mm(g, w)                                       # [num_dst, in]
+        xs_rows = x[:num_src]
+        n_in = x.shape[1]
+        tg = _ops.transposed(ptr, idx, num_dst, num_src)
+        g_ev = torch.empty((ev.shape[0], 1), dtype=torch.float32, device=g.device)
+        if tg.n_edges < ev.shape[0]:
+            g_ev[tg.n_edges:].zero_()
+        if _ops.spmm_dot_supported(1, n_in):
+            g_x, g_ev = _ops.spmm_dot(tg.ptr_t, tg.idx_t, gw_rows.view(-1, 1, n_in), num_src, ev, tg.perm,
+                                      xs_rows.view(-1, 1, n_in), g_ev, dot_at_edge=True)
+            g_x = g_x.view(-1, n_in)
+            g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope,
+                                                   grad_pos=_ops.inverse_perm_transposed(tg))
+        else:
+            g_x = _ops.spmm(tg.ptr_t, tg.idx_t, gw_rows, num_src, val=ev.view(-1), val_perm=tg.perm)
+            g_ev = _ops.sddmm_csr(ptr, idx, xs_rows.view(-1, 1, n_in), gw_rows.view(-1, 1, n_in), num_dst, out=g_ev)
+            g_adst, t_edge = _ops.edge_softmax_bwd(ptr, ev, mask, g_ev, num_dst, slope)
+        g_asrc = _ops.narrow_gather_sum(tg.ptr_t, tg.perm, t_edge, num_src, rows32=_ops.rows32_transposed(tg))
+        m = GatLayerOP._logit_rows(w, att_src, att_dst, 1, C)
+        need_x = ctx.needs_input_grad[0]
+        _, g_m = _ops.attention_logits_proj_bwd(xs_rows, m, g_asrc, g_adst, 1, add_to=g_x if need_x else None,
+                                                need_x=False)
+        g_att_src, g_att_dst = g_m[0:1] @ w.t(), g_m[1:2] @ w.t()           # [1, C]
+        if g_w is not None:
+            g_w.addmm_(att_src.reshape(C, 1), g_m[0:1]).addmm_(att_dst.reshape(C, 1), g_m[1:2])
+        if not need_x:
+            g_x = None
+        elif g_x.shape[0] < x.shape[0]:
+            g_x = torch.cat([g_x, g_x.new_zeros(x.shape[0] - g_x.shape[0], n_in)])
+        return (g_x, g_w, g_att_src.view_as(att_src), g_att_dst.view_as(att_dst), g_bias,
+                None, None, None, None, None, None, None, None)
+
+    @staticmethod
     def backward(ctx, g):
-        x, w, att_src, att_dst, xs, ev, mask, ptr, idx = ctx.saved_tensors
+        x, w, att_src, att_dst, xs, ev, mask, ptr, idx, aggr = ctx.saved_tensors
         num_dst, num_src, H, C, concat, slope, has_bias, from_input = ctx.dims
         g = g.contiguous()
+        if aggr is not None:
+            return GatLayerOP._backward_single_first(ctx, g, x, w, att_src, att_dst, ev, mask, ptr, idx, aggr)
         if xs is None:                       # the forward pass aggregated the input rows and never formed them
             xs = _mm(x[:num_src], w.t()).view(-1, H, C)
         g_bias = _ops.column_sum(g) if has_bias and ctx.needs_input_grad[4] else None
@@ -675,6 +724,13 @@ class MyGATConv(torch.nn.Module):
         return out + self.bias if self.bias is not None else out
 
     def forward_1(self, x, ptr, idx, num_dst, num_src, num_edge):
+        if x.is_cuda and x.dim() == 2 and self.edge_softmax_schedule == "fused" and self.out_channels % 4 == 0:
+            # the same layer node as several heads take; it picks the order of aggregation and
+            # transform by the widths, as the expressions below do
+            x = TimerOP.apply(x, "gat layer", True)
+            out = GatLayerOP.apply(x, self.lin_src, self.att_src, self.att_dst, self.bias, ptr, idx, int(num_dst),
+                                   int(num_src), int(num_edge), self.negative_slope, 1, True)
+            return TimerOP.apply(out, "gat layer", False)
         w = self.lin_src.T.view(-1, self.heads, self.out_channels)
         x = TimerOP.apply(x, "einsum1", True)
         alpha_src = torch.einsum("mn,nho,ho->mh", x, w, self.att_src.squeeze(0)).view(-1, self.heads)

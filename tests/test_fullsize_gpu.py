@@ -256,6 +256,55 @@ def test_gat_layer_full_size(big, route, monkeypatch):
     assert all(bool(torch.isfinite(t).all()) for t in got.values())
 
 
+@pytest.mark.parametrize("fin,C", [(128, 256), (256, 512), (256, 64)])
+def test_gat_single_head_layer_full_size(big, fin, C):
+    """MyGATConv with one head on the 61.9M-edge graph -- 128 -> 256 (input rows aggregated, then
+    transformed; backward on 128-float rows), 256 -> 512 (the same with the backward pass over the
+    reversed graph that also leaves the edge-value gradient) and 256 -> 64 (transformed rows
+    aggregated) -- against the composition of the separately verified operators, as for several
+    heads above.  Slope 1, where LeakyReLU has no kink and the two sides' differently rounded
+    logits cannot put an edge on different sides of it: every tensor element by element, 1e-4 of
+    its scale + 1e-5 (grad att_dst is 0 in exact arithmetic there: 1e-5 of grad att_src's scale)."""
+    import cxgnncomp
+    import cxgnncomp_backend as B
+    from cxgnncomp.graph_conv import AttentionLogitsOP, linear
+    from cxgnncomp.graph_kernel import SpMMValOP
+    cxgnncomp.set_timers()
+    ptr, idx = big
+    E = idx.shape[0]
+    torch.manual_seed(fin + C)
+    layer = cxgnncomp.MyGATConv(fin, C, heads=1, negative_slope=1.0).cuda()
+    with torch.no_grad():
+        layer.bias.normal_()
+    x = (torch.randn(N_NODES, fin, device="cuda") / 4).requires_grad_(True)
+    gout = torch.randn(N_NODES, C, device="cuda") / 16
+    announce("MyGATConv one head %d -> %d fwd+bwd full size" % (fin, C))
+    out = layer(x, ptr, idx, N_NODES, N_NODES, E)
+    out.backward(gout)
+    torch.cuda.synchronize()
+    got = {"out": out.detach(), "x": x.grad.clone()}
+    got.update({k: v.grad.clone() for k, v in layer.named_parameters()})
+    x.grad = None
+    for v in layer.parameters():
+        v.grad = None
+    del out
+    announce("the same layer as a composition of its operators, full size")
+    xs = linear(x, layer.lin_src).view(-1, 1, C)
+    a_src, a_dst = AttentionLogitsOP.apply(xs, layer.att_src, layer.att_dst, N_NODES)
+    ev = B.edge_attention(ptr=ptr, idx=idx, att_dst=a_dst, att_src=a_src, num_edge=E, relu_l=1.0)
+    ref = SpMMValOP.apply(xs, ptr, idx, ev, N_NODES).view(-1, C) + layer.bias
+    ref.backward(gout)
+    torch.cuda.synchronize()
+    want = {"out": ref.detach(), "x": x.grad}
+    want.update({k: v.grad for k, v in layer.named_parameters()})
+    for k in want:
+        assert got[k].shape == want[k].shape, k
+        sc = max(1e-30, float(want["att_src" if k == "att_dst" else k].abs().max()))
+        err = float((got[k].double() - want[k].double()).abs().max()) / sc
+        assert err <= 1e-4 + 1e-5, "%s: largest difference %.3e of the tensor's scale %.3e" % (k, err, sc)
+    assert all(bool(torch.isfinite(t).all()) for t in got.values())
+
+
 def test_gspmm_full_size(big):
     """GSpMM_u MAX / GSpMM_u_e MIN x ADD on the full graph (thousands of rows above the
     512-edge piece size, hubs of ~17 k edges): exact against torch.segment_reduce over

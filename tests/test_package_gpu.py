@@ -528,21 +528,11 @@ def test_sage_layer_on_a_row_prefix(widths):
         assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "frozen input, grad " + k)
 
 
-@pytest.mark.parametrize("heads_channels", [(4, 8), (4, 64), (2, 32), (8, 16)])
-@pytest.mark.parametrize("concat", [True, False])
-@pytest.mark.parametrize("max_deg", [12, 40])
-def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
-    """MyGATConv (several heads, one autograd node on CUDA) on a sampled-batch layer: num_dst
-    destination rows over num_src source rows of a longer x; output and every gradient against
-    the float64 composition of the upstream expressions.  With about 20 edges per row and an
-    input of 24 columns against 64 or more of transformed features the layer aggregates the
-    input rows under the H edge weights and transforms afterwards; with about 6 it aggregates
-    the transformed rows."""
+def _gat_layer_on_a_row_prefix(H, C, concat, max_deg, fin, frozen=False):
     import cxgnncomp
     cxgnncomp.set_timers()               # MyGATConv brackets its phases with TimerOP, as upstream
     torch.manual_seed(6)
-    n_all, n_src, n_dst, fin = 700, 600, 200, 24
-    H, C = heads_channels       # 4 x 64 = 256 floats per row: the backward pass with the fused edge products
+    n_all, n_src, n_dst = 700, 600, 200
     deg = torch.randint(0, max_deg, (n_dst,))
     deg[3] = 0
     ptr = torch.zeros(n_dst + 1, dtype=torch.int64)
@@ -550,12 +540,12 @@ def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
     E = int(ptr[-1])
     idx = torch.randint(0, n_src, (E,))
     dst = torch.repeat_interleave(torch.arange(n_dst), deg)
-    x = torch.randn(n_all, fin)
+    x = torch.randn(n_all, fin) / (fin / 24) ** 0.5
     layer = cxgnncomp.MyGATConv(fin, C, heads=H, concat=concat).cuda()
     with torch.no_grad():
         layer.bias.normal_()
-    xg = x.cuda().requires_grad_(True)
-    announce("GatLayerOP prefix rows concat=%s H=%d C=%d E=%d" % (concat, H, C, E))
+    xg = x.cuda().requires_grad_(not frozen)
+    announce("GatLayerOP prefix rows concat=%s H=%d C=%d in=%d E=%d frozen=%s" % (concat, H, C, fin, E, frozen))
     out = layer(xg, ptr.cuda(), idx.cuda(), n_dst, n_src, E)
     w = torch.randn(*out.shape)
     (out * w.cuda()).sum().backward()
@@ -571,12 +561,41 @@ def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
     (ref * w.double()).sum().backward()
     assert out.shape == ref.shape
     assert_close(_np(out), ref.detach().numpy(), 2e-4, 2e-5, "fwd")
-    assert xg.grad.shape == x.shape and float(xg.grad[n_src:].abs().max()) == 0.0
-    sc = max(1.0, float(x64.grad.abs().max()))
-    assert_close(_np(xg.grad) / sc, x64.grad.numpy() / sc, 2e-4, 2e-5, "grad x")
+    if frozen:
+        assert xg.grad is None
+    else:
+        assert xg.grad.shape == x.shape and float(xg.grad[n_src:].abs().max()) == 0.0
+        sc = max(1.0, float(x64.grad.abs().max()))
+        assert_close(_np(xg.grad) / sc, x64.grad.numpy() / sc, 2e-4, 2e-5, "grad x")
     for k, v in layer.named_parameters():
         sc = max(1.0, float(P[k].grad.abs().max()))
         assert_close(_np(v.grad) / sc, P[k].grad.numpy() / sc, 2e-4, 2e-5, "grad " + k)
+
+
+@pytest.mark.parametrize("heads_channels", [(4, 8), (4, 64), (2, 32), (8, 16)])
+@pytest.mark.parametrize("concat", [True, False])
+@pytest.mark.parametrize("max_deg", [12, 40])
+def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
+    """MyGATConv (several heads, one autograd node on CUDA) on a sampled-batch layer: num_dst
+    destination rows over num_src source rows of a longer x; output and every gradient against
+    the float64 composition of the upstream expressions.  With about 20 edges per row and an
+    input of 24 columns against 64 or more of transformed features the layer aggregates the
+    input rows under the H edge weights and transforms afterwards; with about 6 it aggregates
+    the transformed rows."""
+    H, C = heads_channels       # 4 x 64 = 256 floats per row: the backward pass with the fused edge products
+    _gat_layer_on_a_row_prefix(H, C, concat, max_deg, 24)
+
+
+@pytest.mark.parametrize("fin,C", [(24, 64), (24, 16), (24, 24), (256, 512), (256, 256), (128, 256), (100, 128), (30, 64)])
+@pytest.mark.parametrize("frozen", [False, True])
+def test_gat_single_head_layer_on_a_row_prefix(fin, C, frozen):
+    """MyGATConv with one head (upstream's forward_1, cxgnncomp/graph_conv.py:497-545) on the same
+    layer node: an input narrower than the output is aggregated first and transformed afterwards,
+    forward and backward on rows of `in` floats (with 256 columns the backward pass over the
+    reversed graph also leaves the edge-value gradient; 30 columns are not a multiple of 4 and
+    take the transformed rows); otherwise the transformed rows are aggregated.  Output and every
+    gradient against float64, also with an input that needs no gradient."""
+    _gat_layer_on_a_row_prefix(1, C, False, 40, fin, frozen)
 
 
 @pytest.mark.parametrize("opname", ["RGCNOP", "RGCNOP2", "TypedLinearS2DSort"])
