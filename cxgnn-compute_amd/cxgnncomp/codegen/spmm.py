@@ -2,7 +2,7 @@
 by name; the work is done by the edge-span SpMM kernels."""
 import torch
 
-from cxgnncomp_backend import _ops
+from cxgnncomp_backend import _ops, _typed
 
 
 def spmm_triton(x, ptr, idx, num_nodes, val=None):
@@ -13,4 +13,5 @@ def spmm_triton(x, ptr, idx, num_nodes, val=None):
 def spmm_mm_triton(x, ptr, idx, weight, num_nodes):
     """Aggregate, then multiply by ``weight`` given transposed ([out, in]) as upstream."""
     agg = _ops.spmm(ptr, idx, x.contiguous(), int(num_nodes))
-    return torch.mm(agg, weight.t())
+    out = _typed.dense_linear(agg, weight.t())        # the split GEMM where it takes the shape
+    return out if out is not None else torch.mm(agg, weight.t())
