@@ -544,8 +544,14 @@ __device__ __forceinline__ void store_bf16x8(uint16_t* p, float8 v) {
 // HM > 1 (WMODE == 3): every edge carries HM weights and the gathered row is added HM times, once per
 // weight, into HM output blocks of F floats: out[r, h, :] = sum_e val[e, h] * x[idx[e], :] (out rows
 // and carried partial rows of HM * F floats).  One gather of F floats serves HM heads.
-template <typename IdxT, int V, int L, int WMODE, bool PERM, int IO = 0, int HM = 1>
+// DOT: beside the aggregation, dot_out[p] = <x[idx[p], :], dot_b[r, :]> for every edge position p of row r
+// (the product of the gathered row with the row the sums go to).  A group forms its edge's product when
+// the gathered row arrives; the products of a 64-edge chunk are collected lane by lane in one register
+// (a scalar read of the group's first lane and a select, no memory) and leave with one contiguous store per chunk.  The row of dot_b for the
+// next output row is requested one row ahead.
+template <typename IdxT, int V, int L, int WMODE, bool PERM, int IO = 0, int HM = 1, bool DOT = false>
 __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
+  static_assert(!DOT || (HM == 1 && IO == 0 && V == 4), "edge products: fp32 rows of 16-byte pieces, one weight per edge");
   static_assert(IO == 0 || V == 4 || (V == 8 && (IO & 1)), "bf16 rows are handled four or eight values at a time");
   static_assert(V != 8 || (IO & 1), "eight values per lane: bf16 rows of x only");
   static_assert((HM == 1) == (WMODE != 3), "several weights per edge are WMODE 3");
@@ -595,6 +601,19 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
 #pragma unroll
   for (int h = 0; h < HM; ++h) acc[h] = vzero<V>();
   int row_take = 0;                          // most groups used by a step of the current row
+  // DOT: the row of dot_b that belongs to output row r, and the one after it (requested a row ahead)
+  vec_t brow = vzero<V>(), brow_next = vzero<V>();
+  int64_t brow_next_row = -1;
+  auto load_brow_row = [&](int64_t row) -> vec_t {
+    return (row >= 0 && row < n_rows && col_ok) ? *reinterpret_cast<const vec_t*>(a.dot_b + row * a.ld_dot_b + col) : vzero<V>();
+  };
+  auto enter_row = [&]() {                    // r has changed
+    if constexpr (DOT) {
+      brow = (r == brow_next_row) ? brow_next : load_brow_row(r);
+      brow_next_row = r + 1;
+      brow_next = load_brow_row(brow_next_row);
+    }
+  };
   float* const carry_head = a.carry + (size_t)(2 * s) * F * HM;
   float* const carry_tail = carry_head + F * HM;
 
@@ -669,6 +688,7 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
     skip_rows_without_edges(0);
     cur_end = (r < n_rows) ? bcast_i32(row_ends, (int)(r - rbase)) : 0x7fffffff;
   }
+  enter_row();
   // sum of the groups' partials, valid in group 0 afterwards
   auto reduce_groups = [&]() {
 #pragma unroll
@@ -779,11 +799,28 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
         for (int h = 0; h < HM; ++h) vfma(acc[h], widen_piece(v), w[h]);
       }
     };
+    // DOT: the product of chunk edge i ends up in lane i of my_dot
+    float my_dot = 0.f;
+    auto note_products = [&](const raw_t& v, int first_edge, int n_groups) {
+      if constexpr (DOT) {
+        const float total = lane_group_sum<L>(vdot4(widen_piece(v), brow));     // in the group's first lane
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi) {
+          if (gi < n_groups) {
+            const int sv = __builtin_amdgcn_readlane((int)__float_as_uint(total), gi * L);
+            if (lane == ((first_edge + gi) & 63)) my_dot = __uint_as_float((unsigned)sv);
+          }
+        }
+      }
+    };
     int j = 0;
     while (j < cn) {
-      while (c0 + j >= cur_end) {
-        finish_row();
-        next_row(true);
+      if (c0 + j >= cur_end) {
+        do {
+          finish_row();
+          next_row(true);
+        } while (c0 + j >= cur_end);
+        enter_row();
       }
       const int left = (cur_end - (c0 + j)) < (cn - j) ? (cur_end - (c0 + j)) : (cn - j);
       if (left >= UF * G) {                   // long row: UF steps of G edges, loads first
@@ -792,7 +829,10 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
 #pragma unroll
         for (int u = 0; u < UF; ++u) gather(j + u * G + g, true, v[u], w[u]);
 #pragma unroll
-        for (int u = 0; u < UF; ++u) add_edge(v[u], w[u]);
+        for (int u = 0; u < UF; ++u) {
+          add_edge(v[u], w[u]);
+          note_products(v[u], j + u * G, G);
+        }
         row_take = G;
         j += UF * G;
       } else {
@@ -801,9 +841,13 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(SpmmArgs<IdxT> a) {
         float w[HM] = {};
         gather(j + g, g < take, v, w);
         add_edge(v, w);
+        note_products(v, j, take);
         if (take > row_take) row_take = take;
         j += take;
       }
+    }
+    if constexpr (DOT) {
+      if (lane < cn) stream_store(a.dot_out + (e0 + c0 + lane), my_dot);
     }
   }
 
@@ -1147,6 +1191,27 @@ int spmm_common(const IdxT* ptr, const IdxT* idx, const float* val, const int64_
       const uintptr_t align_bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)a.carry | (uintptr_t)dot->b |
                                    (uintptr_t)a.bias |
                                    (uintptr_t)(ldx * 4) | (uintptr_t)(ldo * 4) | (uintptr_t)(dot->ld_b * 4);
+      if (heads == 1 && F <= 128 && F % 4 == 0 && F >= 16 && (align_bits & 15) == 0 && perm && dot->at_edge && !a.mean &&
+          !a.accumulate && !a.bias) {
+        // narrow single-head rows: the grouped-lane kernel forms the products (weights through perm,
+        // products at the edge's own position)
+        a.dot_b = dot->b; a.ld_dot_b = dot->ld_b; a.dot_out = dot->out; a.dot_at_edge = 1;
+        // the lane groups of the plain weighted aggregation of this width: the sums agree bit for bit
+        const int L = F > 64 ? 32 : (F > 32 ? 16 : (F > 16 ? 8 : 4));
+        const dim3 grid((unsigned)ceil_div(plan.n_spans_cap, kWavesPerBlock), 1, 1), block(kBlock, 1, 1);
+        if (L == 32) hipLaunchKernelGGL((spmm_group_kernel<IdxT, 4, 32, 1, true, 0, 1, true>), grid, block, 0, st, a);
+        else if (L == 16) hipLaunchKernelGGL((spmm_group_kernel<IdxT, 4, 16, 1, true, 0, 1, true>), grid, block, 0, st, a);
+        else if (L == 8) hipLaunchKernelGGL((spmm_group_kernel<IdxT, 4, 8, 1, true, 0, 1, true>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((spmm_group_kernel<IdxT, 4, 4, 1, true, 0, 1, true>), grid, block, 0, st, a);
+        CXG_LAUNCH_CHECK("spmm_group_kernel");
+        if (F % 128 == 0) {
+          hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 2, false>), dim3(grid.x, (unsigned)(F / 128), 1), block, 0, st, a);
+        } else {
+          hipLaunchKernelGGL((spmm_fixup_kernel<IdxT, 1, true>), dim3(grid.x, (unsigned)ceil_div(F, CXG_WAVE), 1), block, 0, st, a);
+        }
+        CXG_LAUNCH_CHECK("spmm_fixup_kernel");
+        return CXG_OK;
+      }
       CXG_REQUIRE(F % 256 == 0 && (align_bits & 15) == 0 &&
                       (channels == 32 || channels == 64 || channels == 128 || channels == 256),
                   CXG_ERR_UNSUPPORTED, "spmm with dot products needs heads*channels %% 256 == 0, channels in "

@@ -559,7 +559,8 @@ class GatLayerOP(torch.autograd.Function):
         g_ev = torch.empty((ev.shape[0], 1), dtype=torch.float32, device=g.device)
         if tg.n_edges < ev.shape[0]:
             g_ev[tg.n_edges:].zero_()
-        if _ops.spmm_dot_supported(1, n_in):
+        # (rows under 96 floats: reading the products back through positions costs what the fused pass saves)
+        if n_in >= 96 and _ops.spmm_dot_supported(1, n_in, at_edge=True):
             g_x, g_ev = _ops.spmm_dot(tg.ptr_t, tg.idx_t, gw_rows.view(-1, 1, n_in), num_src, ev, tg.perm,
                                       xs_rows.view(-1, 1, n_in), g_ev, dot_at_edge=True)
             g_x = g_x.view(-1, n_in)
@@ -602,7 +603,7 @@ class GatLayerOP(torch.autograd.Function):
         g_ev = torch.empty((ev.shape[0], H), dtype=torch.float32, device=g.device)
         if tg.n_edges < ev.shape[0]:
             g_ev[tg.n_edges:].zero_()
-        if _ops.spmm_dot_supported(H, C):
+        if H * C >= 96 and _ops.spmm_dot_supported(H, C, at_edge=True):
             # one pass over the reversed graph gathers the rows of g once for both results; the
             # edge-value gradient stays in that pass's edge order (contiguous stores) and the
             # softmax backward reads it through the inverse permutation

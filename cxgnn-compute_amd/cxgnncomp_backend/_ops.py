@@ -63,9 +63,13 @@ def spmm(ptr, idx, x, n_rows, *, mean=False, val=None, val_perm=None, out=None, 
     return _C.spmm(ptr, idx, x, int(n_rows), mean, val, val_perm, out, accumulate, bias)
 
 
-def spmm_dot_supported(heads, channels):
-    """Shapes ``spmm_dot`` takes (the others use spmm and sddmm_csr)."""
-    return (heads * channels) % 256 == 0 and channels in (32, 64, 128, 256)
+def spmm_dot_supported(heads, channels, at_edge=False):
+    """Shapes ``spmm_dot`` takes (the others use spmm and sddmm_csr): rows of 256 * k floats, and --
+    with the weights read through ``val_perm`` and the products left at the edge's own position
+    (``at_edge``) -- single-head rows of 16 .. 128 floats, a multiple of 4."""
+    if (heads * channels) % 256 == 0 and channels in (32, 64, 128, 256):
+        return True
+    return bool(at_edge) and heads == 1 and 16 <= channels <= 128 and channels % 4 == 0
 
 
 def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out, dot_at_edge=False):
@@ -94,8 +98,9 @@ def spmm_dot(ptr, idx, x, n_rows, val, val_perm, dot_b, dot_out, dot_at_edge=Fal
             raise ValueError("dot_out must have a row per row of val")
     elif val.shape[0] < idx.shape[0] or dot_out.shape[0] < idx.shape[0]:
         raise ValueError("val / dot_out shorter than idx")
-    if not spmm_dot_supported(heads, channels):
-        raise ValueError("spmm_dot needs heads*channels %% 256 == 0 and channels in (32, 64, 128, 256)")
+    if not spmm_dot_supported(heads, channels, at_edge=dot_at_edge and val_perm is not None):
+        raise ValueError("spmm_dot needs heads*channels %% 256 == 0 and channels in (32, 64, 128, 256), or -- with "
+                         "val_perm and dot_at_edge -- one head of 16 .. 128 channels, a multiple of 4")
     row = heads * channels
     out = torch.empty((n_rows, heads, channels), dtype=torch.float32, device=x.device)
     if n_rows == 0:

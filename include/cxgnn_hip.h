@@ -194,7 +194,9 @@ int cxg_spmm_weighted_bias_f32(const int64_t* ptr, const int64_t* idx, const flo
  * store per edge (a consumer then reads row e of the original order at the inverse
  * permutation's position, see cxg_edge_softmax_bwd_at_f32).
  * Shapes: heads*channels a multiple of 256, channels in {32, 64, 128, 256}, 16-byte
- * aligned rows (CXG_ERR_UNSUPPORTED otherwise: use the two separate calls).
+ * aligned rows; also one head of 16 .. 128 channels (a multiple of 4) when val is read
+ * through val_perm and CXG_SPMM_DOT_AT_EDGE is set (the single-head layer's backward pass
+ * on narrow rows).  CXG_ERR_UNSUPPORTED otherwise: use the two separate calls.
  */
 int cxg_spmm_weighted_dot_f32(const int64_t* ptr, const int64_t* idx, const float* val,
                               const int64_t* val_perm, const float* x, int64_t ldx, float* out,

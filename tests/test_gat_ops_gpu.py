@@ -382,6 +382,51 @@ def test_spmm_with_edge_dot_products(kind, shape):
     assert torch.equal(dot3[inv], dot)
 
 
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub", "c2", "empty_runs"])
+@pytest.mark.parametrize("feat", [128, 64, 100, 36, 24, 16])
+def test_spmm_with_edge_dot_products_on_narrow_rows(kind, feat):
+    """cxg_spmm_weighted_dot_f32 for one head of 16 .. 128 channels (weights through the
+    transposition's permutation, products left at the edge's own position in the reversed graph):
+    the aggregation equals the plain weighted SpMM bit for bit, the products equal the oracle's
+    SDDMM of the original graph read through the permutation; rows of the reversed graph that
+    cross spans, hubs, rows without edges."""
+    from cxgnncomp import synthetic as S
+    from cxgnncomp_backend import _ops
+    from test_spmm_gpu import _graph_with_empty_runs
+    if kind == "c2":
+        if feat not in (128, 36):
+            pytest.skip("the large graph runs two widths")
+        ptr, idx = S.powerlaw_directed_symmetrised(169343, 1166243, seed=3)
+    elif kind == "empty_runs":
+        ptr, idx, _ = _graph_with_empty_runs(5)
+    else:
+        ptr, idx = _graph(kind)
+    n = ptr.shape[0] - 1
+    E = idx.shape[0]
+    assert _ops.spmm_dot_supported(1, feat, at_edge=True) and (feat == 256 or not _ops.spmm_dot_supported(1, feat))
+    torch.manual_seed(feat)
+    xs = torch.randn(n, 1, feat) / 8
+    g = torch.randn(n, 1, feat) / 8
+    ev = torch.rand(E, 1)
+    pc, ic = ptr.cuda(), idx.cuda()
+    tg = _ops.transposed(pc, ic, n, n)
+    announce("spmm_dot narrow rows kind=%s F=%d n=%d E=%d" % (kind, feat, n, E))
+    dot = torch.full((E, 1), float("nan"), device="cuda")
+    gx, dot = _ops.spmm_dot(tg.ptr_t, tg.idx_t, g.cuda(), n, ev.cuda(), tg.perm, xs.cuda(), dot, dot_at_edge=True)
+    want_gx = _ops.spmm(tg.ptr_t, tg.idx_t, g.cuda().view(n, feat), n, val=ev.cuda().view(-1), val_perm=tg.perm)
+    torch.cuda.synchronize()
+    assert torch.equal(gx.view(n, feat), want_gx)
+    rows = np.repeat(np.arange(n), np.diff(ptr.numpy()))
+    ref = oracle.sddmm(idx.numpy(), rows, xs.numpy(), g.numpy()).reshape(E, 1)
+    perm = tg.perm.cpu().numpy()
+    assert_close(_np(dot), ref[perm], RTOL, ATOL, "edge dot products in the reversed graph's edge order")
+    gx2, dot2 = _ops.spmm_dot(tg.ptr_t, tg.idx_t, g.cuda(), n, ev.cuda(), tg.perm, xs.cuda(), torch.empty_like(dot),
+                              dot_at_edge=True)
+    assert torch.equal(gx2, gx) and torch.equal(dot2, dot)
+    with pytest.raises(ValueError):
+        _ops.spmm_dot(tg.ptr_t, tg.idx_t, g.cuda(), n, ev.cuda(), tg.perm, xs.cuda(), dot)      # not at the edge
+
+
 @pytest.mark.parametrize("kind", ["uniform", "powerlaw", "empty_rows", "one_hub"])
 @pytest.mark.parametrize("heads", [1, 2, 4, 8, 3])
 def test_edge_softmax_backward_reads_the_gradient_through_positions(kind, heads):

@@ -586,15 +586,17 @@ def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
     _gat_layer_on_a_row_prefix(H, C, concat, max_deg, 24)
 
 
-@pytest.mark.parametrize("fin,C", [(24, 64), (24, 16), (24, 24), (256, 512), (256, 256), (128, 256), (100, 128), (30, 64)])
+@pytest.mark.parametrize("fin,C", [(24, 64), (24, 16), (24, 24), (256, 512), (256, 256), (128, 256), (100, 128), (30, 64),
+                                   (256, 128), (256, 100)])
 @pytest.mark.parametrize("frozen", [False, True])
 def test_gat_single_head_layer_on_a_row_prefix(fin, C, frozen):
     """MyGATConv with one head (upstream's forward_1, cxgnncomp/graph_conv.py:497-545) on the same
     layer node: an input narrower than the output is aggregated first and transformed afterwards,
-    forward and backward on rows of `in` floats (with 256 columns the backward pass over the
+    forward and backward on rows of `in` floats (from 96 columns on the backward pass over the
     reversed graph also leaves the edge-value gradient; 30 columns are not a multiple of 4 and
-    take the transformed rows); otherwise the transformed rows are aggregated.  Output and every
-    gradient against float64, also with an input that needs no gradient."""
+    take the transformed rows); otherwise the transformed rows are aggregated (with the fused
+    backward pass from 96 output columns on).  Output and every gradient against float64, also
+    with an input that needs no gradient."""
     _gat_layer_on_a_row_prefix(1, C, False, 40, fin, frozen)
 
 
