@@ -559,9 +559,31 @@ struct SageFunction : public torch::autograd::Function<SageFunction> {
     }
     const Tensor& x = saved[2];
     const Tensor& ev = saved[3];
+    const bool need_ev = ctx->saved_data["ev_needs_grad"].toBool();
+    const int64_t heads = ev.dim() == 2 ? ev.size(1) : 1;
+    const int64_t channels = x.size(-1);
+    const int64_t row = heads * channels;
+    // Rows of 256 * k floats: ONE pass over the reversed graph gathers the rows of grad_out for the
+    // input gradient and multiplies them with the source's own row of x for the edge-value
+    // gradient (stored at the edge's original position), instead of an aggregation and an SDDMM
+    // that each gather every row once.
+    if (need_ev && row % 256 == 0 && (channels == 32 || channels == 64 || channels == 128 || channels == 256) &&
+        ev.size(0) == idx.size(0) && grad_out.numel() == n * row && n_src > 0 && g->n_edges > 0) {
+      gx = torch::empty({n_src, row}, x.options());
+      gval = torch::empty({ev.size(0), heads}, ev.options());
+      if (g->n_edges < ev.size(0)) gval.narrow(0, g->n_edges, ev.size(0) - g->n_edges).zero_();
+      const int64_t n_cap = g->idx_t.size(0);
+      Tensor ws = workspace(cxg_spmm_workspace_bytes(n_cap, row), x);
+      c10::DeviceGuard guard(x.device());
+      check(cxg_spmm_weighted_dot_f32((const int64_t*)g->ptr_t.data_ptr(), (const int64_t*)ptr_or_null(g->idx_t),
+                                      (const float*)ev.data_ptr(), (const int64_t*)ptr_or_null(g->perm),
+                                      (const float*)grad_out.data_ptr(), row, (float*)gx.data_ptr(), row,
+                                      (const float*)x.data_ptr(), row, (float*)gval.data_ptr(), n_src, n_cap, (int)heads,
+                                      (int)channels, 0u, ws.data_ptr(), (size_t)ws.numel(), stream_of(x)));
+      return {gx.reshape(x_shape), Tensor(), Tensor(), gval.reshape(ev.sizes()), Tensor(), Tensor()};
+    }
     gx = spmm(g->ptr_t, g->idx_t, grad_out, n_src, false, ev, g->perm, c10::nullopt, false, c10::nullopt);
-    if (ctx->saved_data["ev_needs_grad"].toBool())
-      gval = sddmm_csr(ptr, idx, x, grad_out, n, c10::nullopt).reshape(ev.sizes());
+    if (need_ev) gval = sddmm_csr(ptr, idx, x, grad_out, n, c10::nullopt).reshape(ev.sizes());
     return {gx.reshape(x_shape), Tensor(), Tensor(), gval, Tensor(), Tensor()};
   }
 };

@@ -89,7 +89,8 @@ def test_run_spmm_configurable_bwd_and_int32(kind):
 
 
 @pytest.mark.parametrize("kind", ["uniform", "powerlaw", "one_hub"])
-@pytest.mark.parametrize("shape", [(1, 128), (1, 40), (4, 64), (2, 24), (3, 100), (8, 16), (8, 8), (4, 4)])
+@pytest.mark.parametrize("shape", [(1, 128), (1, 40), (4, 64), (2, 24), (3, 100), (8, 16), (8, 8), (4, 4), (1, 256), (2, 128),
+                                   (8, 32), (1, 512)])
 def test_weighted_spmm_forward_backward(kind, shape):
     import cxgnncomp_backend as B
     H, C = shape
