@@ -513,6 +513,9 @@ Tensor rows32_transposed(TransposedGraph& g) {
 // ---------------------------------------------------------------------------------------------
 // sum / mean / edge-weighted aggregation with autograd (SAGEFunction, SAGEEdgeValueFunction)
 // ---------------------------------------------------------------------------------------------
+Tensor inverse_perm_transposed(TransposedGraph& g);
+Tensor gather_rows(const Tensor& inp, const Tensor& sel);
+
 struct SageFunction : public torch::autograd::Function<SageFunction> {
   static Tensor forward(AutogradContext* ctx, Tensor x, Tensor ptr, Tensor idx, OptTensor edge_value, int64_t num_node,
                         bool mean) {
@@ -569,17 +572,27 @@ struct SageFunction : public torch::autograd::Function<SageFunction> {
     // that each gather every row once.
     if (need_ev && row % 256 == 0 && (channels == 32 || channels == 64 || channels == 128 || channels == 256) &&
         ev.size(0) == idx.size(0) && grad_out.numel() == n * row && n_src > 0 && g->n_edges > 0) {
+      // (the products leave the pass in its own edge order -- contiguous stores -- and one row gather
+      // through the inverse permutation puts them into the original order: faster than scattering
+      // them from the pass, the same bits)
       gx = torch::empty({n_src, row}, x.options());
-      gval = torch::empty({ev.size(0), heads}, ev.options());
-      if (g->n_edges < ev.size(0)) gval.narrow(0, g->n_edges, ev.size(0) - g->n_edges).zero_();
+      Tensor in_pass_order = torch::empty({ev.size(0), heads}, ev.options());
       const int64_t n_cap = g->idx_t.size(0);
       Tensor ws = workspace(cxg_spmm_workspace_bytes(n_cap, row), x);
       c10::DeviceGuard guard(x.device());
       check(cxg_spmm_weighted_dot_f32((const int64_t*)g->ptr_t.data_ptr(), (const int64_t*)ptr_or_null(g->idx_t),
                                       (const float*)ev.data_ptr(), (const int64_t*)ptr_or_null(g->perm),
                                       (const float*)grad_out.data_ptr(), row, (float*)gx.data_ptr(), row,
-                                      (const float*)x.data_ptr(), row, (float*)gval.data_ptr(), n_src, n_cap, (int)heads,
-                                      (int)channels, 0u, ws.data_ptr(), (size_t)ws.numel(), stream_of(x)));
+                                      (const float*)x.data_ptr(), row, (float*)in_pass_order.data_ptr(), n_src, n_cap,
+                                      (int)heads, (int)channels, CXG_SPMM_DOT_AT_EDGE, ws.data_ptr(), (size_t)ws.numel(),
+                                      stream_of(x)));
+      Tensor ordered = gather_rows(in_pass_order, inverse_perm_transposed(*g));       // [n_edges, heads]
+      if (g->n_edges == ev.size(0)) {
+        gval = ordered;
+      } else {
+        gval = torch::zeros({ev.size(0), heads}, ev.options());
+        gval.narrow(0, 0, g->n_edges).copy_(ordered);
+      }
       return {gx.reshape(x_shape), Tensor(), Tensor(), gval.reshape(ev.sizes()), Tensor(), Tensor()};
     }
     gx = spmm(g->ptr_t, g->idx_t, grad_out, n_src, false, ev, g->perm, c10::nullopt, false, c10::nullopt);

@@ -37,10 +37,16 @@ class SpMMValOP(torch.autograd.Function):
                 and _ops.spmm_dot_supported(x.shape[1], x.shape[2]) and val.shape[0] == idx.shape[0]):
             # both gradients from one pass over the reversed graph: the rows of grad_out gathered
             # for grad_x are also multiplied with the row of x they are added into
-            grad_val = torch.empty_like(val)
-            if g.n_edges < val.shape[0]:
-                grad_val[g.n_edges:].zero_()
-            grad_x, grad_val = _ops.spmm_dot(g.ptr_t, g.idx_t, grad_out, x.shape[0], val, g.perm, x, grad_val)
+            # the products leave the pass in its own edge order (contiguous stores) and are put into
+            # the original order by one 4H-byte row gather: faster than scattering them from the
+            # pass (61.9 M edges, 4 x 64: 10.3 against 11.0 ms), the same bits
+            grad_x, in_pass_order = _ops.spmm_dot(g.ptr_t, g.idx_t, grad_out, x.shape[0], val, g.perm, x,
+                                                  torch.empty_like(val), dot_at_edge=True)
+            if g.n_edges == val.shape[0]:
+                grad_val = _ops.gather_rows(in_pass_order, _ops.inverse_perm_transposed(g))
+            else:
+                grad_val = torch.zeros_like(val)
+                grad_val[:g.n_edges] = _ops.gather_rows(in_pass_order, _ops.inverse_perm_transposed(g))
             return grad_x, None, None, grad_val, None
         if ctx.needs_input_grad[0]:
             # spmm_multihead_bwd adds into a zeroed tensor; writing the rows of the transposed
