@@ -273,6 +273,15 @@ def c3(iters):
     report("c3", "the same as two passes (Naive, then a sum over the heads)",
            timeit(lambda: _ops._C.head_sum(B.spmm_multihead(ptr, idx, ev, x, N, B.SPMM_MULTIHEAD_SCHEDULE.Naive)), iters),
            E * (4 * H * C + 8 + 4 * H) + 4 * N * C + 8 * (N + 1), 2 * E * H * C)
+    from cxgnncomp.graph_kernel import SpMMValOP
+    xv, evv = x.clone().requires_grad_(True), ev.clone().requires_grad_(True)
+
+    def valop_step():
+        xv.grad = None
+        evv.grad = None
+        SpMMValOP.apply(xv, ptr, idx, evv, N).backward(g)
+    report("c3", "SpMMValOP H=4 C=64 forward + backward (input and edge-value gradients)", timeit(valop_step, max(2, iters // 3)))
+    del xv, evv
     report("c3", "spmm_multihead_bwd H=4 C=64",
            timeit(lambda: _ops.spmm(gt.ptr_t, gt.idx_t, g, N, val=ev, val_perm=gt.perm), iters),
            spmm_bytes(N, E, H * C, H) + 8 * E, 2 * E * H * C)
