@@ -74,7 +74,8 @@ class SeastarRGCNOP(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weights, ptr, idx, rel, num_center):
-        rel = rel.to(torch.int64)
+        if rel.dtype not in (torch.int32, torch.int64):     # integer ids pass as they are: structures built from them are cached per tensor
+            rel = rel.to(torch.int64)
         ctx.save_for_backward(x, weights, ptr, idx, rel)
         return cxgnncomp_backend.seastar_forward(x, ptr, idx, weights, rel)
 
@@ -86,7 +87,17 @@ class SeastarRGCNOP(torch.autograd.Function):
 
 
 class RGCNOP(torch.autograd.Function):
-    """Transform all nodes per relation, then masked aggregation (upstream :205-243)."""
+    """Transform all nodes per relation, then masked aggregation (upstream :205-243): one
+    product over all nodes and one pass over all edges per relation.  CUDA tensors take the
+    same computation in that order as two typed operators -- one typed GEMM over the
+    (source, relation) pairs that occur, one aggregation (``TypedLinearS2DMMAggrOP``) -- instead
+    of 2 R products and 2 R masked passes over the whole edge array."""
+
+    @classmethod
+    def apply(cls, x, weights, ptr, idx, rel, num_center):
+        if x.is_cuda and weights.is_cuda and weights.dim() == 3:
+            return TypedLinearS2DMMAggrOP.apply(x, weights, ptr, idx, rel, num_center)
+        return super().apply(x, weights, ptr, idx, rel, num_center)
 
     @staticmethod
     def forward(ctx, x, weights, ptr, idx, rel, num_center):
@@ -143,7 +154,10 @@ class RGCNOP3(torch.autograd.Function):
         with torch.enable_grad():
             xd = x.detach().requires_grad_(True)
             wd = weights.detach().requires_grad_(True)
-            out = aggr_rgcn_direct_func(xd, ptr, idx, wd, rel.int(), _num(num_center))
+            # (no dtype conversion of integer relation ids: a fresh tensor per call would miss the
+            # cache of structures built from the index arrays)
+            rel_ids = rel if rel.dtype in (torch.int32, torch.int64) else rel.int()
+            out = aggr_rgcn_direct_func(xd, ptr, idx, wd, rel_ids, _num(num_center))
         ctx.inner = (xd, wd, out)
         return out.detach()
 
