@@ -8,7 +8,9 @@ import cxgnncomp_backend
 
 
 def _rel32(rel):
-    return rel if rel.dtype == torch.int32 else rel.to(torch.int32)
+    # integer ids pass as they are: the relational layer caches its pair tables per (ptr, idx, rel)
+    # tensor, and a converted copy per call would rebuild them every time
+    return rel if rel.dtype in (torch.int32, torch.int64) else rel.to(torch.int32)
 
 
 def rgcn_triton(x, ptr, idx, rel, weights, num_nodes):
