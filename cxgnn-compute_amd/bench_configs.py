@@ -523,6 +523,13 @@ def c4(iters):
            timeit(op_step(TypedLinearS2DAggrMMOP.apply), max(2, iters // 3)))
     report("c4", "TypedLinearS2DSort fwd+bwd (relation-segmented edges, one typed GEMM)",
            timeit(op_step(TypedLinearS2DSort), 2))
+    from cxgnncomp import graph_conv as _gc
+    report("c4", "RGCNOP (by its upstream name; CUDA tensors take TypedLinearS2DMMAggrOP) fwd+bwd",
+           timeit(op_step(_gc.RGCNOP.apply), max(2, iters // 3)))
+    report("c4", "RGCNOP3 = aggr_rgcn_direct_func with its gradients, fwd+bwd",
+           timeit(op_step(_gc.RGCNOP3.apply), max(2, iters // 3)))
+    report("c4", "SeastarRGCNOP = seastar_forward + seastar_backward, fwd+bwd",
+           timeit(op_step(_gc.SeastarRGCNOP.apply), max(2, iters // 3)))
     del xr1, wr1
     layer = cxgnncomp.MyRGCNConv(K, K, R).cuda()
     xg = x.clone().requires_grad_(True)
