@@ -505,7 +505,7 @@ class GatLayerOP(torch.autograd.Function):
     more on average, the forward aggregation gathers input rows under the H edge weights
     (``sum_e ev[e, h] x[idx[e]]``, [num_dst, H, in]) and transforms per head afterwards -- the
     order "aggregate, then transform" that upstream's single-head path takes when
-    in < out (cxgnncomp/graph_conv.py:513-527); the transformed features are then formed in the
+    in < out (cxgnncomp/graph_conv.py:523-542); the transformed features are then formed in the
     backward pass only, which needs them for the edge-value gradient."""
 
     @staticmethod

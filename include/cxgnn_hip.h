@@ -141,8 +141,8 @@ int cxg_spmm_prereduce_f32(const int64_t* ptr, const int64_t* idx, const float* 
  * Where a multi-head layer's features are a linear map of a narrower input, xs[:, h, :] = x W_h^T,
  * its aggregation sum_e val[e, h] xs[idx[e], h, :] equals out[r, h, :] W_h^T: the edges gather
  * feat floats instead of heads * channels, the product follows per destination row (the order
- * "aggregate, then transform" of MyGATConv.forward_1, cxgnncomp/graph_conv.py:513-527, applied to
- * forward_many's aggregation, :488-490).  Takes 2, 4 or 8 heads and 20 <= feat <= 128, a
+ * "aggregate, then transform" of MyGATConv.forward_1, cxgnncomp/graph_conv.py:523-542, applied to
+ * forward_many's aggregation, :481-487).  Takes 2, 4 or 8 heads and 20 <= feat <= 128, a
  * multiple of 4; x, out and val 16-byte aligned, strides multiples of 4; otherwise
  * CXG_ERR_UNSUPPORTED.  Workspace: cxg_spmm_workspace_bytes(n_edges_cap, heads * feat).
  * Deterministic (no atomics), like the other aggregations.

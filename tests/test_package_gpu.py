@@ -590,7 +590,7 @@ def test_gat_layer_on_a_row_prefix(concat, heads_channels, max_deg):
                                    (256, 128), (256, 100)])
 @pytest.mark.parametrize("frozen", [False, True])
 def test_gat_single_head_layer_on_a_row_prefix(fin, C, frozen):
-    """MyGATConv with one head (upstream's forward_1, cxgnncomp/graph_conv.py:497-545) on the same
+    """MyGATConv with one head (upstream's forward_1, cxgnncomp/graph_conv.py:498-547) on the same
     layer node: an input narrower than the output is aggregated first and transformed afterwards,
     forward and backward on rows of `in` floats (from 96 columns on the backward pass over the
     reversed graph also leaves the edge-value gradient; 30 columns are not a multiple of 4 and
